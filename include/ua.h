@@ -1,0 +1,132 @@
+/* C ABI of libua_hip.so -- Universal Attention forward/backward on AMD Instinct MI355X (gfx950).
+ *
+ * These entry points are what a binding for the reference's hot path would call in place of its
+ * Triton launchers.  Each declaration cites the reference interface it replaces
+ * (paths relative to the reference repository root).
+ *
+ * Conventions
+ *  - All pointers are DEVICE pointers unless stated; the caller owns every buffer.
+ *  - No entry point allocates or frees device memory; scratch comes from `ws` (size from
+ *    ua_workspace_bytes).  Work is enqueued on `stream` and the call returns without synchronising
+ *    (ua_autotune is the exception: it times candidates and synchronises).
+ *  - Return value: 0 on success, a negative UA_E* code otherwise; ua_last_error() then describes it.
+ *    Nothing throws, nothing aborts.
+ *  - z indices: Zk = b*h (batch x kv head), Zq = b*h*r (r query groups per kv head, kv-major).
+ */
+#ifndef UA_H_
+#define UA_H_
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ihipStream_t* ua_stream_t; /* == hipStream_t */
+
+enum { UA_F32 = 0, UA_BF16 = 1 };
+enum {
+  UA_OK = 0,
+  UA_EINVAL = -1,    /* bad shape / dtype / null pointer / unsupported size */
+  UA_EWORKSPACE = -2,/* workspace too small or misaligned */
+  UA_ELAUNCH = -3    /* HIP reported an error while enqueuing */
+};
+enum {
+  UA_OP_FWD = 0,       /* ua_fwd        */
+  UA_OP_BWD = 1,       /* ua_bwd        */
+  UA_OP_FUSED_FWD = 2, /* ua_fused_fwd  */
+  UA_OP_FUSED_BWD = 3  /* ua_fused_bwd  */
+};
+enum {
+  UA_FLAG_SKIP_MASKED = 1 /* ua_bwd: the upstream gradient is zero for (query, chunk) pairs in which the
+                             query precedes the whole chunk (true when it comes from ua_merge_bwd) */
+};
+
+/* Problem description.  kc, vc: [b,h,L,d] seen as [b,h,n,c,d]; xq: [b,h,r,L,d]; gates: [b,h,L]. */
+typedef struct ua_desc {
+  int32_t b, h, r, L, d;
+  int32_t chunk; /* keys per chunk c (L % c == 0; c == 16 or c % 32 == 0, c <= 256); ignored by fused ops */
+  int32_t dtype; /* UA_F32 or UA_BF16, the dtype of every tensor except where noted */
+  int32_t flags;
+} ua_desc;
+
+/* A row-major tensor whose last (feature) dimension has stride 1; all strides in ELEMENTS.
+ * Row index `row` in [0,L) is addressed as (row / inner_len)*stride_outer + (row % inner_len)*stride_inner,
+ * which covers both [.., L, d] (inner_len = L) and chunked [.., n, c, d] views. */
+typedef struct ua_rows {
+  const void* ptr;
+  int64_t stride_b, stride_h, stride_r, stride_outer, stride_inner;
+  int32_t inner_len;
+} ua_rows;
+
+/* The per-chunk partial output tensor out[b,h,r,L,d,n]: element (zq, t, dd, i) lives at
+ * ptr + zq*stride_z + t*stride_t + dd*stride_d + i*stride_i (elements). */
+typedef struct ua_chunked {
+  void* ptr;
+  int64_t stride_z, stride_t, stride_d, stride_i;
+} ua_chunked;
+
+int ua_version(void);
+/* Thread-local description of the last failure on this thread ("" if none). */
+const char* ua_last_error(void);
+
+/* Bytes of scratch `ws` the given op needs (0 and an error string if the shape is unsupported).
+ * The backward ops can reuse the forward's workspace contents: size it with the backward op and pass
+ * the same buffer to both calls. */
+size_t ua_workspace_bytes(const ua_desc* desc, int op);
+
+/* Chunked forward: replaces _universal_attention_fwd
+ * (Universal_Attention/triton/universal_attention_kernel.py:192-239) and the torch operator
+ * UniversalAttention.forward (universal_attention_autograd.py:9-38).
+ * static_src, static_dest: contiguous [b,h,L].  denom: contiguous [b,h,r,L,n] in desc->dtype. */
+int ua_fwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
+           const void* static_dest, const ua_chunked* out, void* denom, void* ws, size_t ws_bytes, ua_stream_t stream);
+
+/* Chunked backward: replaces _universal_attention_bwd (universal_attention_kernel.py:793-862) and
+ * UniversalAttention.backward (universal_attention_autograd.py:47-99).
+ * out: the forward's result; g_out: same indexing; g_denom: contiguous float32 [b,h,r,L,n].
+ * Gradients are written contiguous: dkc, dvc [b,h,L,d]; dxq [b,h,r,L,d]; dsrc, ddest [b,h,L].
+ * ws_has_fwd != 0: `ws` still holds what ua_fwd left there for the same inputs (skips the recompute). */
+int ua_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
+           const void* static_dest, const ua_chunked* out, const ua_chunked* g_out, const float* g_denom, void* dkc,
+           void* dvc, void* dxq, void* dsrc, void* ddest, void* ws, size_t ws_bytes, int ws_has_fwd, ua_stream_t stream);
+
+/* Fused forward: the chunked operator followed by SMVecMatMul (universal_attention_autograd.py:278-283)
+ * without materialising the per-chunk tensor; same role as the reference's second-generation
+ * _attention.forward (Universal_Attention/triton/universal_attention_kernel_opt.py:436-502).
+ * O: contiguous [b,h,r,L,d]; lse: contiguous float32 [b,h,r,L] (natural log). */
+int ua_fused_fwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
+                 const void* static_dest, void* O, float* lse, void* ws, size_t ws_bytes, ua_stream_t stream);
+
+/* Fused backward: replaces SMVecMatMul.backward + UniversalAttention.backward
+ * (universal_attention_autograd.py:291-297, :47-99) / _attention.backward (universal_attention_kernel_opt.py:504-581).
+ * O, lse: as produced by ua_fused_fwd; dO contiguous [b,h,r,L,d]. */
+int ua_fused_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
+                 const void* static_dest, const void* O, const float* lse, const void* dO, void* dkc, void* dvc,
+                 void* dxq, void* dsrc, void* ddest, void* ws, size_t ws_bytes, int ws_has_fwd, ua_stream_t stream);
+
+/* Chunk merge: replaces SMVecMatMul.forward / .backward (universal_attention_autograd.py:278-297).
+ * rows = number of (b,h,r,t) rows, n chunks, d features.  mat element (row, dd, i) at
+ * row_off(row) + dd*stride_d + i*stride_i with row_off = (row / L)*stride_z + (row % L)*stride_t.
+ * vec: contiguous [rows, n] in `dtype`; result contiguous [rows, d]. */
+int ua_merge_fwd(int dtype, int64_t rows, int32_t L, int32_t d, int32_t n, const ua_chunked* mat, const void* vec,
+                 void* result, ua_stream_t stream);
+/* g: contiguous [rows, d]; d_mat indexed like mat; d_vec contiguous [rows, n] in `dtype`. */
+int ua_merge_bwd(int dtype, int64_t rows, int32_t L, int32_t d, int32_t n, const ua_chunked* mat, const void* vec,
+                 const void* g, const ua_chunked* d_mat, void* d_vec, ua_stream_t stream);
+
+/* On-device autotune table: replaces the @triton.autotune wrappers
+ * (universal_attention_kernel.py:10-25, universal_attention_kernel_opt.py:8-36).  Times the kernel variants
+ * available for (op, desc) on `stream` using `ws` and records the fastest in the process-wide table that
+ * the ops consult.  Synchronises.  Returns the chosen variant id (>= 0) or a negative error. */
+int ua_autotune(const ua_desc* desc, int op, void* ws, size_t ws_bytes, ua_stream_t stream);
+/* Table access for persistence: get / force the variant of (op, desc). -1 = no entry / built-in default. */
+int ua_tune_get(const ua_desc* desc, int op);
+int ua_tune_set(const ua_desc* desc, int op, int variant);
+/* Number of variants an op has for this description (>= 1), or a negative error. */
+int ua_tune_variants(const ua_desc* desc, int op);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* UA_H_ */

@@ -1,0 +1,79 @@
+"""ctypes binding of libua_hip.so (the C ABI declared in include/ua.h).
+
+The library is the product path: there is no CPU or PyTorch fallback.  Loading fails
+loudly when the shared object is missing, and every op raises if the C call reports an error.
+"""
+import ctypes
+import os
+import threading
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libua_hip.so")
+
+UA_F32, UA_BF16 = 0, 1
+UA_OP_FWD, UA_OP_BWD, UA_OP_FUSED_FWD, UA_OP_FUSED_BWD = 0, 1, 2, 3
+UA_FLAG_SKIP_MASKED = 1
+
+c_void_p, c_int, c_size_t, c_int64, c_int32 = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_int64, ctypes.c_int32
+
+
+class UaDesc(ctypes.Structure):
+    _fields_ = [(n, c_int32) for n in ("b", "h", "r", "L", "d", "chunk", "dtype", "flags")]
+
+
+class UaRows(ctypes.Structure):
+    _fields_ = [("ptr", c_void_p)] + [(n, c_int64) for n in ("stride_b", "stride_h", "stride_r", "stride_outer", "stride_inner")] + [("inner_len", c_int32)]
+
+
+class UaChunked(ctypes.Structure):
+    _fields_ = [("ptr", c_void_p)] + [(n, c_int64) for n in ("stride_z", "stride_t", "stride_d", "stride_i")]
+
+
+P = ctypes.POINTER
+# name -> (restype, argtypes); every symbol include/ua.h declares
+SIGNATURES = {
+    "ua_version": (c_int, []),
+    "ua_last_error": (ctypes.c_char_p, []),
+    "ua_workspace_bytes": (c_size_t, [P(UaDesc), c_int]),
+    "ua_fwd": (c_int, [P(UaDesc), P(UaRows), P(UaRows), P(UaRows), c_void_p, c_void_p, P(UaChunked), c_void_p, c_void_p, c_size_t, c_void_p]),
+    "ua_bwd": (c_int, [P(UaDesc), P(UaRows), P(UaRows), P(UaRows), c_void_p, c_void_p, P(UaChunked), P(UaChunked), c_void_p,
+                       c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
+    "ua_fused_fwd": (c_int, [P(UaDesc), P(UaRows), P(UaRows), P(UaRows), c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "ua_fused_bwd": (c_int, [P(UaDesc), P(UaRows), P(UaRows), P(UaRows), c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
+    "ua_merge_fwd": (c_int, [c_int, c_int64, c_int32, c_int32, c_int32, P(UaChunked), c_void_p, c_void_p, c_void_p]),
+    "ua_merge_bwd": (c_int, [c_int, c_int64, c_int32, c_int32, c_int32, P(UaChunked), c_void_p, c_void_p, P(UaChunked), c_void_p, c_void_p]),
+    "ua_autotune": (c_int, [P(UaDesc), c_int, c_void_p, c_size_t, c_void_p]),
+    "ua_tune_get": (c_int, [P(UaDesc), c_int]),
+    "ua_tune_set": (c_int, [P(UaDesc), c_int, c_int]),
+    "ua_tune_variants": (c_int, [P(UaDesc), c_int]),
+}
+
+_lib = None
+_lock = threading.Lock()
+
+
+class UaError(RuntimeError):
+    pass
+
+
+def load():
+    """Returns the loaded library; raises if it has not been built (python -m universal_attention_triton_amd.build)."""
+    global _lib
+    with _lock:
+        if _lib is None:
+            if not os.path.exists(LIB_PATH):
+                raise UaError("%s is missing: build it with `python -m universal_attention_triton_amd.build` "
+                              "(there is no fallback path)" % LIB_PATH)
+            lib = ctypes.CDLL(LIB_PATH)
+            for name, (res, args) in SIGNATURES.items():
+                fn = getattr(lib, name)
+                fn.restype, fn.argtypes = res, args
+            _lib = lib
+    return _lib
+
+
+def check(code, what):
+    if code < 0:
+        raise UaError("%s failed (%d): %s" % (what, code, load().ua_last_error().decode()))
+    return code

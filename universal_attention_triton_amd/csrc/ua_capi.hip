@@ -1,0 +1,405 @@
+// C ABI of libua_hip.so: validation, workspace layout, kernel sequencing, autotune table.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <tuple>
+
+#include "../../include/ua.h"
+#include "ua_internal.hpp"
+#include "ua_merge.hpp"
+#include "ua_pack.hpp"
+#include "ua_bwd.hpp"   // k_bwd_finish only (k_bwd_keys is instantiated in ua_inst_bwd.hip)
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+struct Layout {
+  int D, Lp, nT, nch, Zk, Zq;
+  size_t esz;
+  // forward state
+  size_t Kp, KT, Ks, KsT, Kd, KdT, Vp, VT, Qp, QT, C, lse2, fwd_end;
+  // backward scratch
+  size_t dOp, dOT, delta, dQacc, dKdacc, dKrow, dVrow, dsrc_raw, total;
+};
+
+int check_desc(const ua_desc* d, bool chunked) {
+  if (!d) return fail(UA_EINVAL, "null descriptor");
+  if (d->dtype != UA_F32 && d->dtype != UA_BF16) return fail(UA_EINVAL, "dtype %d: only UA_F32 and UA_BF16 are supported", d->dtype);
+  if (d->b < 1 || d->h < 1 || d->r < 1 || d->L < 1 || d->d < 1) return fail(UA_EINVAL, "b,h,r,L,d must be positive (got %d,%d,%d,%d,%d)", d->b, d->h, d->r, d->L, d->d);
+  if (d->d > 128) return fail(UA_EINVAL, "head dim %d > 128 is not supported", d->d);
+  if ((long)d->b * d->h * d->r > 65535) return fail(UA_EINVAL, "b*h*r = %ld exceeds the grid limit 65535", (long)d->b * d->h * d->r);
+  if (chunked) {
+    const int c = d->chunk;
+    if (c < 1 || d->L % c != 0) return fail(UA_EINVAL, "chunk %d must divide L = %d", c, d->L);
+    if (!(c == 16 || c % 32 == 0) || c > 256) return fail(UA_EINVAL, "chunk %d unsupported: need 16 or a multiple of 32, at most 256", c);
+    if (d->L / c > ua::kMergeMaxN * 64) return fail(UA_EINVAL, "too many chunks");
+  }
+  return UA_OK;
+}
+
+Layout make_layout(const ua_desc& d, bool chunked) {
+  Layout l{};
+  l.D = d.d <= 64 ? 64 : 128;
+  l.Lp = (int)align_up((size_t)d.L, 128);
+  l.nT = l.Lp / 32;
+  l.nch = chunked ? d.L / d.chunk : 1;
+  l.Zk = d.b * d.h;
+  l.Zq = l.Zk * d.r;
+  l.esz = d.dtype == UA_BF16 ? 2 : 4;
+  size_t off = 0;
+  auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
+  const size_t kbytes = (size_t)l.Zk * l.Lp * l.D * l.esz, qbytes = (size_t)l.Zq * l.Lp * l.D * l.esz;
+  l.Kp = take(kbytes); l.KT = take(kbytes); l.Ks = take(kbytes); l.KsT = take(kbytes);
+  l.Kd = take(kbytes); l.KdT = take(kbytes); l.Vp = take(kbytes); l.VT = take(kbytes);
+  l.Qp = take(qbytes); l.QT = take(qbytes);
+  l.C = take((size_t)l.Zk * l.nT * l.Lp * 4);
+  l.lse2 = take((size_t)l.Zq * l.nch * l.Lp * 4);
+  l.fwd_end = off;
+  const size_t gbytes = (size_t)l.Zq * l.nch * l.Lp * l.D * l.esz;
+  l.dOp = take(gbytes); l.dOT = take(gbytes);
+  l.delta = take((size_t)l.Zq * l.nch * l.Lp * 4);
+  l.dQacc = take((size_t)l.Zq * l.Lp * l.D * 4);
+  l.dKdacc = take((size_t)l.Zk * l.Lp * l.D * 4);
+  l.dKrow = take((size_t)l.Zk * l.Lp * l.D * 4);
+  l.dVrow = take((size_t)l.Zk * l.Lp * l.D * 4);
+  l.dsrc_raw = take((size_t)l.Zk * l.Lp * 4);
+  l.total = off;
+  return l;
+}
+
+ua::RowsView rows_view(const ua_rows& r, int H, int R) {
+  ua::RowsView v;
+  v.p = r.ptr; v.sb = r.stride_b; v.sh = r.stride_h; v.sr = r.stride_r; v.sn = 0;
+  v.so = r.stride_outer; v.si = r.stride_inner; v.sc = 1; v.inner = r.inner_len > 0 ? r.inner_len : 1;
+  v.H = H; v.R = R; v.N = 1;
+  return v;
+}
+// contiguous [Z][L] (gates, lse) or [Z][L][d]
+ua::RowsView contiguous_view(const void* p, long z_stride, long row_stride) {
+  ua::RowsView v;
+  v.p = p; v.sb = z_stride; v.sh = 0; v.sr = 0; v.sn = 0; v.so = 0; v.si = row_stride; v.sc = 1;
+  v.inner = 1 << 30; v.H = 1; v.R = 1; v.N = 1;
+  return v;
+}
+// chunked tensor (zq, t, dd, i) seen as rows of z = zq*nch + i
+ua::RowsView chunked_view(const ua_chunked& c, int nch) {
+  ua::RowsView v;
+  v.p = c.ptr; v.sb = c.stride_z; v.sh = 0; v.sr = 0; v.sn = c.stride_i; v.so = 0; v.si = c.stride_t; v.sc = c.stride_d;
+  v.inner = 1 << 30; v.H = 1; v.R = 1; v.N = nch;
+  return v;
+}
+ua::RowsView null_view() { ua::RowsView v{}; v.inner = 1; v.H = v.R = v.N = 1; return v; }
+
+template <class T>
+hipError_t pack_t(int D, const ua::RowsView& x, const ua::RowsView& gate, int gate_div, void* nat, void* tr, int d, int L,
+                  int Lp, int Z, hipStream_t s) {
+  if (D == 64) hipLaunchKernelGGL((ua::k_pack<T, 64>), dim3(Lp / 32, Z), dim3(256), 0, s, x, gate, gate_div, (T*)nat, (T*)tr, d, L, Lp);
+  else hipLaunchKernelGGL((ua::k_pack<T, 128>), dim3(Lp / 32, Z), dim3(256), 0, s, x, gate, gate_div, (T*)nat, (T*)tr, d, L, Lp);
+  return hipGetLastError();
+}
+hipError_t pack(int dtype, int D, const ua::RowsView& x, const ua::RowsView& gate, int gate_div, void* nat, void* tr, int d,
+                int L, int Lp, int Z, hipStream_t s) {
+  return dtype == UA_BF16 ? pack_t<ua::bf16>(D, x, gate, gate_div, nat, tr, d, L, Lp, Z, s)
+                          : pack_t<float>(D, x, gate, gate_div, nat, tr, d, L, Lp, Z, s);
+}
+
+#define UA_HIP(expr)                                                                         \
+  do {                                                                                       \
+    hipError_t e_ = (expr);                                                                  \
+    if (e_ != hipSuccess) return fail(UA_ELAUNCH, "%s: %s", #expr, hipGetErrorString(e_));   \
+  } while (0)
+
+int check_common(const ua_desc* desc, bool chunked, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq,
+                 const void* src, const void* dest, void* ws, size_t ws_bytes, const Layout& l, bool bwd) {
+  (void)desc; (void)chunked;
+  if (!kc || !vc || !xq || !kc->ptr || !vc->ptr || !xq->ptr || !src || !dest) return fail(UA_EINVAL, "null input tensor");
+  if (!ws) return fail(UA_EWORKSPACE, "null workspace");
+  if ((uintptr_t)ws % 256 != 0) return fail(UA_EWORKSPACE, "workspace must be 256-byte aligned");
+  const size_t need = bwd ? l.total : l.fwd_end;
+  if (ws_bytes < need) return fail(UA_EWORKSPACE, "workspace has %zu bytes, %zu needed", ws_bytes, need);
+  return UA_OK;
+}
+
+hipError_t zero_fill(void* p, size_t bytes, hipStream_t s) {   // bytes is a multiple of 16
+  const size_t n16 = bytes / 16;
+  const unsigned grid = (unsigned)((n16 + 255) / 256 < 4096 ? (n16 + 255) / 256 : 4096);
+  hipLaunchKernelGGL(ua::k_zero, dim3(grid), dim3(256), 0, s, (float4*)p, n16);
+  return hipGetLastError();
+}
+
+// packs K (plain, src-scaled, dest-scaled), V and Q in both orientations
+int pack_inputs(const ua_desc& d, const Layout& l, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* src,
+                const void* dest, char* ws, hipStream_t s) {
+  const ua::RowsView K = rows_view(*kc, d.h, 1), V = rows_view(*vc, d.h, 1), Q = rows_view(*xq, d.h, d.r);
+  const ua::RowsView gs = contiguous_view(src, d.L, 1), gd = contiguous_view(dest, d.L, 1), none = null_view();
+  UA_HIP(pack(d.dtype, l.D, K, none, 1, ws + l.Kp, ws + l.KT, d.d, d.L, l.Lp, l.Zk, s));
+  UA_HIP(pack(d.dtype, l.D, K, gs, 1, ws + l.Ks, ws + l.KsT, d.d, d.L, l.Lp, l.Zk, s));
+  UA_HIP(pack(d.dtype, l.D, K, gd, 1, ws + l.Kd, ws + l.KdT, d.d, d.L, l.Lp, l.Zk, s));
+  UA_HIP(pack(d.dtype, l.D, V, none, 1, ws + l.Vp, ws + l.VT, d.d, d.L, l.Lp, l.Zk, s));
+  UA_HIP(pack(d.dtype, l.D, Q, none, 1, ws + l.Qp, ws + l.QT, d.d, d.L, l.Lp, l.Zq, s));
+  return UA_OK;
+}
+
+// ---- autotune table ------------------------------------------------------------------------
+using TuneKey = std::tuple<int, int, int, int, int, int>;  // op, dtype, D, r, chunk, L bucket
+std::mutex g_tune_mu;
+std::map<TuneKey, int> g_tune;
+
+int l_bucket(int L) { int b = 0; while ((128 << b) < L) ++b; return b; }
+TuneKey tune_key(const ua_desc& d, int op) {
+  const bool chunked = (op == UA_OP_FWD || op == UA_OP_BWD);
+  return TuneKey(op, d.dtype, d.d <= 64 ? 64 : 128, d.r, chunked ? d.chunk : 0, l_bucket(d.L));
+}
+int n_variants(const ua_desc& d, int op) {
+  if (op == UA_OP_FUSED_FWD) return ua::fwd_fused_variants(d.dtype, d.d <= 64 ? 64 : 128);
+  return 1;
+}
+int tuned_variant(const ua_desc& d, int op) {
+  std::lock_guard<std::mutex> g(g_tune_mu);
+  auto it = g_tune.find(tune_key(d, op));
+  return it == g_tune.end() ? 0 : it->second;
+}
+
+int run_fused_fwd_kernels(const ua_desc& d, const Layout& l, char* ws, void* O, float* lse, int variant, hipStream_t s) {
+  UA_HIP(ua::launch_carry(d.dtype, l.D, ws + l.Ks, ws + l.Kd, (float*)(ws + l.C), l.Lp, l.Zk, s));
+  UA_HIP(ua::launch_fwd_fused(d.dtype, l.D, variant, ws + l.Qp, ws + l.Kd, ws + l.Ks, ws + l.Kp, ws + l.VT,
+                              (const float*)(ws + l.C), O, lse, (float*)(ws + l.lse2), d.r, d.L, l.Lp, d.d, l.Zq, s));
+  return UA_OK;
+}
+
+template <class T>
+hipError_t finish_t(const Layout& l, const ua_desc& d, char* ws, const void* src, const void* dest, void* dk, void* dv,
+                    void* dq, void* dsrc, void* ddest, hipStream_t s) {
+  const int Z = l.Zq > l.Zk ? l.Zq : l.Zk;
+  hipLaunchKernelGGL((ua::k_bwd_finish<T>), dim3((d.L + 3) / 4, Z), dim3(256), 0, s, (const float*)(ws + l.dKrow),
+                     (const float*)(ws + l.dVrow), (const float*)(ws + l.dKdacc), (const float*)(ws + l.dQacc),
+                     (const float*)(ws + l.dsrc_raw), (const T*)(ws + l.Kp), (const T*)src, (const T*)dest, (T*)dk, (T*)dv,
+                     (T*)dq, (T*)dsrc, (T*)ddest, l.Zk, l.Zq, d.L, l.Lp, l.D, d.d);
+  return hipGetLastError();
+}
+
+template <class T>
+hipError_t delta_t(const ua::RowsView& O, const ua::RowsView& dO, const ua::RowsView& sub, const ua::RowsView& lse_in,
+                   float* delta, float* lse2, int d, int L, int Lp, int Z, hipStream_t s) {
+  hipLaunchKernelGGL((ua::k_delta<T>), dim3(Lp / 4, Z), dim3(256), 0, s, O, dO, sub, lse_in, delta, lse2, d, L, Lp);
+  return hipGetLastError();
+}
+
+int run_bwd_common(const ua_desc& d, const Layout& l, char* ws, bool chunked, const void* src, const void* dest, void* dkc,
+                   void* dvc, void* dxq, void* dsrc, void* ddest, hipStream_t s) {
+  UA_HIP(zero_fill(ws + l.dQacc, (size_t)l.Zq * l.Lp * l.D * 4, s));
+  UA_HIP(zero_fill(ws + l.dKdacc, (size_t)l.Zk * l.Lp * l.D * 4, s));
+  ua::BwdArgsV a{};
+  a.Ks = ws + l.Ks; a.Kp = ws + l.Kp; a.Vp = ws + l.Vp; a.Kd = ws + l.Kd; a.KdT = ws + l.KdT; a.KT = ws + l.KT;
+  a.KsT = ws + l.KsT; a.Qp = ws + l.Qp; a.QT = ws + l.QT; a.dOp = ws + l.dOp; a.dOT = ws + l.dOT;
+  a.lse2 = (const float*)(ws + l.lse2); a.delta = (const float*)(ws + l.delta); a.C = (const float*)(ws + l.C);
+  a.src = src;
+  a.dQacc = (float*)(ws + l.dQacc); a.dKdacc = (float*)(ws + l.dKdacc); a.dKrow = (float*)(ws + l.dKrow);
+  a.dVrow = (float*)(ws + l.dVrow); a.dsrc_raw = (float*)(ws + l.dsrc_raw);
+  a.R = d.r; a.L = d.L; a.Lp = l.Lp; a.c = chunked ? d.chunk : 128; a.nch = l.nch; a.chunked = chunked ? 1 : 0;
+  a.skip_masked = (d.flags & UA_FLAG_SKIP_MASKED) ? 1 : 0;
+  UA_HIP(ua::launch_bwd_keys(d.dtype, l.D, a, l.Zk, s));
+  if (d.dtype == UA_BF16) UA_HIP(finish_t<ua::bf16>(l, d, ws, src, dest, dkc, dvc, dxq, dsrc, ddest, s));
+  else UA_HIP(finish_t<float>(l, d, ws, src, dest, dkc, dvc, dxq, dsrc, ddest, s));
+  return UA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ua_version(void) { return 1; }
+const char* ua_last_error(void) { return g_err; }
+
+size_t ua_workspace_bytes(const ua_desc* desc, int op) {
+  const bool chunked = (op == UA_OP_FWD || op == UA_OP_BWD);
+  if (op < UA_OP_FWD || op > UA_OP_FUSED_BWD) { fail(UA_EINVAL, "unknown op %d", op); return 0; }
+  if (check_desc(desc, chunked) != UA_OK) return 0;
+  const Layout l = make_layout(*desc, chunked);
+  return (op == UA_OP_FWD || op == UA_OP_FUSED_FWD) ? l.fwd_end : l.total;
+}
+
+int ua_fused_fwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
+                 const void* static_dest, void* O, float* lse, void* ws, size_t ws_bytes, ua_stream_t stream) {
+  if (int e = check_desc(desc, false)) return e;
+  const Layout l = make_layout(*desc, false);
+  if (int e = check_common(desc, false, kc, vc, xq, static_src, static_dest, ws, ws_bytes, l, false)) return e;
+  if (!O || !lse) return fail(UA_EINVAL, "null output tensor");
+  char* w = (char*)ws;
+  hipStream_t s = (hipStream_t)stream;
+  if (int e = pack_inputs(*desc, l, kc, vc, xq, static_src, static_dest, w, s)) return e;
+  return run_fused_fwd_kernels(*desc, l, w, O, lse, tuned_variant(*desc, UA_OP_FUSED_FWD), s);
+}
+
+int ua_fused_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
+                 const void* static_dest, const void* O, const float* lse, const void* dO, void* dkc, void* dvc, void* dxq,
+                 void* dsrc, void* ddest, void* ws, size_t ws_bytes, int ws_has_fwd, ua_stream_t stream) {
+  if (int e = check_desc(desc, false)) return e;
+  const Layout l = make_layout(*desc, false);
+  if (int e = check_common(desc, false, kc, vc, xq, static_src, static_dest, ws, ws_bytes, l, true)) return e;
+  if (!O || !lse || !dO || !dkc || !dvc || !dxq || !dsrc || !ddest) return fail(UA_EINVAL, "null tensor");
+  char* w = (char*)ws;
+  hipStream_t s = (hipStream_t)stream;
+  const ua_desc& d = *desc;
+  if (!ws_has_fwd) {
+    if (int e = pack_inputs(d, l, kc, vc, xq, static_src, static_dest, w, s)) return e;
+    UA_HIP(ua::launch_carry(d.dtype, l.D, w + l.Ks, w + l.Kd, (float*)(w + l.C), l.Lp, l.Zk, s));
+  }
+  const long rowsz = (long)d.L * d.d;
+  const ua::RowsView Ov = contiguous_view(O, rowsz, d.d), dOv = contiguous_view(dO, rowsz, d.d);
+  const ua::RowsView lsev = contiguous_view(lse, d.L, 1), none = null_view();
+  UA_HIP(pack(d.dtype, l.D, dOv, none, 1, w + l.dOp, w + l.dOT, d.d, d.L, l.Lp, l.Zq, s));
+  if (d.dtype == UA_BF16) UA_HIP(delta_t<ua::bf16>(Ov, dOv, none, lsev, (float*)(w + l.delta), (float*)(w + l.lse2), d.d, d.L, l.Lp, l.Zq, s));
+  else UA_HIP(delta_t<float>(Ov, dOv, none, lsev, (float*)(w + l.delta), (float*)(w + l.lse2), d.d, d.L, l.Lp, l.Zq, s));
+  return run_bwd_common(d, l, w, false, static_src, static_dest, dkc, dvc, dxq, dsrc, ddest, s);
+}
+
+int ua_fwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
+           const void* static_dest, const ua_chunked* out, void* denom, void* ws, size_t ws_bytes, ua_stream_t stream) {
+  if (int e = check_desc(desc, true)) return e;
+  const Layout l = make_layout(*desc, true);
+  if (int e = check_common(desc, true, kc, vc, xq, static_src, static_dest, ws, ws_bytes, l, false)) return e;
+  if (!out || !out->ptr || !denom) return fail(UA_EINVAL, "null output tensor");
+  char* w = (char*)ws;
+  hipStream_t s = (hipStream_t)stream;
+  const ua_desc& d = *desc;
+  if (int e = pack_inputs(d, l, kc, vc, xq, static_src, static_dest, w, s)) return e;
+  UA_HIP(ua::launch_fwd_chunked(d.dtype, l.D, w + l.Qp, w + l.Kd, w + l.Ks, w + l.Kp, w + l.VT, out->ptr, denom,
+                                (float*)(w + l.lse2), out->stride_z, out->stride_t, out->stride_d, out->stride_i, d.r, d.L,
+                                l.Lp, d.d, d.chunk, l.nch, l.Zk, s));
+  return UA_OK;
+}
+
+int ua_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
+           const void* static_dest, const ua_chunked* out, const ua_chunked* g_out, const float* g_denom, void* dkc,
+           void* dvc, void* dxq, void* dsrc, void* ddest, void* ws, size_t ws_bytes, int ws_has_fwd, ua_stream_t stream) {
+  if (int e = check_desc(desc, true)) return e;
+  const Layout l = make_layout(*desc, true);
+  if (int e = check_common(desc, true, kc, vc, xq, static_src, static_dest, ws, ws_bytes, l, true)) return e;
+  if (!out || !out->ptr || !g_out || !g_out->ptr || !g_denom || !dkc || !dvc || !dxq || !dsrc || !ddest)
+    return fail(UA_EINVAL, "null tensor");
+  char* w = (char*)ws;
+  hipStream_t s = (hipStream_t)stream;
+  const ua_desc& d = *desc;
+  if (!ws_has_fwd) {
+    // recompute the per-chunk normalisers (the partial outputs themselves are passed in)
+    if (int e = pack_inputs(d, l, kc, vc, xq, static_src, static_dest, w, s)) return e;
+    UA_HIP(ua::launch_fwd_chunked(d.dtype, l.D, w + l.Qp, w + l.Kd, w + l.Ks, w + l.Kp, w + l.VT, nullptr, nullptr,
+                                  (float*)(w + l.lse2), 0, 0, 0, 0, d.r, d.L, l.Lp, d.d, d.chunk, l.nch, l.Zk, s));
+  }
+  UA_HIP(ua::launch_carry(d.dtype, l.D, w + l.Ks, w + l.Kd, (float*)(w + l.C), l.Lp, l.Zk, s));
+  const ua::RowsView outv = chunked_view(*out, l.nch);
+  ua_chunked gmut = *g_out;
+  const ua::RowsView gv = chunked_view(gmut, l.nch), none = null_view();
+  // g_denom [zq][t][i] seen per z = zq*nch + i
+  ua::RowsView gdv;
+  gdv.p = g_denom; gdv.sb = (long)d.L * l.nch; gdv.sh = 0; gdv.sr = 0; gdv.sn = 1; gdv.so = 0; gdv.si = l.nch; gdv.sc = 1;
+  gdv.inner = 1 << 30; gdv.H = 1; gdv.R = 1; gdv.N = l.nch;
+  UA_HIP(pack(d.dtype, l.D, gv, none, 1, w + l.dOp, w + l.dOT, d.d, d.L, l.Lp, l.Zq * l.nch, s));
+  if (d.dtype == UA_BF16) UA_HIP(delta_t<ua::bf16>(outv, gv, gdv, none, (float*)(w + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s));
+  else UA_HIP(delta_t<float>(outv, gv, gdv, none, (float*)(w + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s));
+  return run_bwd_common(d, l, w, true, static_src, static_dest, dkc, dvc, dxq, dsrc, ddest, s);
+}
+
+int ua_merge_fwd(int dtype, int64_t rows, int32_t L, int32_t d, int32_t n, const ua_chunked* mat, const void* vec,
+                 void* result, ua_stream_t stream) {
+  if (!mat || !mat->ptr || !vec || !result) return fail(UA_EINVAL, "null tensor");
+  if (rows < 1 || L < 1 || d < 1 || n < 1 || n > ua::kMergeMaxN) return fail(UA_EINVAL, "bad merge shape rows=%ld L=%d d=%d n=%d", (long)rows, L, d, n);
+  if (dtype != UA_F32 && dtype != UA_BF16) return fail(UA_EINVAL, "dtype %d unsupported", dtype);
+  ua::ChunkedView m{mat->ptr, mat->stride_z, mat->stride_t, mat->stride_d, mat->stride_i};
+  const dim3 grid((unsigned)((rows + 3) / 4));
+  const size_t lds = 4 * (size_t)n * sizeof(float);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == UA_BF16) hipLaunchKernelGGL((ua::k_merge_fwd<ua::bf16>), grid, dim3(256), lds, s, m, (const ua::bf16*)vec, (ua::bf16*)result, (long)rows, L, d, n);
+  else hipLaunchKernelGGL((ua::k_merge_fwd<float>), grid, dim3(256), lds, s, m, (const float*)vec, (float*)result, (long)rows, L, d, n);
+  UA_HIP(hipGetLastError());
+  return UA_OK;
+}
+
+int ua_merge_bwd(int dtype, int64_t rows, int32_t L, int32_t d, int32_t n, const ua_chunked* mat, const void* vec,
+                 const void* g, const ua_chunked* d_mat, void* d_vec, ua_stream_t stream) {
+  if (!mat || !mat->ptr || !vec || !g || !d_mat || !d_mat->ptr || !d_vec) return fail(UA_EINVAL, "null tensor");
+  if (rows < 1 || L < 1 || d < 1 || n < 1 || n > ua::kMergeMaxN) return fail(UA_EINVAL, "bad merge shape rows=%ld L=%d d=%d n=%d", (long)rows, L, d, n);
+  if (dtype != UA_F32 && dtype != UA_BF16) return fail(UA_EINVAL, "dtype %d unsupported", dtype);
+  ua::ChunkedView m{mat->ptr, mat->stride_z, mat->stride_t, mat->stride_d, mat->stride_i};
+  ua::ChunkedView dm{d_mat->ptr, d_mat->stride_z, d_mat->stride_t, d_mat->stride_d, d_mat->stride_i};
+  const dim3 grid((unsigned)((rows + 3) / 4));
+  const size_t lds = 8 * (size_t)n * sizeof(float);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == UA_BF16) hipLaunchKernelGGL((ua::k_merge_bwd<ua::bf16>), grid, dim3(256), lds, s, m, (const ua::bf16*)vec, (const ua::bf16*)g, dm, (ua::bf16*)d_vec, (long)rows, L, d, n);
+  else hipLaunchKernelGGL((ua::k_merge_bwd<float>), grid, dim3(256), lds, s, m, (const float*)vec, (const float*)g, dm, (float*)d_vec, (long)rows, L, d, n);
+  UA_HIP(hipGetLastError());
+  return UA_OK;
+}
+
+int ua_tune_variants(const ua_desc* desc, int op) {
+  if (op < UA_OP_FWD || op > UA_OP_FUSED_BWD) return fail(UA_EINVAL, "unknown op %d", op);
+  if (int e = check_desc(desc, op == UA_OP_FWD || op == UA_OP_BWD)) return e;
+  return n_variants(*desc, op);
+}
+int ua_tune_get(const ua_desc* desc, int op) {
+  if (!desc) return -1;
+  std::lock_guard<std::mutex> g(g_tune_mu);
+  auto it = g_tune.find(tune_key(*desc, op));
+  return it == g_tune.end() ? -1 : it->second;
+}
+int ua_tune_set(const ua_desc* desc, int op, int variant) {
+  const int n = ua_tune_variants(desc, op);
+  if (n < 0) return n;
+  if (variant < 0 || variant >= n) return fail(UA_EINVAL, "variant %d out of range [0,%d)", variant, n);
+  std::lock_guard<std::mutex> g(g_tune_mu);
+  g_tune[tune_key(*desc, op)] = variant;
+  return UA_OK;
+}
+
+int ua_autotune(const ua_desc* desc, int op, void* ws, size_t ws_bytes, ua_stream_t stream) {
+  const int n = ua_tune_variants(desc, op);
+  if (n < 0) return n;
+  if (n == 1) { ua_tune_set(desc, op, 0); return 0; }
+  // only the fused forward has more than one variant: time the main kernel on whatever the workspace holds
+  const Layout l = make_layout(*desc, false);
+  if (!ws || ws_bytes < l.total) return fail(UA_EWORKSPACE, "autotune needs the backward-sized workspace (%zu bytes)", l.total);
+  char* w = (char*)ws;
+  hipStream_t s = (hipStream_t)stream;
+  // deterministic, finite operands: zero the packed inputs; throw-away outputs go to backward scratch
+  UA_HIP(zero_fill(w, l.fwd_end, s));
+  void* Otmp = w + l.dOp;
+  float* lsetmp = (float*)(w + l.delta);
+  hipEvent_t e0, e1;
+  UA_HIP(hipEventCreate(&e0)); UA_HIP(hipEventCreate(&e1));
+  int best = 0; float best_ms = 1e30f;
+  for (int v = 0; v < n; ++v) {
+    for (int rep = 0; rep < 2; ++rep) {   // first pass warms up
+      UA_HIP(hipEventRecord(e0, s));
+      hipError_t e = ua::launch_fwd_fused(desc->dtype, l.D, v, w + l.Qp, w + l.Kd, w + l.Ks, w + l.Kp, w + l.VT,
+                                          (const float*)(w + l.C), Otmp, lsetmp, (float*)(w + l.lse2), desc->r, desc->L,
+                                          l.Lp, desc->d, l.Zq, s);
+      if (e != hipSuccess) return fail(UA_ELAUNCH, "autotune launch: %s", hipGetErrorString(e));
+      UA_HIP(hipEventRecord(e1, s));
+      UA_HIP(hipEventSynchronize(e1));
+      float ms = 0.f;
+      UA_HIP(hipEventElapsedTime(&ms, e0, e1));
+      if (rep == 1 && ms < best_ms) { best_ms = ms; best = v; }
+    }
+  }
+  hipEventDestroy(e0); hipEventDestroy(e1);
+  ua_tune_set(desc, op, best);
+  return best;
+}
+
+}  // extern "C"

@@ -1,0 +1,173 @@
+// Shared device helpers for the Universal Attention kernels (gfx950 / CDNA4, wave64).
+//
+// Tile convention used by every kernel in this library
+// ----------------------------------------------------
+// All pairwise quantities (key s, query t) are produced by v_mfma_f32_32x32x* as
+// 32x32 blocks in the orientation  D[t, s] = X_t . Y_s^T :
+//     A operand = 32 rows of X (query side),   lane (l%32) <-> row t, 8 k-values per lane
+//     B operand = 32 rows of Y (key side),     lane (l%32) <-> col s, 8 k-values per lane
+//     result    = f32x16 per lane: lane <-> key s = l%32, register v <-> query
+//                 t = 8*(v/4) + 4*(l/32) + (v%4)
+// so one lane owns ONE key and 16 of the 32 queries of the block.  The decay bias is
+// a cumulative sum over queries for a fixed key, i.e. an in-lane scan plus one
+// exchange with lane^32.  A result block re-enters the matrix core as a B operand
+// (K index = t, N index = s) with no data movement: registers 8q..8q+7 are exactly
+// the 8 k-values of k-chunk q under the k-permutation
+//     t(q, hi, e) = 16q + 8*(e/4) + 4*hi + (e%4),
+// provided the A operand of that product is fetched with the same permutation
+// (two 4-element pieces of a [feature][t] tile).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ua {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __bf16 bf16;
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+constexpr float kAMax = (float)(1.0 - 1e-6);      // upper clamp of the affinity (forward and backward)
+constexpr float kAMinBwd = 1e-6f;                 // lower clamp used only in the backward divisor
+constexpr float kNegFill = -1e12f;                // bias of a (key, query) pair with key > query
+constexpr int kPad16 = 16;                        // bytes of padding per LDS row
+
+// ---------------------------------------------------------------------------------
+// MFMA operand fragment: 8 consecutive k-values of one row/column
+// ---------------------------------------------------------------------------------
+template <class T> struct alignas(16) Frag { T v[8]; };
+
+__device__ __forceinline__ void mma(f32x16& c, const Frag<bf16>& a, const Frag<bf16>& b) {
+  c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+// fp32: lane (row, hi) supplies k = hi of each 32x32x2 step; with 8 values per lane at
+// k = 16q + 8*hi + e the e-th step contracts {16q+e, 16q+8+e}.
+__device__ __forceinline__ void mma(f32x16& c, const Frag<float>& a, const Frag<float>& b) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a.v[e], b.v[e], c, 0, 0, 0);
+}
+
+template <class T> __device__ __forceinline__ T cvt(float x);
+template <> __device__ __forceinline__ float cvt<float>(float x) { return x; }
+template <> __device__ __forceinline__ bf16 cvt<bf16>(float x) { return (bf16)x; }
+
+// k-chunk q (0 or 1) of a result block as a B operand (see header comment)
+template <class T> __device__ __forceinline__ Frag<T> as_operand(const f32x16& c, int q) {
+  Frag<T> f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) f.v[e] = cvt<T>(c[8 * q + e]);
+  return f;
+}
+
+// 8 contiguous elements (global or LDS); p must be 16-byte aligned
+template <class T> __device__ __forceinline__ Frag<T> ld8(const T* p) {
+  Frag<T> f;
+  if constexpr (sizeof(T) == 2) {
+    *reinterpret_cast<uint4*>(&f) = *reinterpret_cast<const uint4*>(p);
+  } else {
+    reinterpret_cast<uint4*>(&f)[0] = reinterpret_cast<const uint4*>(p)[0];
+    reinterpret_cast<uint4*>(&f)[1] = reinterpret_cast<const uint4*>(p)[1];
+  }
+  return f;
+}
+// two 4-element pieces p[0..3], p[8..11] (the permuted-t A operand; p points at t = 16q + 4*hi)
+template <class T> __device__ __forceinline__ Frag<T> ld4x2(const T* p) {
+  Frag<T> f;
+  if constexpr (sizeof(T) == 2) {
+    reinterpret_cast<uint2*>(&f)[0] = *reinterpret_cast<const uint2*>(p);
+    reinterpret_cast<uint2*>(&f)[1] = *reinterpret_cast<const uint2*>(p + 8);
+  } else {
+    reinterpret_cast<uint4*>(&f)[0] = *reinterpret_cast<const uint4*>(p);
+    reinterpret_cast<uint4*>(&f)[1] = *reinterpret_cast<const uint4*>(p + 8);
+  }
+  return f;
+}
+
+// LDS row stride (elements) of a tile with `cols` payload columns
+template <class T> __host__ __device__ constexpr int lds_stride(int cols) { return cols + kPad16 / (int)sizeof(T); }
+
+// cooperative copy of a [rows][cols] tile, global (row stride gstride) -> LDS (row stride lstride)
+template <class T>
+__device__ __forceinline__ void stage_tile(T* __restrict__ lds, const T* __restrict__ g, int rows, int cols,
+                                           long gstride, int lstride, int tid, int nthreads) {
+  constexpr int V = 16 / (int)sizeof(T);
+  const int vec_per_row = cols / V;
+  for (int i = tid; i < rows * vec_per_row; i += nthreads) {
+    int r = i / vec_per_row, c = (i - r * vec_per_row) * V;
+    *reinterpret_cast<uint4*>(lds + r * lstride + c) = *reinterpret_cast<const uint4*>(g + (long)r * gstride + c);
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// lane exchanges
+// ---------------------------------------------------------------------------------
+__device__ __forceinline__ float xor_lane(float v, int mask) { return __shfl_xor(v, mask, 64); }
+
+// all-reduce over the 32 lanes that share l/32 (i.e. over the 32 keys of a block)
+__device__ __forceinline__ float allmax32(float v) {
+  v = fmaxf(v, xor_lane(v, 1)); v = fmaxf(v, xor_lane(v, 2)); v = fmaxf(v, xor_lane(v, 4));
+  v = fmaxf(v, xor_lane(v, 8)); v = fmaxf(v, xor_lane(v, 16));
+  return v;
+}
+__device__ __forceinline__ float allsum32(float v) {
+  v += xor_lane(v, 1); v += xor_lane(v, 2); v += xor_lane(v, 4); v += xor_lane(v, 8); v += xor_lane(v, 16);
+  return v;
+}
+
+// query index inside a 32-block of register v of lane-half hi
+__device__ __forceinline__ constexpr int t_of(int v, int hi) { return 8 * (v >> 2) + 4 * hi + (v & 3); }
+
+// Inclusive prefix sum over the 32 queries of a block (per key = per lane pair l, l^32).
+// On return x[v] = sum_{t' <= t(v)} x_in[t'];  returns the block total.
+__device__ __forceinline__ float block_prefix(f32x16& x, int hi) {
+  float gs[4], ps[4];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    x[4 * g + 1] += x[4 * g]; x[4 * g + 2] += x[4 * g + 1]; x[4 * g + 3] += x[4 * g + 2];
+    gs[g] = x[4 * g + 3];
+  }
+#pragma unroll
+  for (int g = 0; g < 4; ++g) ps[g] = xor_lane(gs[g], 32);
+  float run = 0.f;
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    float off = run + (hi ? ps[g] : 0.f);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) x[4 * g + e] += off;
+    run += gs[g] + ps[g];
+  }
+  return run;
+}
+// Inclusive suffix sum: x[v] = sum_{t' >= t(v)} x_in[t'];  returns the block total.
+__device__ __forceinline__ float block_suffix(f32x16& x, int hi) {
+  float gs[4], ps[4];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    x[4 * g + 2] += x[4 * g + 3]; x[4 * g + 1] += x[4 * g + 2]; x[4 * g] += x[4 * g + 1];
+    gs[g] = x[4 * g];
+  }
+#pragma unroll
+  for (int g = 0; g < 4; ++g) ps[g] = xor_lane(gs[g], 32);
+  float run = 0.f;
+#pragma unroll
+  for (int g = 3; g >= 0; --g) {
+    float off = run + (hi ? 0.f : ps[g]);     // the hi=1 piece of group g lies after the hi=0 piece
+#pragma unroll
+    for (int e = 0; e < 4; ++e) x[4 * g + e] += off;
+    run += gs[g] + ps[g];
+  }
+  return run;
+}
+
+// ---------------------------------------------------------------------------------
+// affinity:  A = relu(g)^(2/3) with g = (k_s sqrt(src_s)).(k_t sqrt(dest_t)), which equals
+// relu(k_s.k_t)^(2/3) src_s^(1/3) dest_t^(1/3);  returns log2(1 - min(A, 1-1e-6)).
+// ---------------------------------------------------------------------------------
+__device__ __forceinline__ float affinity(float g) {
+  // exp2(2/3 log2 g); log2(0) = -inf -> 0
+  return __builtin_amdgcn_exp2f((2.0f / 3.0f) * __builtin_amdgcn_logf(fmaxf(g, 0.f)));
+}
+__device__ __forceinline__ float log2_one_minus(float a) { return __builtin_amdgcn_logf(1.0f - fminf(a, kAMax)); }
+
+}  // namespace ua

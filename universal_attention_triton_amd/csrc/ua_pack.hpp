@@ -1,0 +1,79 @@
+// Layout kernels: bring user tensors (arbitrary strides, head dim d) into the padded,
+// contiguous working layouts the matrix-core kernels read, plus small row reductions.
+#pragma once
+#include "ua_common.hpp"
+
+namespace ua {
+
+// A tensor addressed as (z, row, col) with z = ((b*H + h)*R + r)*N + i; element offset
+//   b*sb + h*sh + r*sr + i*sn + (row / inner)*so + (row % inner)*si + col*sc
+struct RowsView {
+  const void* p;
+  long sb, sh, sr, sn, so, si, sc;
+  int inner, H, R, N;
+};
+__device__ __forceinline__ long rows_offset(const RowsView& v, int z, int row) {
+  int i = z % v.N; z /= v.N;
+  int r = z % v.R; z /= v.R;
+  int h = z % v.H, b = z / v.H;
+  return (long)b * v.sb + (long)h * v.sh + (long)r * v.sr + (long)i * v.sn + (long)(row / v.inner) * v.so +
+         (long)(row % v.inner) * v.si;
+}
+
+// x (dtype T) -> nat [Z][Lp][D] and/or tr [Z][D][Lp], zero padded (rows >= L, cols >= d).
+// gate (optional, dtype T, one value per row, addressed with z / gate_div): rows are scaled by sqrt(gate).
+template <class T, int D>
+__global__ void __launch_bounds__(256) k_pack(RowsView x, RowsView gate, int gate_div, T* __restrict__ nat,
+                                              T* __restrict__ tr, int d, int L, int Lp) {
+  __shared__ float tile[32][D + 1];
+  const int z = blockIdx.y, row0 = blockIdx.x * 32, tid = threadIdx.x;
+  const T* xp = reinterpret_cast<const T*>(x.p);
+  const T* gp = reinterpret_cast<const T*>(gate.p);
+  for (int i = tid; i < 32 * D; i += 256) {
+    int rr = i / D, col = i - rr * D, row = row0 + rr;
+    float val = 0.f;
+    if (row < L && col < d) {
+      val = (float)xp[rows_offset(x, z, row) + (long)col * x.sc];
+      if (gp) val *= __builtin_sqrtf((float)gp[rows_offset(gate, z / gate_div, row)]);
+    }
+    tile[rr][col] = val;
+    if (nat) nat[((long)z * Lp + row) * D + col] = cvt<T>(val);
+  }
+  if (!tr) return;
+  __syncthreads();
+  for (int i = tid; i < 32 * D; i += 256) {
+    int dd = i >> 5, rr = i & 31;
+    tr[((long)z * D + dd) * Lp + row0 + rr] = cvt<T>(tile[rr][dd]);
+  }
+}
+
+// delta[z][t] = sum_dd O[z][t][dd] * dO[z][t][dd] - sub[z][t]   (fp32; padded rows -> 0)
+// O, dO, sub are views (sub optional, float); one wave per row.
+// lse_in (optional, natural log, float view) is rewritten in log2 units into lse2 [Z][Lp].
+template <class T>
+__global__ void __launch_bounds__(256) k_delta(RowsView O, RowsView dO, RowsView sub, RowsView lse_in,
+                                               float* __restrict__ delta, float* __restrict__ lse2, int d, int L, int Lp) {
+  const int z = blockIdx.y, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + wave;
+  if (t >= Lp) return;
+  float s = 0.f;
+  if (t < L) {
+    const T* o = reinterpret_cast<const T*>(O.p) + rows_offset(O, z, t);
+    const T* g = reinterpret_cast<const T*>(dO.p) + rows_offset(dO, z, t);
+    for (int c = lane; c < d; c += 64) s += (float)o[(long)c * O.sc] * (float)g[(long)c * dO.sc];
+  }
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) s += __shfl_xor(s, m, 64);
+  if (lane == 0) {
+    if (sub.p && t < L) s -= reinterpret_cast<const float*>(sub.p)[rows_offset(sub, z, t)];
+    delta[(long)z * Lp + t] = s;
+    if (lse_in.p) lse2[(long)z * Lp + t] = (t < L) ? reinterpret_cast<const float*>(lse_in.p)[rows_offset(lse_in, z, t)] * kLog2e : 0.f;
+  }
+}
+
+// plain fill (kept as a kernel so that callers may capture the sequence in a HIP graph)
+__global__ void __launch_bounds__(256) k_zero(float4* __restrict__ p, size_t n16) {
+  for (size_t i = blockIdx.x * (size_t)256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256) p[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
+}  // namespace ua

@@ -1,0 +1,203 @@
+"""Host-side operators over the C ABI: tensor plumbing only (device memory, strides, streams)."""
+import ctypes
+
+import torch
+
+from . import _lib
+from ._lib import UaChunked, UaDesc, UaRows
+
+
+def _dtype_code(t):
+    if t.dtype == torch.bfloat16:
+        return _lib.UA_BF16
+    if t.dtype == torch.float32:
+        return _lib.UA_F32
+    raise TypeError("Universal Attention HIP kernels take float32 or bfloat16 tensors, got %s" % t.dtype)
+
+
+def _require_gpu(*ts):
+    for t in ts:
+        if not t.is_cuda:
+            raise _lib.UaError("Universal Attention HIP kernels need tensors on the GPU (got %s); there is no CPU path" % t.device)
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _last_contig(t):
+    return t if t.stride(-1) == 1 else t.contiguous()
+
+
+def _rows_k(t):
+    """kc / vc: [b,h,n,c,d]"""
+    return UaRows(t.data_ptr(), t.stride(0), t.stride(1), 0, t.stride(2), t.stride(3), t.shape[3])
+
+
+def _rows_q(t):
+    """xq: [b,h,r,l,d] or [b,h,r,_n,_c,d]"""
+    if t.dim() == 5:
+        return UaRows(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2), 0, t.stride(3), t.shape[3])
+    return UaRows(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2), t.stride(3), t.stride(4), t.shape[4])
+
+
+def _chunked(t):
+    """[b,h,r,l,d,n] tensor whose leading three dims are mergeable into one index"""
+    b, h, r = t.shape[:3]
+    if not (t.stride(0) == h * t.stride(1) and t.stride(1) == r * t.stride(2)):
+        t = t.contiguous()
+    return t, UaChunked(t.data_ptr(), t.stride(2), t.stride(3), t.stride(4), t.stride(5))
+
+
+def _desc(kc, xq, chunked, flags=0):
+    b, h, n, c, d = kc.shape
+    r = xq.shape[2]
+    return UaDesc(b, h, r, n * c, d, c if chunked else 0, _dtype_code(xq), flags)
+
+
+def _workspace(desc, op, device):
+    lib = _lib.load()
+    nbytes = lib.ua_workspace_bytes(ctypes.byref(desc), op)
+    if nbytes == 0:
+        raise _lib.UaError("unsupported problem: " + lib.ua_last_error().decode())
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
+def _prep(kc, vc, xq, static_src, static_dest):
+    _require_gpu(kc, vc, xq, static_src, static_dest)
+    if not (kc.dtype == vc.dtype == xq.dtype == static_src.dtype == static_dest.dtype):
+        raise TypeError("all five inputs must share one dtype")
+    b, h, n, c, d = kc.shape
+    kc, vc, xq = _last_contig(kc), _last_contig(vc), _last_contig(xq)
+    src = static_src.reshape(b, h, n * c).contiguous()
+    dest = static_dest.reshape(b, h, n * c).contiguous()
+    return kc, vc, xq, src, dest
+
+
+def chunked_forward(kc, vc, xq, static_src, static_dest, for_backward=False):
+    """-> out [b,h,r,l,d,n] (chunk-major storage, returned as a permuted view), denom [b,h,r,l,n], state"""
+    kc, vc, xq, src, dest = _prep(kc, vc, xq, static_src, static_dest)
+    lib = _lib.load()
+    b, h, n, c, d = kc.shape
+    r = xq.shape[2]
+    L = n * c
+    desc = _desc(kc, xq, True)
+    ws = _workspace(desc, _lib.UA_OP_BWD if for_backward else _lib.UA_OP_FWD, xq.device)
+    store = torch.empty(b, h, r, n, L, d, dtype=xq.dtype, device=xq.device)
+    out = store.permute(0, 1, 2, 4, 5, 3)
+    denom = torch.empty(b, h, r, L, n, dtype=xq.dtype, device=xq.device)
+    _, oc = _chunked(out)
+    _lib.check(lib.ua_fwd(ctypes.byref(desc), ctypes.byref(_rows_k(kc)), ctypes.byref(_rows_k(vc)), ctypes.byref(_rows_q(xq)),
+                          src.data_ptr(), dest.data_ptr(), ctypes.byref(oc), denom.data_ptr(), ws.data_ptr(), ws.numel(), _stream()),
+               "ua_fwd")
+    return out, denom, ws
+
+
+def chunked_backward(kc, vc, xq, static_src, static_dest, out, g_out, g_denom, ws=None, skip_masked=False):
+    kc, vc, xq, src, dest = _prep(kc, vc, xq, static_src, static_dest)
+    lib = _lib.load()
+    b, h, n, c, d = kc.shape
+    r = xq.shape[2]
+    L = n * c
+    desc = _desc(kc, xq, True, _lib.UA_FLAG_SKIP_MASKED if skip_masked else 0)
+    has_fwd = ws is not None
+    need = lib.ua_workspace_bytes(ctypes.byref(desc), _lib.UA_OP_BWD)
+    if ws is None or ws.numel() < need:
+        ws, has_fwd = _workspace(desc, _lib.UA_OP_BWD, xq.device), False
+    out_t, oc = _chunked(out)
+    g_out_t, gc = _chunked(g_out.to(xq.dtype))
+    gd = g_denom.float().contiguous()
+    dk = torch.empty(b, h, n, c, d, dtype=kc.dtype, device=kc.device)
+    dv = torch.empty_like(dk)
+    dq = torch.empty(b, h, r, L, d, dtype=xq.dtype, device=xq.device)
+    dsrc = torch.empty(b, h, L, dtype=src.dtype, device=src.device)
+    ddest = torch.empty_like(dsrc)
+    _lib.check(lib.ua_bwd(ctypes.byref(desc), ctypes.byref(_rows_k(kc)), ctypes.byref(_rows_k(vc)), ctypes.byref(_rows_q(xq)),
+                          src.data_ptr(), dest.data_ptr(), ctypes.byref(oc), ctypes.byref(gc), gd.data_ptr(), dk.data_ptr(),
+                          dv.data_ptr(), dq.data_ptr(), dsrc.data_ptr(), ddest.data_ptr(), ws.data_ptr(), ws.numel(),
+                          1 if has_fwd else 0, _stream()), "ua_bwd")
+    del out_t, g_out_t
+    return dk, dv, dq, dsrc, ddest
+
+
+def fused_forward(kc, vc, xq, static_src, static_dest, for_backward=False):
+    """-> O [b,h,r,l,d], lse [b,h,r,l] (float32), state"""
+    kc, vc, xq, src, dest = _prep(kc, vc, xq, static_src, static_dest)
+    lib = _lib.load()
+    b, h, n, c, d = kc.shape
+    r = xq.shape[2]
+    L = n * c
+    desc = _desc(kc, xq, False)
+    ws = _workspace(desc, _lib.UA_OP_FUSED_BWD if for_backward else _lib.UA_OP_FUSED_FWD, xq.device)
+    O = torch.empty(b, h, r, L, d, dtype=xq.dtype, device=xq.device)
+    lse = torch.empty(b, h, r, L, dtype=torch.float32, device=xq.device)
+    _lib.check(lib.ua_fused_fwd(ctypes.byref(desc), ctypes.byref(_rows_k(kc)), ctypes.byref(_rows_k(vc)), ctypes.byref(_rows_q(xq)),
+                                src.data_ptr(), dest.data_ptr(), O.data_ptr(), lse.data_ptr(), ws.data_ptr(), ws.numel(), _stream()),
+               "ua_fused_fwd")
+    return O, lse, ws
+
+
+def fused_backward(kc, vc, xq, static_src, static_dest, O, lse, dO, ws=None):
+    kc, vc, xq, src, dest = _prep(kc, vc, xq, static_src, static_dest)
+    lib = _lib.load()
+    b, h, n, c, d = kc.shape
+    r = xq.shape[2]
+    L = n * c
+    desc = _desc(kc, xq, False)
+    has_fwd = ws is not None
+    need = lib.ua_workspace_bytes(ctypes.byref(desc), _lib.UA_OP_FUSED_BWD)
+    if ws is None or ws.numel() < need:
+        ws, has_fwd = _workspace(desc, _lib.UA_OP_FUSED_BWD, xq.device), False
+    O = O.contiguous()
+    dO = dO.to(xq.dtype).contiguous()
+    lse = lse.float().contiguous()
+    dk = torch.empty(b, h, n, c, d, dtype=kc.dtype, device=kc.device)
+    dv = torch.empty_like(dk)
+    dq = torch.empty(b, h, r, L, d, dtype=xq.dtype, device=xq.device)
+    dsrc = torch.empty(b, h, L, dtype=src.dtype, device=src.device)
+    ddest = torch.empty_like(dsrc)
+    _lib.check(lib.ua_fused_bwd(ctypes.byref(desc), ctypes.byref(_rows_k(kc)), ctypes.byref(_rows_k(vc)), ctypes.byref(_rows_q(xq)),
+                                src.data_ptr(), dest.data_ptr(), O.data_ptr(), lse.data_ptr(), dO.data_ptr(), dk.data_ptr(),
+                                dv.data_ptr(), dq.data_ptr(), dsrc.data_ptr(), ddest.data_ptr(), ws.data_ptr(), ws.numel(),
+                                1 if has_fwd else 0, _stream()), "ua_fused_bwd")
+    return dk, dv, dq, dsrc, ddest
+
+
+def _merge_views(mat):
+    """mat [..., L, d, n] -> 4-D view [Z, L, d, n] whose Z stride is uniform"""
+    L, d, n = mat.shape[-3:]
+    m4 = mat.reshape(-1, L, d, n) if mat.dim() != 4 else mat
+    return m4, UaChunked(m4.data_ptr(), m4.stride(0), m4.stride(1), m4.stride(2), m4.stride(3))
+
+
+def merge_forward(mat, vec):
+    """SMVecMatMul forward: mat [..., L, d, n], vec [..., L, n] -> [..., L, d]"""
+    _require_gpu(mat, vec)
+    lib = _lib.load()
+    L, d, n = mat.shape[-3:]
+    m4, mc = _merge_views(mat)
+    vec_c = vec.to(mat.dtype).contiguous()
+    rows = m4.shape[0] * L
+    res = torch.empty(*mat.shape[:-2], d, dtype=mat.dtype, device=mat.device)
+    _lib.check(lib.ua_merge_fwd(_dtype_code(mat), rows, L, d, n, ctypes.byref(mc), vec_c.data_ptr(), res.data_ptr(), _stream()),
+               "ua_merge_fwd")
+    return res
+
+
+def merge_backward(mat, vec, g):
+    _require_gpu(mat, vec, g)
+    lib = _lib.load()
+    L, d, n = mat.shape[-3:]
+    m4, mc = _merge_views(mat)
+    vec_c = vec.to(mat.dtype).contiguous()
+    g_c = g.to(mat.dtype).contiguous()
+    rows = m4.shape[0] * L
+    # chunk-major storage: the gradient is consumed chunk by chunk by the chunked backward
+    store = torch.empty(m4.shape[0], n, L, d, dtype=mat.dtype, device=mat.device)
+    d4 = store.permute(0, 2, 3, 1)
+    dc = UaChunked(d4.data_ptr(), d4.stride(0), d4.stride(1), d4.stride(2), d4.stride(3))
+    d_vec = torch.empty(*vec.shape, dtype=mat.dtype, device=mat.device)
+    _lib.check(lib.ua_merge_bwd(_dtype_code(mat), rows, L, d, n, ctypes.byref(mc), vec_c.data_ptr(), g_c.data_ptr(), ctypes.byref(dc),
+                                d_vec.data_ptr(), _stream()), "ua_merge_bwd")
+    d_mat = d4.unflatten(0, tuple(mat.shape[:-3])) if mat.dim() != 4 else d4
+    return d_mat, d_vec.to(vec.dtype)
