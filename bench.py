@@ -1,0 +1,125 @@
+"""Headline benchmark: fused Universal Attention forward + backward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2] [--no-cpu]
+
+A step is one forward + backward of the fused operator over one synthetic batch (inputs resident in HBM,
+upstream gradient dO shaped like the output).  Prints ONE JSON line:
+  value     algorithmic TFLOP/s of the whole step ((1+2r) + (3+5r)) * d * L^2 * b * h flops, causal pairs only
+  roofline  the dominant kernel (k_bwd_keys: (3+5r) d L^2 b h flops per launch) against the bf16 dense MFMA peak,
+            its duration measured with hipEvents on the launch stream during the timed steps
+  cpu_baseline  the oracle (a port of the reference's torch operator) timed on the host cores on ONE kv head of the
+            same workload
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+CONFIGS = {  # BASELINE.json configs: b, h, r, L, d, chunk, dtype, gate_mean, passes
+    0: dict(b=1, h=4, r=1, L=512, d=64, c=64, dtype="fp32", mu=0.0),
+    1: dict(b=2, h=16, r=1, L=2048, d=64, c=128, dtype="bf16", mu=0.0),
+    2: dict(b=1, h=32, r=1, L=8192, d=128, c=128, dtype="bf16", mu=0.0),
+    3: dict(b=1, h=8, r=4, L=4096, d=128, c=128, dtype="bf16", mu=0.0),
+    4: dict(b=1, h=8, r=1, L=32768, d=128, c=128, dtype="bf16", mu=2.0),
+}
+PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}   # MI355X dense MFMA peaks
+
+
+def flops(cfg):
+    base = cfg["d"] * cfg["L"] ** 2 * cfg["b"] * cfg["h"]
+    r = cfg["r"]
+    return (1 + 2 * r) * base, (3 + 5 * r) * base
+
+
+def cpu_baseline(cfg, index):
+    """Oracle forward + backward (merge included) on one kv head of the workload, all host cores."""
+    from oracle import ua_oracle as orc
+    torch.set_num_threads(os.cpu_count())
+    dt = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float32
+    inp = orc.make_inputs(1, 1, cfg["r"], cfg["L"], cfg["d"], cfg["c"], dtype=dt, seed=1000 + index, gate_mean=cfg["mu"])
+    names = ("kc", "vc", "xq", "static_src", "static_dest")
+    t0 = time.time()
+    out, denom = orc.chunked_forward(*[inp[k] for k in names])
+    O = orc.merge(out, denom)
+    d_out, d_denom = orc.merge_backward(out, denom, inp["dO"])
+    orc.chunked_backward(*[inp[k] for k in names], d_out, d_denom.float())
+    dt_s = time.time() - t0
+    one = dict(cfg, b=1, h=1)
+    f, bw = flops(one)
+    del O
+    return {"value": (f + bw) / dt_s / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "seconds": round(dt_s, 2),
+            "sample": "1 of %d kv heads of the workload (b=1,h=1,r=%d,L=%d,d=%d,chunk=%d), chunked forward + merge + backward"
+                      % (cfg["b"] * cfg["h"], cfg["r"], cfg["L"], cfg["d"], cfg["c"])}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", type=int, default=2)
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (every (batch, kv head) is independent; nothing here uses a "
+                 "second device). Re-run with --gpus 1.")
+    from oracle import ua_oracle as orc
+    from universal_attention_triton_amd import _lib
+    from universal_attention_triton_amd.universal_attention import universal_attention
+
+    cfg = CONFIGS[args.config]
+    dt = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float32
+    inp = orc.make_inputs(cfg["b"], cfg["h"], cfg["r"], cfg["L"], cfg["d"], cfg["c"], dtype=dt, seed=1000 + args.config,
+                          gate_mean=cfg["mu"])
+    names = ("kc", "vc", "xq", "static_src", "static_dest")
+    leaves = [inp[k].cuda().requires_grad_() for k in names]
+    dO = inp["dO"].cuda()
+
+    def step():
+        O = universal_attention(*leaves)
+        return torch.autograd.grad(O, leaves, dO)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    _lib.prof_collect()
+    _lib.prof_enable(True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    _lib.prof_enable(False)
+    prof = _lib.prof_collect()
+    ms = elapsed * 1e3 / args.steps
+    f_fwd, f_bwd = flops(cfg)
+    kern = {k: round(v[1] / v[0], 4) for k, v in prof.items()}
+    dom_ms = prof["k_bwd_keys"][1] / prof["k_bwd_keys"][0]
+    peak = PEAK_TFLOPS[cfg["dtype"]]
+    achieved = f_bwd / (dom_ms * 1e-3) / 1e12
+    out = {
+        "metric": "fwd+bwd TFLOP/s (bf16, L=8192, d=128) on 1 MI355X", "value": round((f_fwd + f_bwd) / (ms * 1e-3) / 1e12, 2),
+        "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": cfg["dtype"], "data": "synthetic",
+        "config": {"workload": "BASELINE config %d: fused fwd+bwd b=%d h=%d r=%d L=%d d=%d, upstream dO like the output"
+                               % (args.config, cfg["b"], cfg["h"], cfg["r"], cfg["L"], cfg["d"]),
+                   "pct_of_mfma_peak": round(100 * (f_fwd + f_bwd) / (ms * 1e-3) / 1e12 / peak, 2),
+                   "kernel_ms": kern},
+        "roofline": {"bound": "mfma", "kernel": "k_bwd_keys", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
+                     "frac": round(achieved / peak, 4), "traffic": None},
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(cfg, args.config)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -126,6 +126,13 @@ int ua_tune_set(const ua_desc* desc, int op, int variant);
 /* Number of variants an op has for this description (>= 1), or a negative error. */
 int ua_tune_variants(const ua_desc* desc, int op);
 
+/* Per-kernel timing, no counterpart in the reference (its harness times whole calls with CUDA events,
+ * Universal_Attention/triton/_debug.py:413-446).  While enabled every kernel group the ops enqueue is bracketed
+ * by hipEvents on the launch stream.  ua_prof_collect synchronises the device, writes "name:count:total_ms;..."
+ * into buf (NUL terminated, truncated to cap) and clears the records; returns the untruncated length. */
+void ua_prof_enable(int on);
+int ua_prof_collect(char* buf, size_t cap);
+
 #ifdef __cplusplus
 }
 #endif

@@ -47,6 +47,8 @@ SIGNATURES = {
     "ua_tune_get": (c_int, [P(UaDesc), c_int]),
     "ua_tune_set": (c_int, [P(UaDesc), c_int, c_int]),
     "ua_tune_variants": (c_int, [P(UaDesc), c_int]),
+    "ua_prof_enable": (None, [c_int]),
+    "ua_prof_collect": (c_int, [ctypes.c_char_p, c_size_t]),
 }
 
 _lib = None
@@ -77,3 +79,19 @@ def check(code, what):
     if code < 0:
         raise UaError("%s failed (%d): %s" % (what, code, load().ua_last_error().decode()))
     return code
+
+
+def prof_enable(on=True):
+    load().ua_prof_enable(1 if on else 0)
+
+
+def prof_collect():
+    """-> {kernel group: (launches, total_ms)} since the last call; synchronises the device."""
+    buf = ctypes.create_string_buffer(8192)
+    load().ua_prof_collect(buf, len(buf))
+    out = {}
+    for item in buf.value.decode().split(";"):
+        if item:
+            name, cnt, ms = item.rsplit(":", 2)
+            out[name] = (int(cnt), float(ms))
+    return out

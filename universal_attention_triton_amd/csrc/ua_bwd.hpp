@@ -10,11 +10,11 @@
 //   P = exp(S - lse_t)            dS = P (V_s.dO_t - delta_t)           (delta carries -g_denom in chunked mode)
 //   dBias = sum_r dS              dlog[s,u] = sum_{t>=u} dBias[s,t]  (u > s)
 //   dA = dlog / (clamp(A,1e-6,1-1e-6) - 1) [A <= 1-1e-6]
-// With g = (k_s sqrt(src_s)).(k_u sqrt(dest_u)) and A = relu(g)^(2/3):
-//   dg = (2/3) dA A / g          (g > 0)
-//   dk_s += sqrt(src_s)  sum_u dg k~_u ,   k~_u = k_u sqrt(dest_u)      (row side, here)
-//   dk~_u = sum_s dg k^_s ,      k^_s = k_s sqrt(src_s)                 (column side, atomics)
-//   dsrc_s = sum_u dA A / (3 src_s) ;  ddest_u = (dk~_u . k~_u) / (2 dest_u)   (k_bwd_finish)
+// With g = k_s.k_u and A = relu(g)^(2/3) (src_s dest_u)^(1/3):
+//   dg = dA (2/3) g^(-1/3) (src_s dest_u)^(1/3)   (g > 0)         [= (2/3) dA A / g]
+//   dk_s += sum_u dg k_u   (row side, here)        dkcol_u = sum_s dg k_s   (column side, atomics)
+//   dsrc_s = sum_u dA A / (3 src_s)
+//   ddest_u = sum_s dA A / (3 dest_u) = (k_u . dkcol_u) / (2 dest_u)          (k_bwd_finish)
 #pragma once
 #include "ua_common.hpp"
 #include "ua_fwd.hpp"
@@ -23,14 +23,13 @@ namespace ua {
 
 template <class T>
 struct BwdArgs {
-  const T *Ks, *Kp, *Vp;        // [Zk][Lp][D]   key-side operands (stationary strips)
-  const T *Kd, *KdT;            // [Zk][Lp][D], [Zk][D][Lp]
-  const T *KT, *KsT;            // [Zk][D][Lp]   key-side, transposed (column-side products)
+  const T *Kp, *Vp;             // [Zk][Lp][D]
+  const T *KT;                  // [Zk][D][Lp]
+  const float *lsrc, *ldest;    // [Zk][Lp]  log2(gate)/3
   const T *Qp, *QT;             // [Zq][Lp][D], [Zq][D][Lp]
   const T *dOp, *dOT;           // [Zq*nch][Lp][D], [Zq*nch][D][Lp]
   const float *lse2, *delta;    // [Zq*nch][Lp]
   const float* C;               // [Zk][Lp/32][Lp]
-  const T* src;                 // [Zk][L] contiguous gate values (for sqrt(src))
   float *dQacc;                 // [Zq][Lp][D]  atomics
   float *dKdacc;                // [Zk][Lp][D]  atomics
   float *dKrow, *dVrow;         // [Zk][Lp][D]
@@ -74,19 +73,19 @@ __global__ void __launch_bounds__(64 * NW) k_bwd_keys(BwdArgs<T> a) {
   const bool wave_live = (32 * w) < wg_keys;
   const float inv_c = 1.0f / (float)a.c;
 
-  Frag<T> ks[NQ], kp[NQ], vf[NQ];
+  Frag<T> kp[NQ], vf[NQ];
   {
     const long ro = ((long)zk * Lp + spos) * D + 8 * hi;
 #pragma unroll
     for (int q = 0; q < NQ; ++q) {
-      if (valid) { ks[q] = ld8(a.Ks + ro + 16 * q); kp[q] = ld8(a.Kp + ro + 16 * q); vf[q] = ld8(a.Vp + ro + 16 * q); }
+      if (valid) { kp[q] = ld8(a.Kp + ro + 16 * q); vf[q] = ld8(a.Vp + ro + 16 * q); }
       else {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) { ks[q].v[e] = cvt<T>(0.f); kp[q].v[e] = cvt<T>(0.f); vf[q].v[e] = cvt<T>(0.f); }
+        for (int e = 0; e < 8; ++e) { kp[q].v[e] = cvt<T>(0.f); vf[q].v[e] = cvt<T>(0.f); }
       }
     }
   }
-  const float p_s = (valid && spos < L) ? __builtin_sqrtf((float)a.src[(long)zk * L + spos]) : 0.f;
+  const float la = valid ? a.lsrc[(long)zk * Lp + min(spos, Lp - 1)] : kGatePad;
 
   f32x16 dVt[NB], dKt[NB];
 #pragma unroll
@@ -99,19 +98,23 @@ __global__ void __launch_bounds__(64 * NW) k_bwd_keys(BwdArgs<T> a) {
     // mode of this wave for this query block: 2 = has decay part, 1 = score part only (no visible key), 0 = idle
     const int mode = !wave_live ? 0 : (tb >= tb_first ? 2 : ((a.chunked && !a.skip_masked) ? 1 : 0));
     __syncthreads();
-    stage_tile(sKd, a.Kd + ((long)zk * Lp + 32 * tb) * D, 32, D, D, LS, tid, NT);
-    stage_tile(sKdT, a.KdT + (long)zk * D * Lp + 32 * tb, D, 32, Lp, TS, tid, NT);
+    stage_tile(sKd, a.Kp + ((long)zk * Lp + 32 * tb) * D, 32, D, D, LS, tid, NT);
+    stage_tile(sKdT, a.KT + (long)zk * D * Lp + 32 * tb, D, 32, Lp, TS, tid, NT);
     __syncthreads();
-    f32x16 aff, bias, gk;
+    f32x16 aff, bias, gk;      // gk holds log2(relu(k_s.k_t)) after the forward recompute
+    float lab[16];
     if (mode == 2) {
       gk = (f32x16){0};
 #pragma unroll
-      for (int q = 0; q < NQ; ++q) mma(gk, ld8(sKd + col * LS + 16 * q + 8 * hi), ks[q]);
+      for (int q = 0; q < NQ; ++q) mma(gk, ld8(sKd + col * LS + 16 * q + 8 * hi), kp[q]);
+      load_t16(a.ldest + (long)zk * Lp + 32 * tb, hi, lab);
       f32x16 x;
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int tpos = 32 * tb + t_of(v, hi);
-        aff[v] = affinity(gk[v]);
+        lab[v] += la;
+        gk[v] = log2_relu(gk[v]);
+        aff[v] = affinity(gk[v], lab[v]);
         const float l2 = log2_one_minus(aff[v]);
         x[v] = (valid && tpos > spos) ? l2 : 0.f;
       }
@@ -197,17 +200,15 @@ __global__ void __launch_bounds__(64 * NW) k_bwd_keys(BwdArgs<T> a) {
         const float av = aff[v];
         const float den = fmaxf(fminf(av, kAMax), kAMinBwd) - 1.0f;
         const float dA = (av <= kAMax) ? dl * __builtin_amdgcn_rcpf(den) : 0.f;
-        const float wv = dA * av;
-        dsrc_acc += wv;
-        dg[v] = (gk[v] > 1e-30f) ? wv * (2.0f / 3.0f) * __builtin_amdgcn_rcpf(gk[v]) : 0.f;
+        dsrc_acc += dA * av;
+        // (2/3) g^(-1/3) (src dest)^(1/3); g <= 0 (log2 = -inf) contributes nothing
+        const float f = (2.0f / 3.0f) * __builtin_amdgcn_exp2f(__builtin_fmaf(gk[v], -1.0f / 3.0f, lab[v]));
+        dg[v] = (gk[v] > -1.0e30f) ? dA * f : 0.f;
       }
       dcar += tot;
-      f32x16 dgs;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) dgs[v] = dg[v] * p_s;
 #pragma unroll
       for (int q2 = 0; q2 < 2; ++q2) {
-        const Frag<T> b = as_operand<T>(dgs, q2);
+        const Frag<T> b = as_operand<T>(dg, q2);
 #pragma unroll
         for (int n = 0; n < NB; ++n) mma(dKt[n], ld4x2(sKdT + (32 * n + col) * TS + 16 * q2 + 4 * hi), b);
       }
@@ -228,7 +229,7 @@ __global__ void __launch_bounds__(64 * NW) k_bwd_keys(BwdArgs<T> a) {
           for (int kq = 0; kq < NKQ; ++kq) {
             const int s0 = wg_key0 + 16 * kq + 8 * hi;
             if (s0 + 8 <= Lp)
-              mma(acc, ld8(sX + col * SS + 16 * kq + 8 * hi), ld8(a.KsT + ((long)zk * D + 32 * n + col) * Lp + s0));
+              mma(acc, ld8(sX + col * SS + 16 * kq + 8 * hi), ld8(a.KT + ((long)zk * D + 32 * n + col) * Lp + s0));
           }
 #pragma unroll
           for (int v = 0; v < 16; ++v)
@@ -271,19 +272,19 @@ __global__ void __launch_bounds__(256) k_bwd_finish(const float* __restrict__ dK
     for (int c = lane; c < d; c += 64) dq[((long)z * L + t) * d + c] = cvt<T>(dQacc[((long)z * Lp + t) * D + c]);
   }
   if (z < Zk) {
-    const float sd = (float)dest[(long)z * L + t], q_s = __builtin_sqrtf(sd);
+    const float sd = (float)dest[(long)z * L + t];
     float dot = 0.f;
     for (int c = lane; c < d; c += 64) {
       const long i = ((long)z * Lp + t) * D + c;
       const float kd = dKdacc[i];
       dot += kd * (float)Kp[i];
-      dk[((long)z * L + t) * d + c] = cvt<T>(dKrow[i] + q_s * kd);
+      dk[((long)z * L + t) * d + c] = cvt<T>(dKrow[i] + kd);
       dv[((long)z * L + t) * d + c] = cvt<T>(dVrow[i]);
     }
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) dot += __shfl_xor(dot, m, 64);
     if (lane == 0) {
-      ddest[(long)z * L + t] = cvt<T>(dot / (2.0f * q_s));
+      ddest[(long)z * L + t] = cvt<T>(dot / (2.0f * sd));
       dsrc[(long)z * L + t] = cvt<T>(dsrc_raw[(long)z * Lp + t] / (3.0f * (float)src[(long)z * L + t]));
     }
   }

@@ -6,7 +6,9 @@
 #include <cstring>
 #include <map>
 #include <mutex>
+#include <string>
 #include <tuple>
+#include <vector>
 
 #include "../../include/ua.h"
 #include "ua_internal.hpp"
@@ -32,7 +34,7 @@ struct Layout {
   int D, Lp, nT, nch, Zk, Zq;
   size_t esz;
   // forward state
-  size_t Kp, KT, Ks, KsT, Kd, KdT, Vp, VT, Qp, QT, C, lse2, fwd_end;
+  size_t Kp, KT, Vp, VT, Qp, QT, lsrc, ldest, C, lse2, fwd_end;
   // backward scratch
   size_t dOp, dOT, delta, dQacc, dKdacc, dKrow, dVrow, dsrc_raw, total;
 };
@@ -47,7 +49,7 @@ int check_desc(const ua_desc* d, bool chunked) {
     const int c = d->chunk;
     if (c < 1 || d->L % c != 0) return fail(UA_EINVAL, "chunk %d must divide L = %d", c, d->L);
     if (!(c == 16 || c % 32 == 0) || c > 256) return fail(UA_EINVAL, "chunk %d unsupported: need 16 or a multiple of 32, at most 256", c);
-    if (d->L / c > ua::kMergeMaxN * 64) return fail(UA_EINVAL, "too many chunks");
+    if ((long)d->b * d->h * d->r * (d->L / c) > 65535) return fail(UA_EINVAL, "b*h*r*(L/chunk) exceeds the grid limit 65535");
   }
   return UA_OK;
 }
@@ -64,9 +66,9 @@ Layout make_layout(const ua_desc& d, bool chunked) {
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
   const size_t kbytes = (size_t)l.Zk * l.Lp * l.D * l.esz, qbytes = (size_t)l.Zq * l.Lp * l.D * l.esz;
-  l.Kp = take(kbytes); l.KT = take(kbytes); l.Ks = take(kbytes); l.KsT = take(kbytes);
-  l.Kd = take(kbytes); l.KdT = take(kbytes); l.Vp = take(kbytes); l.VT = take(kbytes);
+  l.Kp = take(kbytes); l.KT = take(kbytes); l.Vp = take(kbytes); l.VT = take(kbytes);
   l.Qp = take(qbytes); l.QT = take(qbytes);
+  l.lsrc = take((size_t)l.Zk * l.Lp * 4); l.ldest = take((size_t)l.Zk * l.Lp * 4);
   l.C = take((size_t)l.Zk * l.nT * l.Lp * 4);
   l.lse2 = take((size_t)l.Zq * l.nch * l.Lp * 4);
   l.fwd_end = off;
@@ -106,17 +108,34 @@ ua::RowsView chunked_view(const ua_chunked& c, int nch) {
 ua::RowsView null_view() { ua::RowsView v{}; v.inner = 1; v.H = v.R = v.N = 1; return v; }
 
 template <class T>
-hipError_t pack_t(int D, const ua::RowsView& x, const ua::RowsView& gate, int gate_div, void* nat, void* tr, int d, int L,
-                  int Lp, int Z, hipStream_t s) {
-  if (D == 64) hipLaunchKernelGGL((ua::k_pack<T, 64>), dim3(Lp / 32, Z), dim3(256), 0, s, x, gate, gate_div, (T*)nat, (T*)tr, d, L, Lp);
-  else hipLaunchKernelGGL((ua::k_pack<T, 128>), dim3(Lp / 32, Z), dim3(256), 0, s, x, gate, gate_div, (T*)nat, (T*)tr, d, L, Lp);
+hipError_t pack_t(int D, const ua::RowsView& x, void* nat, void* tr, int d, int L, int Lp, int Z, hipStream_t s) {
+  if (D == 64) hipLaunchKernelGGL((ua::k_pack<T, 64>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp);
+  else hipLaunchKernelGGL((ua::k_pack<T, 128>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp);
   return hipGetLastError();
 }
-hipError_t pack(int dtype, int D, const ua::RowsView& x, const ua::RowsView& gate, int gate_div, void* nat, void* tr, int d,
-                int L, int Lp, int Z, hipStream_t s) {
-  return dtype == UA_BF16 ? pack_t<ua::bf16>(D, x, gate, gate_div, nat, tr, d, L, Lp, Z, s)
-                          : pack_t<float>(D, x, gate, gate_div, nat, tr, d, L, Lp, Z, s);
+hipError_t pack(int dtype, int D, const ua::RowsView& x, void* nat, void* tr, int d, int L, int Lp, int Z, hipStream_t s) {
+  return dtype == UA_BF16 ? pack_t<ua::bf16>(D, x, nat, tr, d, L, Lp, Z, s) : pack_t<float>(D, x, nat, tr, d, L, Lp, Z, s);
 }
+
+// ---- optional per-kernel timing (hipEvents on the launch stream) ---------------------------
+struct ProfRec { const char* name; hipEvent_t e0, e1; };
+std::mutex g_prof_mu;
+bool g_prof_on = false;
+std::vector<ProfRec> g_prof;
+struct ProfScope {
+  hipEvent_t e1 = nullptr; hipStream_t s;
+  ProfScope(const char* name, hipStream_t stream) : s(stream) {
+    if (!g_prof_on) return;
+    ProfRec r{name, nullptr, nullptr};
+    if (hipEventCreate(&r.e0) != hipSuccess || hipEventCreate(&r.e1) != hipSuccess) return;
+    (void)hipEventRecord(r.e0, s);
+    e1 = r.e1;
+    std::lock_guard<std::mutex> g(g_prof_mu);
+    g_prof.push_back(r);
+  }
+  ~ProfScope() { if (e1) (void)hipEventRecord(e1, s); }
+};
+#define UA_PROF(name, s) ProfScope prof_scope_(name, s)
 
 #define UA_HIP(expr)                                                                         \
   do {                                                                                       \
@@ -142,16 +161,22 @@ hipError_t zero_fill(void* p, size_t bytes, hipStream_t s) {   // bytes is a mul
   return hipGetLastError();
 }
 
-// packs K (plain, src-scaled, dest-scaled), V and Q in both orientations
+// packs K, V and Q in both orientations and the log-gates
 int pack_inputs(const ua_desc& d, const Layout& l, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* src,
                 const void* dest, char* ws, hipStream_t s) {
+  UA_PROF("pack_inputs", s);
   const ua::RowsView K = rows_view(*kc, d.h, 1), V = rows_view(*vc, d.h, 1), Q = rows_view(*xq, d.h, d.r);
-  const ua::RowsView gs = contiguous_view(src, d.L, 1), gd = contiguous_view(dest, d.L, 1), none = null_view();
-  UA_HIP(pack(d.dtype, l.D, K, none, 1, ws + l.Kp, ws + l.KT, d.d, d.L, l.Lp, l.Zk, s));
-  UA_HIP(pack(d.dtype, l.D, K, gs, 1, ws + l.Ks, ws + l.KsT, d.d, d.L, l.Lp, l.Zk, s));
-  UA_HIP(pack(d.dtype, l.D, K, gd, 1, ws + l.Kd, ws + l.KdT, d.d, d.L, l.Lp, l.Zk, s));
-  UA_HIP(pack(d.dtype, l.D, V, none, 1, ws + l.Vp, ws + l.VT, d.d, d.L, l.Lp, l.Zk, s));
-  UA_HIP(pack(d.dtype, l.D, Q, none, 1, ws + l.Qp, ws + l.QT, d.d, d.L, l.Lp, l.Zq, s));
+  UA_HIP(pack(d.dtype, l.D, K, ws + l.Kp, ws + l.KT, d.d, d.L, l.Lp, l.Zk, s));
+  UA_HIP(pack(d.dtype, l.D, V, ws + l.Vp, ws + l.VT, d.d, d.L, l.Lp, l.Zk, s));
+  UA_HIP(pack(d.dtype, l.D, Q, ws + l.Qp, ws + l.QT, d.d, d.L, l.Lp, l.Zq, s));
+  const dim3 grid((l.Lp + 255) / 256, l.Zk);
+  if (d.dtype == UA_BF16)
+    hipLaunchKernelGGL((ua::k_gates<ua::bf16>), grid, dim3(256), 0, s, (const ua::bf16*)src, (const ua::bf16*)dest,
+                       (float*)(ws + l.lsrc), (float*)(ws + l.ldest), d.L, l.Lp);
+  else
+    hipLaunchKernelGGL((ua::k_gates<float>), grid, dim3(256), 0, s, (const float*)src, (const float*)dest,
+                       (float*)(ws + l.lsrc), (float*)(ws + l.ldest), d.L, l.Lp);
+  UA_HIP(hipGetLastError());
   return UA_OK;
 }
 
@@ -176,9 +201,15 @@ int tuned_variant(const ua_desc& d, int op) {
 }
 
 int run_fused_fwd_kernels(const ua_desc& d, const Layout& l, char* ws, void* O, float* lse, int variant, hipStream_t s) {
-  UA_HIP(ua::launch_carry(d.dtype, l.D, ws + l.Ks, ws + l.Kd, (float*)(ws + l.C), l.Lp, l.Zk, s));
-  UA_HIP(ua::launch_fwd_fused(d.dtype, l.D, variant, ws + l.Qp, ws + l.Kd, ws + l.Ks, ws + l.Kp, ws + l.VT,
-                              (const float*)(ws + l.C), O, lse, (float*)(ws + l.lse2), d.r, d.L, l.Lp, d.d, l.Zq, s));
+  {
+    UA_PROF("k_carry", s);
+    UA_HIP(ua::launch_carry(d.dtype, l.D, ws + l.Kp, (const float*)(ws + l.lsrc), (const float*)(ws + l.ldest),
+                            (float*)(ws + l.C), l.Lp, l.Zk, s));
+  }
+  UA_PROF("k_fwd_fused", s);
+  UA_HIP(ua::launch_fwd_fused(d.dtype, l.D, variant, ws + l.Qp, ws + l.Kp, ws + l.VT, (const float*)(ws + l.lsrc),
+                              (const float*)(ws + l.ldest), (const float*)(ws + l.C), O, lse, (float*)(ws + l.lse2), d.r,
+                              d.L, l.Lp, d.d, l.Zq, s));
   return UA_OK;
 }
 
@@ -202,18 +233,24 @@ hipError_t delta_t(const ua::RowsView& O, const ua::RowsView& dO, const ua::Rows
 
 int run_bwd_common(const ua_desc& d, const Layout& l, char* ws, bool chunked, const void* src, const void* dest, void* dkc,
                    void* dvc, void* dxq, void* dsrc, void* ddest, hipStream_t s) {
-  UA_HIP(zero_fill(ws + l.dQacc, (size_t)l.Zq * l.Lp * l.D * 4, s));
-  UA_HIP(zero_fill(ws + l.dKdacc, (size_t)l.Zk * l.Lp * l.D * 4, s));
+  {
+    UA_PROF("k_zero", s);
+    UA_HIP(zero_fill(ws + l.dQacc, (size_t)l.Zq * l.Lp * l.D * 4, s));
+    UA_HIP(zero_fill(ws + l.dKdacc, (size_t)l.Zk * l.Lp * l.D * 4, s));
+  }
   ua::BwdArgsV a{};
-  a.Ks = ws + l.Ks; a.Kp = ws + l.Kp; a.Vp = ws + l.Vp; a.Kd = ws + l.Kd; a.KdT = ws + l.KdT; a.KT = ws + l.KT;
-  a.KsT = ws + l.KsT; a.Qp = ws + l.Qp; a.QT = ws + l.QT; a.dOp = ws + l.dOp; a.dOT = ws + l.dOT;
+  a.Kp = ws + l.Kp; a.Vp = ws + l.Vp; a.KT = ws + l.KT; a.Qp = ws + l.Qp; a.QT = ws + l.QT; a.dOp = ws + l.dOp;
+  a.dOT = ws + l.dOT; a.lsrc = (const float*)(ws + l.lsrc); a.ldest = (const float*)(ws + l.ldest);
   a.lse2 = (const float*)(ws + l.lse2); a.delta = (const float*)(ws + l.delta); a.C = (const float*)(ws + l.C);
-  a.src = src;
   a.dQacc = (float*)(ws + l.dQacc); a.dKdacc = (float*)(ws + l.dKdacc); a.dKrow = (float*)(ws + l.dKrow);
   a.dVrow = (float*)(ws + l.dVrow); a.dsrc_raw = (float*)(ws + l.dsrc_raw);
   a.R = d.r; a.L = d.L; a.Lp = l.Lp; a.c = chunked ? d.chunk : 128; a.nch = l.nch; a.chunked = chunked ? 1 : 0;
   a.skip_masked = (d.flags & UA_FLAG_SKIP_MASKED) ? 1 : 0;
-  UA_HIP(ua::launch_bwd_keys(d.dtype, l.D, a, l.Zk, s));
+  {
+    UA_PROF("k_bwd_keys", s);
+    UA_HIP(ua::launch_bwd_keys(d.dtype, l.D, a, l.Zk, s));
+  }
+  UA_PROF("k_bwd_finish", s);
   if (d.dtype == UA_BF16) UA_HIP(finish_t<ua::bf16>(l, d, ws, src, dest, dkc, dvc, dxq, dsrc, ddest, s));
   else UA_HIP(finish_t<float>(l, d, ws, src, dest, dkc, dvc, dxq, dsrc, ddest, s));
   return UA_OK;
@@ -258,12 +295,16 @@ int ua_fused_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, cons
   const ua_desc& d = *desc;
   if (!ws_has_fwd) {
     if (int e = pack_inputs(d, l, kc, vc, xq, static_src, static_dest, w, s)) return e;
-    UA_HIP(ua::launch_carry(d.dtype, l.D, w + l.Ks, w + l.Kd, (float*)(w + l.C), l.Lp, l.Zk, s));
+    UA_HIP(ua::launch_carry(d.dtype, l.D, w + l.Kp, (const float*)(w + l.lsrc), (const float*)(w + l.ldest),
+                            (float*)(w + l.C), l.Lp, l.Zk, s));
   }
   const long rowsz = (long)d.L * d.d;
   const ua::RowsView Ov = contiguous_view(O, rowsz, d.d), dOv = contiguous_view(dO, rowsz, d.d);
   const ua::RowsView lsev = contiguous_view(lse, d.L, 1), none = null_view();
-  UA_HIP(pack(d.dtype, l.D, dOv, none, 1, w + l.dOp, w + l.dOT, d.d, d.L, l.Lp, l.Zq, s));
+  {
+    UA_PROF("pack_dO+delta", s);
+    UA_HIP(pack(d.dtype, l.D, dOv, w + l.dOp, w + l.dOT, d.d, d.L, l.Lp, l.Zq, s));
+  }
   if (d.dtype == UA_BF16) UA_HIP(delta_t<ua::bf16>(Ov, dOv, none, lsev, (float*)(w + l.delta), (float*)(w + l.lse2), d.d, d.L, l.Lp, l.Zq, s));
   else UA_HIP(delta_t<float>(Ov, dOv, none, lsev, (float*)(w + l.delta), (float*)(w + l.lse2), d.d, d.L, l.Lp, l.Zq, s));
   return run_bwd_common(d, l, w, false, static_src, static_dest, dkc, dvc, dxq, dsrc, ddest, s);
@@ -279,8 +320,9 @@ int ua_fwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
   hipStream_t s = (hipStream_t)stream;
   const ua_desc& d = *desc;
   if (int e = pack_inputs(d, l, kc, vc, xq, static_src, static_dest, w, s)) return e;
-  UA_HIP(ua::launch_fwd_chunked(d.dtype, l.D, w + l.Qp, w + l.Kd, w + l.Ks, w + l.Kp, w + l.VT, out->ptr, denom,
-                                (float*)(w + l.lse2), out->stride_z, out->stride_t, out->stride_d, out->stride_i, d.r, d.L,
+  UA_PROF("k_fwd_chunked", s);
+  UA_HIP(ua::launch_fwd_chunked(d.dtype, l.D, w + l.Qp, w + l.Kp, w + l.VT, (const float*)(w + l.lsrc),
+                                (const float*)(w + l.ldest), out->ptr, denom, (float*)(w + l.lse2), out->stride_z, out->stride_t, out->stride_d, out->stride_i, d.r, d.L,
                                 l.Lp, d.d, d.chunk, l.nch, l.Zk, s));
   return UA_OK;
 }
@@ -299,10 +341,11 @@ int ua_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
   if (!ws_has_fwd) {
     // recompute the per-chunk normalisers (the partial outputs themselves are passed in)
     if (int e = pack_inputs(d, l, kc, vc, xq, static_src, static_dest, w, s)) return e;
-    UA_HIP(ua::launch_fwd_chunked(d.dtype, l.D, w + l.Qp, w + l.Kd, w + l.Ks, w + l.Kp, w + l.VT, nullptr, nullptr,
-                                  (float*)(w + l.lse2), 0, 0, 0, 0, d.r, d.L, l.Lp, d.d, d.chunk, l.nch, l.Zk, s));
+    UA_HIP(ua::launch_fwd_chunked(d.dtype, l.D, w + l.Qp, w + l.Kp, w + l.VT, (const float*)(w + l.lsrc),
+                                  (const float*)(w + l.ldest), nullptr, nullptr, (float*)(w + l.lse2), 0, 0, 0, 0, d.r, d.L, l.Lp, d.d, d.chunk, l.nch, l.Zk, s));
   }
-  UA_HIP(ua::launch_carry(d.dtype, l.D, w + l.Ks, w + l.Kd, (float*)(w + l.C), l.Lp, l.Zk, s));
+  UA_HIP(ua::launch_carry(d.dtype, l.D, w + l.Kp, (const float*)(w + l.lsrc), (const float*)(w + l.ldest),
+                          (float*)(w + l.C), l.Lp, l.Zk, s));
   const ua::RowsView outv = chunked_view(*out, l.nch);
   ua_chunked gmut = *g_out;
   const ua::RowsView gv = chunked_view(gmut, l.nch), none = null_view();
@@ -310,7 +353,7 @@ int ua_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
   ua::RowsView gdv;
   gdv.p = g_denom; gdv.sb = (long)d.L * l.nch; gdv.sh = 0; gdv.sr = 0; gdv.sn = 1; gdv.so = 0; gdv.si = l.nch; gdv.sc = 1;
   gdv.inner = 1 << 30; gdv.H = 1; gdv.R = 1; gdv.N = l.nch;
-  UA_HIP(pack(d.dtype, l.D, gv, none, 1, w + l.dOp, w + l.dOT, d.d, d.L, l.Lp, l.Zq * l.nch, s));
+  UA_HIP(pack(d.dtype, l.D, gv, w + l.dOp, w + l.dOT, d.d, d.L, l.Lp, l.Zq * l.nch, s));
   if (d.dtype == UA_BF16) UA_HIP(delta_t<ua::bf16>(outv, gv, gdv, none, (float*)(w + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s));
   else UA_HIP(delta_t<float>(outv, gv, gdv, none, (float*)(w + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s));
   return run_bwd_common(d, l, w, true, static_src, static_dest, dkc, dvc, dxq, dsrc, ddest, s);
@@ -345,6 +388,28 @@ int ua_merge_bwd(int dtype, int64_t rows, int32_t L, int32_t d, int32_t n, const
   else hipLaunchKernelGGL((ua::k_merge_bwd<float>), grid, dim3(256), lds, s, m, (const float*)vec, (const float*)g, dm, (float*)d_vec, (long)rows, L, d, n);
   UA_HIP(hipGetLastError());
   return UA_OK;
+}
+
+void ua_prof_enable(int on) {
+  std::lock_guard<std::mutex> g(g_prof_mu);
+  g_prof_on = on != 0;
+}
+int ua_prof_collect(char* buf, size_t cap) {
+  if (hipDeviceSynchronize() != hipSuccess) return fail(UA_ELAUNCH, "synchronize failed");
+  std::lock_guard<std::mutex> g(g_prof_mu);
+  std::map<std::string, std::pair<int, double>> acc;
+  for (auto& r : g_prof) {
+    float ms = 0.f;
+    if (hipEventElapsedTime(&ms, r.e0, r.e1) == hipSuccess) { auto& a = acc[r.name]; a.first += 1; a.second += ms; }
+    hipEventDestroy(r.e0); hipEventDestroy(r.e1);
+  }
+  g_prof.clear();
+  std::string out;
+  char line[160];
+  for (auto& kv : acc) { snprintf(line, sizeof(line), "%s:%d:%.6f;", kv.first.c_str(), kv.second.first, kv.second.second); out += line; }
+  if (!buf || cap == 0) return (int)out.size();
+  snprintf(buf, cap, "%s", out.c_str());
+  return (int)out.size();
 }
 
 int ua_tune_variants(const ua_desc* desc, int op) {
@@ -386,8 +451,8 @@ int ua_autotune(const ua_desc* desc, int op, void* ws, size_t ws_bytes, ua_strea
   for (int v = 0; v < n; ++v) {
     for (int rep = 0; rep < 2; ++rep) {   // first pass warms up
       UA_HIP(hipEventRecord(e0, s));
-      hipError_t e = ua::launch_fwd_fused(desc->dtype, l.D, v, w + l.Qp, w + l.Kd, w + l.Ks, w + l.Kp, w + l.VT,
-                                          (const float*)(w + l.C), Otmp, lsetmp, (float*)(w + l.lse2), desc->r, desc->L,
+      hipError_t e = ua::launch_fwd_fused(desc->dtype, l.D, v, w + l.Qp, w + l.Kp, w + l.VT, (const float*)(w + l.lsrc),
+                                          (const float*)(w + l.ldest), (const float*)(w + l.C), Otmp, lsetmp, (float*)(w + l.lse2), desc->r, desc->L,
                                           l.Lp, desc->d, l.Zq, s);
       if (e != hipSuccess) return fail(UA_ELAUNCH, "autotune launch: %s", hipGetErrorString(e));
       UA_HIP(hipEventRecord(e1, s));

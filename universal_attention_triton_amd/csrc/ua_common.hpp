@@ -161,13 +161,23 @@ __device__ __forceinline__ float block_suffix(f32x16& x, int hi) {
 }
 
 // ---------------------------------------------------------------------------------
-// affinity:  A = relu(g)^(2/3) with g = (k_s sqrt(src_s)).(k_t sqrt(dest_t)), which equals
-// relu(k_s.k_t)^(2/3) src_s^(1/3) dest_t^(1/3);  returns log2(1 - min(A, 1-1e-6)).
+// affinity  A = relu(g)^(2/3) src_s^(1/3) dest_t^(1/3)  with g = k_s.k_t, evaluated as
+// exp2(2/3 log2 g + lab), lab = (log2 src_s + log2 dest_t)/3   (log2(0) = -inf -> A = 0).
 // ---------------------------------------------------------------------------------
-__device__ __forceinline__ float affinity(float g) {
-  // exp2(2/3 log2 g); log2(0) = -inf -> 0
-  return __builtin_amdgcn_exp2f((2.0f / 3.0f) * __builtin_amdgcn_logf(fmaxf(g, 0.f)));
+__device__ __forceinline__ float log2_relu(float g) { return __builtin_amdgcn_logf(fmaxf(g, 0.f)); }
+__device__ __forceinline__ float affinity(float lg, float lab) {
+  return __builtin_amdgcn_exp2f(__builtin_fmaf(lg, 2.0f / 3.0f, lab));
 }
 __device__ __forceinline__ float log2_one_minus(float a) { return __builtin_amdgcn_logf(1.0f - fminf(a, kAMax)); }
+constexpr float kGatePad = -1.0e4f;   // log-gate of padded rows: makes their affinity exactly 0
+
+// the 16 per-query values of a 32-block that a lane needs (t = 8g + 4hi + e), from a float[32]
+__device__ __forceinline__ void load_t16(const float* __restrict__ p32, int hi, float (&out)[16]) {
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const float4 x = *reinterpret_cast<const float4*>(p32 + 8 * g + 4 * hi);
+    out[4 * g] = x.x; out[4 * g + 1] = x.y; out[4 * g + 2] = x.z; out[4 * g + 3] = x.w;
+  }
+}
 
 }  // namespace ua

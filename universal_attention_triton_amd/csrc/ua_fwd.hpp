@@ -19,8 +19,8 @@ constexpr float kNegBig = -1.0e30f;
 // grid (Lp/128, Z_kv); 4 waves, wave w owns keys 32*(4*bx+w) .. +31 and sweeps query blocks.
 // ---------------------------------------------------------------------------------------------
 template <class T, int D>
-__global__ void __launch_bounds__(256) k_carry(const T* __restrict__ Ks, const T* __restrict__ Kd,
-                                               float* __restrict__ C, int Lp) {
+__global__ void __launch_bounds__(256) k_carry(const T* __restrict__ Kp, const float* __restrict__ lsrc,
+                                               const float* __restrict__ ldest, float* __restrict__ C, int Lp) {
   extern __shared__ __align__(16) char smem[];
   T* sKd = reinterpret_cast<T*>(smem);
   constexpr int NQ = D / 16, LS = lds_stride<T>(D);
@@ -28,24 +28,27 @@ __global__ void __launch_bounds__(256) k_carry(const T* __restrict__ Ks, const T
   const int z = blockIdx.y, nT = Lp / 32, sb = 4 * blockIdx.x + w;
   Frag<T> ks[NQ];
   {
-    const T* krow = Ks + ((long)z * Lp + 32 * sb + col) * D + 8 * hi;
+    const T* krow = Kp + ((long)z * Lp + 32 * sb + col) * D + 8 * hi;
 #pragma unroll
     for (int q = 0; q < NQ; ++q) ks[q] = ld8(krow + 16 * q);
   }
+  const float la = lsrc[(long)z * Lp + 32 * sb + col];
   float carry = 0.f;
   float* Cz = C + (long)z * nT * Lp;
   for (int tb = 4 * blockIdx.x; tb < nT; ++tb) {
     __syncthreads();
-    stage_tile(sKd, Kd + ((long)z * Lp + 32 * tb) * D, 32, D, D, LS, tid, 256);
+    stage_tile(sKd, Kp + ((long)z * Lp + 32 * tb) * D, 32, D, D, LS, tid, 256);
     __syncthreads();
     if (tb >= sb) {
       f32x16 g = {0};
 #pragma unroll
       for (int q = 0; q < NQ; ++q) mma(g, ld8(sKd + col * LS + 16 * q + 8 * hi), ks[q]);
+      float lb[16];
+      load_t16(ldest + (long)z * Lp + 32 * tb, hi, lb);
       float tot = 0.f;
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        float l2 = log2_one_minus(affinity(g[v]));
+        float l2 = log2_one_minus(affinity(log2_relu(g[v]), la + lb[v]));
         if (tb == sb && t_of(v, hi) <= col) l2 = 0.f;
         tot += l2;
       }
@@ -58,19 +61,18 @@ __global__ void __launch_bounds__(256) k_carry(const T* __restrict__ Ks, const T
 
 // ---------------------------------------------------------------------------------------------
 // Fused forward.  grid (Lp/128, Z_q) ; 4 waves ; wave w owns queries 32*(4*jt+w) .. +31.
-// Per key tile of BS keys: G = Kd_t.Ks_s -> log2(1-A) -> in-lane prefix + carry = bias,
+// Per key tile of BS keys: G = K_t.K_s -> A -> log2(1-A) -> in-lane prefix + carry = bias,
 // S = Q_t.K_s, online softmax over keys, P^T through LDS, O += P^T V.
 // ---------------------------------------------------------------------------------------------
 template <class T, int D, int BS>
-__global__ void __launch_bounds__(256) k_fwd_fused(const T* __restrict__ Qp, const T* __restrict__ Kd,
-                                                   const T* __restrict__ Ks, const T* __restrict__ Kp,
-                                                   const T* __restrict__ VT, const float* __restrict__ C,
+__global__ void __launch_bounds__(256) k_fwd_fused(const T* __restrict__ Qp, const T* __restrict__ Kp,
+                                                   const T* __restrict__ VT, const float* __restrict__ lsrc,
+                                                   const float* __restrict__ ldest, const float* __restrict__ C,
                                                    T* __restrict__ O, float* __restrict__ lse, float* __restrict__ lse2,
                                                    int R, int L, int Lp, int d) {
   extern __shared__ __align__(16) char smem[];
   constexpr int NQ = D / 16, NB = D / 32, NSB = BS / 32, LS = lds_stride<T>(D), PS = lds_stride<T>(BS);
-  T* sKs = reinterpret_cast<T*>(smem);
-  T* sKp = sKs + BS * LS;
+  T* sKp = reinterpret_cast<T*>(smem);
   T* sVT = sKp + BS * LS;
   T* sP = sVT + D * PS;
   const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, col = lane & 31, hi = lane >> 5;
@@ -81,10 +83,12 @@ __global__ void __launch_bounds__(256) k_fwd_fused(const T* __restrict__ Qp, con
   Frag<T> qf[NQ], kdf[NQ];
   {
     const T* qrow = Qp + ((long)zq * Lp + 32 * tb + col) * D + 8 * hi;
-    const T* krow = Kd + ((long)zk * Lp + 32 * tb + col) * D + 8 * hi;
+    const T* krow = Kp + ((long)zk * Lp + 32 * tb + col) * D + 8 * hi;
 #pragma unroll
     for (int q = 0; q < NQ; ++q) { qf[q] = ld8(qrow + 16 * q); kdf[q] = ld8(krow + 16 * q); }
   }
+  float lb[16];
+  load_t16(ldest + (long)zk * Lp + 32 * tb, hi, lb);
   f32x16 o[NB];
 #pragma unroll
   for (int n = 0; n < NB; ++n) o[n] = (f32x16){0};
@@ -96,7 +100,6 @@ __global__ void __launch_bounds__(256) k_fwd_fused(const T* __restrict__ Qp, con
   const int n_kt = (128 * jt + 128) / BS;
   for (int kt = 0; kt < n_kt; ++kt) {
     __syncthreads();
-    stage_tile(sKs, Ks + ((long)zk * Lp + BS * kt) * D, BS, D, D, LS, tid, 256);
     stage_tile(sKp, Kp + ((long)zk * Lp + BS * kt) * D, BS, D, D, LS, tid, 256);
     stage_tile(sVT, VT + (long)zk * D * Lp + BS * kt, D, BS, Lp, PS, tid, 256);
     __syncthreads();
@@ -107,11 +110,12 @@ __global__ void __launch_bounds__(256) k_fwd_fused(const T* __restrict__ Qp, con
       if (sbk <= tb) {
         f32x16 g = {0};
 #pragma unroll
-        for (int q = 0; q < NQ; ++q) mma(g, kdf[q], ld8(sKs + (32 * j + col) * LS + 16 * q + 8 * hi));
+        for (int q = 0; q < NQ; ++q) mma(g, kdf[q], ld8(sKp + (32 * j + col) * LS + 16 * q + 8 * hi));
         const bool diag = (sbk == tb);
+        const float la = lsrc[(long)zk * Lp + 32 * sbk + col];
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          float l2 = log2_one_minus(affinity(g[v]));
+          float l2 = log2_one_minus(affinity(log2_relu(g[v]), la + lb[v]));
           g[v] = (diag && t_of(v, hi) <= col) ? 0.f : l2;
         }
         block_prefix(g, hi);
@@ -189,9 +193,9 @@ __global__ void __launch_bounds__(256) k_fwd_fused(const T* __restrict__ Qp, con
 // out element (zq, t, dd, i) is written at  zq*o_sz + t*o_st + dd*o_sd + i*o_si.
 // ---------------------------------------------------------------------------------------------
 template <class T, int D, int NW>
-__global__ void __launch_bounds__(64 * NW) k_fwd_chunked(const T* __restrict__ Qp, const T* __restrict__ Kd,
-                                                         const T* __restrict__ Ks, const T* __restrict__ Kp,
-                                                         const T* __restrict__ VT, T* __restrict__ out,
+__global__ void __launch_bounds__(64 * NW) k_fwd_chunked(const T* __restrict__ Qp, const T* __restrict__ Kp,
+                                                         const T* __restrict__ VT, const float* __restrict__ lsrc,
+                                                         const float* __restrict__ ldest, T* __restrict__ out,
                                                          T* __restrict__ denom, float* __restrict__ lse2,
                                                          long o_sz, long o_st, long o_sd, long o_si,
                                                          int R, int L, int Lp, int d, int c, int nch) {
@@ -211,19 +215,19 @@ __global__ void __launch_bounds__(64 * NW) k_fwd_chunked(const T* __restrict__ Q
   const int nTr = (L + 31) / 32, tb0 = (i * c) / 32;
   const float kFill2 = kNegFill * kLog2e;
 
-  Frag<T> ks[NQ], kp[NQ];
+  Frag<T> kp[NQ];
   {
-    const T* a = Ks + ((long)zk * Lp + spos) * D + 8 * hi;
     const T* b = Kp + ((long)zk * Lp + spos) * D + 8 * hi;
 #pragma unroll
     for (int q = 0; q < NQ; ++q) {
-      if (valid) { ks[q] = ld8(a + 16 * q); kp[q] = ld8(b + 16 * q); }
+      if (valid) kp[q] = ld8(b + 16 * q);
       else {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) { ks[q].v[e] = cvt<T>(0.f); kp[q].v[e] = cvt<T>(0.f); }
+        for (int e = 0; e < 8; ++e) kp[q].v[e] = cvt<T>(0.f);
       }
     }
   }
+  const float la = valid ? lsrc[(long)zk * Lp + spos] : kGatePad;
   // V^T operands of this wave's output column blocks: lane <-> dd, k <-> key inside the chunk
   Frag<T> vt[NBW][NKQ];
   Frag<T> ones;
@@ -269,17 +273,19 @@ __global__ void __launch_bounds__(64 * NW) k_fwd_chunked(const T* __restrict__ Q
   float carry = 0.f;
   for (int tb = tb0; tb < nTr; ++tb) {
     __syncthreads();
-    stage_tile(sKd, Kd + ((long)zk * Lp + 32 * tb) * D, 32, D, D, LS, tid, NT);
+    stage_tile(sKd, Kp + ((long)zk * Lp + 32 * tb) * D, 32, D, D, LS, tid, NT);
     __syncthreads();
     f32x16 bias;
     {
       f32x16 g = {0};
 #pragma unroll
-      for (int q = 0; q < NQ; ++q) mma(g, ld8(sKd + col * LS + 16 * q + 8 * hi), ks[q]);
+      for (int q = 0; q < NQ; ++q) mma(g, ld8(sKd + col * LS + 16 * q + 8 * hi), kp[q]);
+      float lb[16];
+      load_t16(ldest + (long)zk * Lp + 32 * tb, hi, lb);
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int tpos = 32 * tb + t_of(v, hi);
-        float l2 = log2_one_minus(affinity(g[v]));
+        float l2 = log2_one_minus(affinity(log2_relu(g[v]), la + lb[v]));
         g[v] = (valid && tpos > spos) ? l2 : 0.f;
       }
       const float tot = block_prefix(g, hi);

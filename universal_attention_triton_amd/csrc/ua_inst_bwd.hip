@@ -7,9 +7,9 @@ namespace ua {
 template <class T, int D, int NW>
 static hipError_t bwd_t(const BwdArgsV& v, int Zk, hipStream_t s) {
   BwdArgs<T> a;
-  a.Ks = (const T*)v.Ks; a.Kp = (const T*)v.Kp; a.Vp = (const T*)v.Vp; a.Kd = (const T*)v.Kd; a.KdT = (const T*)v.KdT;
-  a.KT = (const T*)v.KT; a.KsT = (const T*)v.KsT; a.Qp = (const T*)v.Qp; a.QT = (const T*)v.QT;
-  a.dOp = (const T*)v.dOp; a.dOT = (const T*)v.dOT; a.lse2 = v.lse2; a.delta = v.delta; a.C = v.C; a.src = (const T*)v.src;
+  a.Kp = (const T*)v.Kp; a.Vp = (const T*)v.Vp; a.KT = (const T*)v.KT; a.Qp = (const T*)v.Qp; a.QT = (const T*)v.QT;
+  a.dOp = (const T*)v.dOp; a.dOT = (const T*)v.dOT; a.lsrc = v.lsrc; a.ldest = v.ldest; a.lse2 = v.lse2; a.delta = v.delta;
+  a.C = v.C;
   a.dQacc = v.dQacc; a.dKdacc = v.dKdacc; a.dKrow = v.dKrow; a.dVrow = v.dVrow; a.dsrc_raw = v.dsrc_raw;
   a.R = v.R; a.L = v.L; a.Lp = v.Lp; a.c = v.c; a.nch = v.nch; a.chunked = v.chunked; a.skip_masked = v.skip_masked;
   constexpr int CP = 32 * NW;

@@ -10,31 +10,32 @@ static void allow_lds(K kernel, size_t bytes) {
 }
 
 template <class T, int D>
-static hipError_t carry_t(const void* Ks, const void* Kd, float* C, int Lp, int Zk, hipStream_t s) {
+static hipError_t carry_t(const void* Kp, const float* lsrc, const float* ldest, float* C, int Lp, int Zk, hipStream_t s) {
   const size_t lds = 32 * lds_stride<T>(D) * sizeof(T);
-  hipLaunchKernelGGL((k_carry<T, D>), dim3(Lp / 128, Zk), dim3(256), lds, s, (const T*)Ks, (const T*)Kd, C, Lp);
+  hipLaunchKernelGGL((k_carry<T, D>), dim3(Lp / 128, Zk), dim3(256), lds, s, (const T*)Kp, lsrc, ldest, C, Lp);
   return hipGetLastError();
 }
-hipError_t launch_carry(int dtype, int D, const void* Ks, const void* Kd, float* C, int Lp, int Zk, hipStream_t s) {
-  if (dtype == 1) return D == 64 ? carry_t<bf16, 64>(Ks, Kd, C, Lp, Zk, s) : carry_t<bf16, 128>(Ks, Kd, C, Lp, Zk, s);
-  return D == 64 ? carry_t<float, 64>(Ks, Kd, C, Lp, Zk, s) : carry_t<float, 128>(Ks, Kd, C, Lp, Zk, s);
+hipError_t launch_carry(int dtype, int D, const void* Kp, const float* lsrc, const float* ldest, float* C, int Lp, int Zk,
+                        hipStream_t s) {
+  if (dtype == 1) return D == 64 ? carry_t<bf16, 64>(Kp, lsrc, ldest, C, Lp, Zk, s) : carry_t<bf16, 128>(Kp, lsrc, ldest, C, Lp, Zk, s);
+  return D == 64 ? carry_t<float, 64>(Kp, lsrc, ldest, C, Lp, Zk, s) : carry_t<float, 128>(Kp, lsrc, ldest, C, Lp, Zk, s);
 }
 
 template <class T, int D, int BS>
-static hipError_t fused_t(const void* Qp, const void* Kd, const void* Ks, const void* Kp, const void* VT, const float* C,
-                          void* O, float* lse, float* lse2, int R, int L, int Lp, int d, int Zq, hipStream_t s) {
-  const size_t lds = (2 * BS * lds_stride<T>(D) + D * lds_stride<T>(BS) + 4 * 32 * lds_stride<T>(BS)) * sizeof(T);
+static hipError_t fused_t(const void* Qp, const void* Kp, const void* VT, const float* lsrc, const float* ldest,
+                          const float* C, void* O, float* lse, float* lse2, int R, int L, int Lp, int d, int Zq, hipStream_t s) {
+  const size_t lds = (BS * lds_stride<T>(D) + D * lds_stride<T>(BS) + 4 * 32 * lds_stride<T>(BS)) * sizeof(T);
   allow_lds(k_fwd_fused<T, D, BS>, lds);
-  hipLaunchKernelGGL((k_fwd_fused<T, D, BS>), dim3(Lp / 128, Zq), dim3(256), lds, s, (const T*)Qp, (const T*)Kd,
-                     (const T*)Ks, (const T*)Kp, (const T*)VT, C, (T*)O, lse, lse2, R, L, Lp, d);
+  hipLaunchKernelGGL((k_fwd_fused<T, D, BS>), dim3(Lp / 128, Zq), dim3(256), lds, s, (const T*)Qp, (const T*)Kp,
+                     (const T*)VT, lsrc, ldest, C, (T*)O, lse, lse2, R, L, Lp, d);
   return hipGetLastError();
 }
 // variants: key-tile size per LDS stage
 int fwd_fused_variants(int dtype, int D) { (void)D; return dtype == 1 ? 2 : 1; }
-hipError_t launch_fwd_fused(int dtype, int D, int variant, const void* Qp, const void* Kd, const void* Ks, const void* Kp,
-                            const void* VT, const float* C, void* O, float* lse, float* lse2, int R, int L, int Lp, int d,
-                            int Zq, hipStream_t s) {
-#define UA_ARGS Qp, Kd, Ks, Kp, VT, C, O, lse, lse2, R, L, Lp, d, Zq, s
+hipError_t launch_fwd_fused(int dtype, int D, int variant, const void* Qp, const void* Kp, const void* VT,
+                            const float* lsrc, const float* ldest, const float* C, void* O, float* lse, float* lse2, int R,
+                            int L, int Lp, int d, int Zq, hipStream_t s) {
+#define UA_ARGS Qp, Kp, VT, lsrc, ldest, C, O, lse, lse2, R, L, Lp, d, Zq, s
   if (dtype == 1) {
     if (D == 64) return variant == 1 ? fused_t<bf16, 64, 128>(UA_ARGS) : fused_t<bf16, 64, 64>(UA_ARGS);
     return variant == 1 ? fused_t<bf16, 128, 128>(UA_ARGS) : fused_t<bf16, 128, 64>(UA_ARGS);
@@ -44,21 +45,21 @@ hipError_t launch_fwd_fused(int dtype, int D, int variant, const void* Qp, const
 }
 
 template <class T, int D, int NW>
-static hipError_t chunked_t(const void* Qp, const void* Kd, const void* Ks, const void* Kp, const void* VT, void* out,
+static hipError_t chunked_t(const void* Qp, const void* Kp, const void* VT, const float* lsrc, const float* ldest, void* out,
                             void* denom, float* lse2, long o_sz, long o_st, long o_sd, long o_si, int R, int L, int Lp,
                             int d, int c, int nch, int Zk, hipStream_t s) {
   const size_t lds = (64 * lds_stride<T>(D) + 32 * lds_stride<T>(32 * NW)) * sizeof(T) + (NW * 32 + D) * sizeof(float);
   allow_lds(k_fwd_chunked<T, D, NW>, lds);
-  hipLaunchKernelGGL((k_fwd_chunked<T, D, NW>), dim3(nch, Zk), dim3(64 * NW), lds, s, (const T*)Qp, (const T*)Kd,
-                     (const T*)Ks, (const T*)Kp, (const T*)VT, (T*)out, (T*)denom, lse2, o_sz, o_st, o_sd, o_si, R, L, Lp,
+  hipLaunchKernelGGL((k_fwd_chunked<T, D, NW>), dim3(nch, Zk), dim3(64 * NW), lds, s, (const T*)Qp, (const T*)Kp,
+                     (const T*)VT, lsrc, ldest, (T*)out, (T*)denom, lse2, o_sz, o_st, o_sd, o_si, R, L, Lp,
                      d, c, nch);
   return hipGetLastError();
 }
 template <class T, int D>
-static hipError_t chunked_nw(int NW, const void* Qp, const void* Kd, const void* Ks, const void* Kp, const void* VT,
+static hipError_t chunked_nw(int NW, const void* Qp, const void* Kp, const void* VT, const float* lsrc, const float* ldest,
                              void* out, void* denom, float* lse2, long o_sz, long o_st, long o_sd, long o_si, int R, int L,
                              int Lp, int d, int c, int nch, int Zk, hipStream_t s) {
-#define UA_ARGS Qp, Kd, Ks, Kp, VT, out, denom, lse2, o_sz, o_st, o_sd, o_si, R, L, Lp, d, c, nch, Zk, s
+#define UA_ARGS Qp, Kp, VT, lsrc, ldest, out, denom, lse2, o_sz, o_st, o_sd, o_si, R, L, Lp, d, c, nch, Zk, s
   switch (NW) {
     case 1: return chunked_t<T, D, 1>(UA_ARGS);
     case 2: return chunked_t<T, D, 2>(UA_ARGS);
@@ -67,11 +68,11 @@ static hipError_t chunked_nw(int NW, const void* Qp, const void* Kd, const void*
   }
 #undef UA_ARGS
 }
-hipError_t launch_fwd_chunked(int dtype, int D, const void* Qp, const void* Kd, const void* Ks, const void* Kp,
-                              const void* VT, void* out, void* denom, float* lse2, long o_sz, long o_st, long o_sd,
+hipError_t launch_fwd_chunked(int dtype, int D, const void* Qp, const void* Kp, const void* VT, const float* lsrc,
+                              const float* ldest, void* out, void* denom, float* lse2, long o_sz, long o_st, long o_sd,
                               long o_si, int R, int L, int Lp, int d, int c, int nch, int Zk, hipStream_t s) {
   int NW = c <= 32 ? 1 : c <= 64 ? 2 : c <= 128 ? 4 : 8;
-#define UA_ARGS NW, Qp, Kd, Ks, Kp, VT, out, denom, lse2, o_sz, o_st, o_sd, o_si, R, L, Lp, d, c, nch, Zk, s
+#define UA_ARGS NW, Qp, Kp, VT, lsrc, ldest, out, denom, lse2, o_sz, o_st, o_sd, o_si, R, L, Lp, d, c, nch, Zk, s
   if (dtype == 1) return D == 64 ? chunked_nw<bf16, 64>(UA_ARGS) : chunked_nw<bf16, 128>(UA_ARGS);
   return D == 64 ? chunked_nw<float, 64>(UA_ARGS) : chunked_nw<float, 128>(UA_ARGS);
 #undef UA_ARGS

@@ -8,21 +8,21 @@ namespace ua {
 
 // type-erased argument block of k_bwd_keys (same field order as BwdArgs<T>)
 struct BwdArgsV {
-  const void *Ks, *Kp, *Vp, *Kd, *KdT, *KT, *KsT, *Qp, *QT, *dOp, *dOT;
-  const float *lse2, *delta, *C;
-  const void* src;
+  const void *Kp, *Vp, *KT, *Qp, *QT, *dOp, *dOT;
+  const float *lsrc, *ldest, *lse2, *delta, *C;
   float *dQacc, *dKdacc, *dKrow, *dVrow, *dsrc_raw;
   int R, L, Lp, c, nch, chunked, skip_masked;
 };
 
 // Every launcher returns hipGetLastError() after enqueuing.  dtype: 0 fp32, 1 bf16.  D in {64,128}.
-hipError_t launch_carry(int dtype, int D, const void* Ks, const void* Kd, float* C, int Lp, int Zk, hipStream_t s);
+hipError_t launch_carry(int dtype, int D, const void* Kp, const float* lsrc, const float* ldest, float* C, int Lp, int Zk,
+                        hipStream_t s);
 int fwd_fused_variants(int dtype, int D);
-hipError_t launch_fwd_fused(int dtype, int D, int variant, const void* Qp, const void* Kd, const void* Ks, const void* Kp,
-                            const void* VT, const float* C, void* O, float* lse, float* lse2, int R, int L, int Lp, int d,
-                            int Zq, hipStream_t s);
-hipError_t launch_fwd_chunked(int dtype, int D, const void* Qp, const void* Kd, const void* Ks, const void* Kp,
-                              const void* VT, void* out, void* denom, float* lse2, long o_sz, long o_st, long o_sd,
+hipError_t launch_fwd_fused(int dtype, int D, int variant, const void* Qp, const void* Kp, const void* VT,
+                            const float* lsrc, const float* ldest, const float* C, void* O, float* lse, float* lse2, int R,
+                            int L, int Lp, int d, int Zq, hipStream_t s);
+hipError_t launch_fwd_chunked(int dtype, int D, const void* Qp, const void* Kp, const void* VT, const float* lsrc,
+                              const float* ldest, void* out, void* denom, float* lse2, long o_sz, long o_st, long o_sd,
                               long o_si, int R, int L, int Lp, int d, int c, int nch, int Zk, hipStream_t s);
 hipError_t launch_bwd_keys(int dtype, int D, const BwdArgsV& a, int Zk, hipStream_t s);
 

@@ -21,21 +21,15 @@ __device__ __forceinline__ long rows_offset(const RowsView& v, int z, int row) {
 }
 
 // x (dtype T) -> nat [Z][Lp][D] and/or tr [Z][D][Lp], zero padded (rows >= L, cols >= d).
-// gate (optional, dtype T, one value per row, addressed with z / gate_div): rows are scaled by sqrt(gate).
 template <class T, int D>
-__global__ void __launch_bounds__(256) k_pack(RowsView x, RowsView gate, int gate_div, T* __restrict__ nat,
-                                              T* __restrict__ tr, int d, int L, int Lp) {
+__global__ void __launch_bounds__(256) k_pack(RowsView x, T* __restrict__ nat, T* __restrict__ tr, int d, int L, int Lp) {
   __shared__ float tile[32][D + 1];
   const int z = blockIdx.y, row0 = blockIdx.x * 32, tid = threadIdx.x;
   const T* xp = reinterpret_cast<const T*>(x.p);
-  const T* gp = reinterpret_cast<const T*>(gate.p);
   for (int i = tid; i < 32 * D; i += 256) {
     int rr = i / D, col = i - rr * D, row = row0 + rr;
     float val = 0.f;
-    if (row < L && col < d) {
-      val = (float)xp[rows_offset(x, z, row) + (long)col * x.sc];
-      if (gp) val *= __builtin_sqrtf((float)gp[rows_offset(gate, z / gate_div, row)]);
-    }
+    if (row < L && col < d) val = (float)xp[rows_offset(x, z, row) + (long)col * x.sc];
     tile[rr][col] = val;
     if (nat) nat[((long)z * Lp + row) * D + col] = cvt<T>(val);
   }
@@ -69,6 +63,21 @@ __global__ void __launch_bounds__(256) k_delta(RowsView O, RowsView dO, RowsView
     delta[(long)z * Lp + t] = s;
     if (lse_in.p) lse2[(long)z * Lp + t] = (t < L) ? reinterpret_cast<const float*>(lse_in.p)[rows_offset(lse_in, z, t)] * kLog2e : 0.f;
   }
+}
+
+// log-gates: out[z][t] = log2(gate[z][t]) / 3 for t < L, kGatePad beyond (gate contiguous [Z][L], dtype T)
+template <class T>
+__global__ void __launch_bounds__(256) k_gates(const T* __restrict__ src, const T* __restrict__ dest, float* __restrict__ lsrc,
+                                               float* __restrict__ ldest, int L, int Lp) {
+  const int z = blockIdx.y, t = blockIdx.x * 256 + threadIdx.x;
+  if (t >= Lp) return;
+  float a = kGatePad, b = kGatePad;
+  if (t < L) {
+    a = __builtin_amdgcn_logf((float)src[(long)z * L + t]) * (1.0f / 3.0f);
+    b = __builtin_amdgcn_logf((float)dest[(long)z * L + t]) * (1.0f / 3.0f);
+  }
+  lsrc[(long)z * Lp + t] = a;
+  ldest[(long)z * Lp + t] = b;
 }
 
 // plain fill (kept as a kernel so that callers may capture the sequence in a HIP graph)
