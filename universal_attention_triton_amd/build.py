@@ -9,7 +9,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libua_hip.so")
 UNITS = ["ua_capi", "ua_inst_fwd", "ua_inst_bwd"]
 # packed-fp32 instructions are disabled for every device compile of this library
-FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-honor-nans", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
 def _compile(unit, objdir, extra):

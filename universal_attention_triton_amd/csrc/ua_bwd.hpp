@@ -52,7 +52,7 @@ __global__ void __launch_bounds__(64 * NW) k_bwd_keys(BwdArgs<T> a) {
   T* sdOT = sQT + D * TS;
   T* sX = sdOT + D * TS;                                  // [32 t][SS]  transposed dS / dg staging
   float* sStat = reinterpret_cast<float*>(sX + 32 * SS);  // lse2[32], delta[32]
-  const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, col = lane & 31, hi = lane >> 5;
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 31, hi = lane >> 5;
   const int zk = blockIdx.y, Lp = a.Lp, L = a.L, nT = Lp / 32;
 
   int chunk_i = 0, wg_key0, wg_keys;

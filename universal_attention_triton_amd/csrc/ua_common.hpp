@@ -100,19 +100,37 @@ __device__ __forceinline__ void stage_tile(T* __restrict__ lds, const T* __restr
 }
 
 // ---------------------------------------------------------------------------------
-// lane exchanges
+// lane exchanges (DPP within rows of 16 lanes, v_permlane{16,32}_swap across rows)
 // ---------------------------------------------------------------------------------
 __device__ __forceinline__ float xor_lane(float v, int mask) { return __shfl_xor(v, mask, 64); }
 
+template <int CTRL> __device__ __forceinline__ float dpp(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+constexpr int kDppXor1 = 0xB1, kDppXor2 = 0x4E, kDppRor4 = 0x124, kDppRor8 = 0x128;
+// values of lanes l and l^16 (resp. l^32): one of the two results is the lane's own value, the other its partner's
+// (vector elements are copied to scalars before the bit cast: a bit cast applied to r[1] directly reads r[0])
+__device__ __forceinline__ void swap16(float v, float& a, float& b) {
+  auto r = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned, v), __builtin_bit_cast(unsigned, v), false, false);
+  const unsigned r0 = r[0], r1 = r[1];
+  a = __builtin_bit_cast(float, r0); b = __builtin_bit_cast(float, r1);
+}
+__device__ __forceinline__ void swap32(float v, float& a, float& b) {
+  auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, v), __builtin_bit_cast(unsigned, v), false, false);
+  const unsigned r0 = r[0], r1 = r[1];
+  a = __builtin_bit_cast(float, r0); b = __builtin_bit_cast(float, r1);
+}
+
 // all-reduce over the 32 lanes that share l/32 (i.e. over the 32 keys of a block)
 __device__ __forceinline__ float allmax32(float v) {
-  v = fmaxf(v, xor_lane(v, 1)); v = fmaxf(v, xor_lane(v, 2)); v = fmaxf(v, xor_lane(v, 4));
-  v = fmaxf(v, xor_lane(v, 8)); v = fmaxf(v, xor_lane(v, 16));
-  return v;
+  v = fmaxf(v, dpp<kDppXor1>(v)); v = fmaxf(v, dpp<kDppXor2>(v)); v = fmaxf(v, dpp<kDppRor4>(v)); v = fmaxf(v, dpp<kDppRor8>(v));
+  float a, b; swap16(v, a, b);
+  return fmaxf(a, b);
 }
 __device__ __forceinline__ float allsum32(float v) {
-  v += xor_lane(v, 1); v += xor_lane(v, 2); v += xor_lane(v, 4); v += xor_lane(v, 8); v += xor_lane(v, 16);
-  return v;
+  v += dpp<kDppXor1>(v); v += dpp<kDppXor2>(v); v += dpp<kDppRor4>(v); v += dpp<kDppRor8>(v);
+  float a, b; swap16(v, a, b);
+  return a + b;
 }
 
 // query index inside a 32-block of register v of lane-half hi
@@ -121,41 +139,33 @@ __device__ __forceinline__ constexpr int t_of(int v, int hi) { return 8 * (v >> 
 // Inclusive prefix sum over the 32 queries of a block (per key = per lane pair l, l^32).
 // On return x[v] = sum_{t' <= t(v)} x_in[t'];  returns the block total.
 __device__ __forceinline__ float block_prefix(f32x16& x, int hi) {
-  float gs[4], ps[4];
-#pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    x[4 * g + 1] += x[4 * g]; x[4 * g + 2] += x[4 * g + 1]; x[4 * g + 3] += x[4 * g + 2];
-    gs[g] = x[4 * g + 3];
-  }
-#pragma unroll
-  for (int g = 0; g < 4; ++g) ps[g] = xor_lane(gs[g], 32);
+  const float him = hi ? 1.f : 0.f;
   float run = 0.f;
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
-    float off = run + (hi ? ps[g] : 0.f);
+    x[4 * g + 1] += x[4 * g]; x[4 * g + 2] += x[4 * g + 1]; x[4 * g + 3] += x[4 * g + 2];
+    float lo, up;                       // group sums of the hi=0 lane and of the hi=1 lane of this key
+    swap32(x[4 * g + 3], lo, up);
+    const float off = __builtin_fmaf(him, lo, run);   // the hi=1 piece follows the hi=0 piece
 #pragma unroll
     for (int e = 0; e < 4; ++e) x[4 * g + e] += off;
-    run += gs[g] + ps[g];
+    run += lo + up;
   }
   return run;
 }
 // Inclusive suffix sum: x[v] = sum_{t' >= t(v)} x_in[t'];  returns the block total.
 __device__ __forceinline__ float block_suffix(f32x16& x, int hi) {
-  float gs[4], ps[4];
-#pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    x[4 * g + 2] += x[4 * g + 3]; x[4 * g + 1] += x[4 * g + 2]; x[4 * g] += x[4 * g + 1];
-    gs[g] = x[4 * g];
-  }
-#pragma unroll
-  for (int g = 0; g < 4; ++g) ps[g] = xor_lane(gs[g], 32);
+  const float lom = hi ? 0.f : 1.f;
   float run = 0.f;
 #pragma unroll
   for (int g = 3; g >= 0; --g) {
-    float off = run + (hi ? 0.f : ps[g]);     // the hi=1 piece of group g lies after the hi=0 piece
+    x[4 * g + 2] += x[4 * g + 3]; x[4 * g + 1] += x[4 * g + 2]; x[4 * g] += x[4 * g + 1];
+    float lo, up;
+    swap32(x[4 * g], lo, up);
+    const float off = __builtin_fmaf(lom, up, run);   // the hi=1 piece of group g lies after the hi=0 piece
 #pragma unroll
     for (int e = 0; e < 4; ++e) x[4 * g + e] += off;
-    run += gs[g] + ps[g];
+    run += lo + up;
   }
   return run;
 }

@@ -24,7 +24,7 @@ __global__ void __launch_bounds__(256) k_carry(const T* __restrict__ Kp, const f
   extern __shared__ __align__(16) char smem[];
   T* sKd = reinterpret_cast<T*>(smem);
   constexpr int NQ = D / 16, LS = lds_stride<T>(D);
-  const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, col = lane & 31, hi = lane >> 5;
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 31, hi = lane >> 5;
   const int z = blockIdx.y, nT = Lp / 32, sb = 4 * blockIdx.x + w;
   Frag<T> ks[NQ];
   {
@@ -75,7 +75,7 @@ __global__ void __launch_bounds__(256) k_fwd_fused(const T* __restrict__ Qp, con
   T* sKp = reinterpret_cast<T*>(smem);
   T* sVT = sKp + BS * LS;
   T* sP = sVT + D * PS;
-  const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, col = lane & 31, hi = lane >> 5;
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 31, hi = lane >> 5;
   const int zq = blockIdx.y, zk = zq / R, nT = Lp / 32;
   const int jt = gridDim.x - 1 - blockIdx.x, tb = 4 * jt + w;
   T* sPw = sP + w * 32 * PS;
@@ -207,7 +207,7 @@ __global__ void __launch_bounds__(64 * NW) k_fwd_chunked(const T* __restrict__ Q
   T* sP = sQ + 32 * LS;
   float* sM = reinterpret_cast<float*>(sP + 32 * PS);   // [NW][32]
   float* sMean = sM + NW * 32;                          // [D]
-  const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, col = lane & 31, hi = lane >> 5;
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 31, hi = lane >> 5;
   const int i = blockIdx.x, zk = blockIdx.y;
   const int kbase = i * c + 32 * w;
   const bool valid = (32 * w + col) < c;
