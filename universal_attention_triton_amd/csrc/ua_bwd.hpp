@@ -30,8 +30,9 @@ struct BwdArgs {
   const T *dOp, *dOT;           // [Zq*nch][Lp][D], [Zq*nch][D][Lp]
   const float *lse2, *delta;    // [Zq*nch][Lp]
   const float* C;               // [Zk][Lp/32][Lp]
-  float *dQacc;                 // [Zq][Lp][D]  atomics
-  float *dKdacc;                // [Zk][Lp][D]  atomics
+  float *dQacc;                 // [Zq][Lp][D]  atomics (COLS only)
+  float *dKdacc;                // [Zk][Lp][D]  atomics (COLS) / plain stores of k_bwd_queries
+  float *Dsuf;                  // [Zk][Lp/32][Lp]  suffix carry of dBias entering each query block (!COLS)
   float *dKrow, *dVrow;         // [Zk][Lp][D]
   float* dsrc_raw;              // [Zk][Lp]
   int R, L, Lp, c, nch, chunked, skip_masked;
@@ -39,7 +40,9 @@ struct BwdArgs {
 
 // grid (key groups, Zk).  chunked == 0: key group = 128 consecutive keys, 4 waves.
 // chunked == 1: key group = min(c, 32*NW) keys of ONE chunk (gridDim.x = nch * ceil(c / (32*NW))).
-template <class T, int D, int NW>
+// Chunked mode (COLS = true): also produces the query-side sums (dQ, dkcol) through atomics.  The fused
+// mode uses k_bwd_keys2 / k_bwd_queries2 (ua_fused.hpp) instead.
+template <class T, int D, int NW, bool COLS>
 __global__ void __launch_bounds__(64 * NW) k_bwd_keys(BwdArgs<T> a) {
   extern __shared__ __align__(16) char smem[];
   constexpr int NQ = D / 16, NB = D / 32, LS = lds_stride<T>(D), TS = lds_stride<T>(32), CP = 32 * NW,
@@ -161,16 +164,17 @@ __global__ void __launch_bounds__(64 * NW) k_bwd_keys(BwdArgs<T> a) {
           const Frag<T> bp = as_operand<T>(P, q2), bs = as_operand<T>(dS, q2);
 #pragma unroll
           for (int n = 0; n < NB; ++n) {
-            mma(dVt[n], ld4x2(sdOT + (32 * n + col) * TS + 16 * q2 + 4 * hi), bp);
-            mma(dKt[n], ld4x2(sQT + (32 * n + col) * TS + 16 * q2 + 4 * hi), bs);
+            mma(dVt[n], ld8(sdOT + (32 * n + col) * TS + 16 * q2 + 8 * hi), bp);
+            mma(dKt[n], ld8(sQT + (32 * n + col) * TS + 16 * q2 + 8 * hi), bs);
           }
         }
       } else {
         dS = (f32x16){0};
       }
       // ---- query side: dQ[t,:] += sum_s dS[s,t] k_s   (all keys of the workgroup, then atomics)
+      if constexpr (COLS) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) sX[t_of(v, hi) * SS + 32 * w + col] = cvt<T>(dS[v]);
+      for (int v = 0; v < 16; ++v) sX[t_of(v, hi) * SS + 32 * w + perm16(col)] = cvt<T>(dS[v]);
       __syncthreads();
 #pragma unroll
       for (int nb = 0; nb < NBW; ++nb) {
@@ -188,10 +192,14 @@ __global__ void __launch_bounds__(64 * NW) k_bwd_keys(BwdArgs<T> a) {
             atomicAdd(a.dQacc + (zq * Lp + 32 * tb + t_of(v, hi)) * D + 32 * n + col, acc[v]);
         }
       }
+      }
     }
     // ---- decay part
     f32x16 dg;
     if (mode == 2) {
+      if constexpr (!COLS) {
+        if (valid && hi == 0) a.Dsuf[((long)zk * nT + tb) * Lp + spos] = dcar;
+      }
       const float tot = block_suffix(dB, hi);
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
@@ -210,14 +218,15 @@ __global__ void __launch_bounds__(64 * NW) k_bwd_keys(BwdArgs<T> a) {
       for (int q2 = 0; q2 < 2; ++q2) {
         const Frag<T> b = as_operand<T>(dg, q2);
 #pragma unroll
-        for (int n = 0; n < NB; ++n) mma(dKt[n], ld4x2(sKdT + (32 * n + col) * TS + 16 * q2 + 4 * hi), b);
+        for (int n = 0; n < NB; ++n) mma(dKt[n], ld8(sKdT + (32 * n + col) * TS + 16 * q2 + 8 * hi), b);
       }
     } else {
       dg = (f32x16){0};
     }
+    if constexpr (COLS) {
     __syncthreads();
 #pragma unroll
-    for (int v = 0; v < 16; ++v) sX[t_of(v, hi) * SS + 32 * w + col] = cvt<T>(dg[v]);
+    for (int v = 0; v < 16; ++v) sX[t_of(v, hi) * SS + 32 * w + perm16(col)] = cvt<T>(dg[v]);
     __syncthreads();
     if (tb >= wg_key0 / 32) {
 #pragma unroll
@@ -236,6 +245,7 @@ __global__ void __launch_bounds__(64 * NW) k_bwd_keys(BwdArgs<T> a) {
             atomicAdd(a.dKdacc + ((long)zk * Lp + 32 * tb + t_of(v, hi)) * D + 32 * n + col, acc[v]);
         }
       }
+    }
     }
   }
   // ---- epilogue: key-side results
@@ -268,7 +278,7 @@ __global__ void __launch_bounds__(256) k_bwd_finish(const float* __restrict__ dK
   const int z = blockIdx.y, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + wave;
   if (t >= L) return;
-  if (z < Zq) {
+  if (z < Zq && dQacc) {
     for (int c = lane; c < d; c += 64) dq[((long)z * L + t) * d + c] = cvt<T>(dQacc[((long)z * Lp + t) * D + c]);
   }
   if (z < Zk) {

@@ -36,7 +36,7 @@ struct Layout {
   // forward state
   size_t Kp, KT, Vp, VT, Qp, QT, lsrc, ldest, C, lse2, fwd_end;
   // backward scratch
-  size_t dOp, dOT, delta, dQacc, dKdacc, dKrow, dVrow, dsrc_raw, total;
+  size_t dOp, dOT, delta, dQacc, dKdacc, Dsuf, dKrow, dVrow, dsrc_raw, total;
 };
 
 int check_desc(const ua_desc* d, bool chunked) {
@@ -75,8 +75,9 @@ Layout make_layout(const ua_desc& d, bool chunked) {
   const size_t gbytes = (size_t)l.Zq * l.nch * l.Lp * l.D * l.esz;
   l.dOp = take(gbytes); l.dOT = take(gbytes);
   l.delta = take((size_t)l.Zq * l.nch * l.Lp * 4);
-  l.dQacc = take((size_t)l.Zq * l.Lp * l.D * 4);
+  l.dQacc = chunked ? take((size_t)l.Zq * l.Lp * l.D * 4) : 0;     // atomics target of the chunked mode only
   l.dKdacc = take((size_t)l.Zk * l.Lp * l.D * 4);
+  l.Dsuf = chunked ? 0 : take((size_t)l.Zk * l.nT * l.Lp * 4);
   l.dKrow = take((size_t)l.Zk * l.Lp * l.D * 4);
   l.dVrow = take((size_t)l.Zk * l.Lp * l.D * 4);
   l.dsrc_raw = take((size_t)l.Zk * l.Lp * 4);
@@ -214,11 +215,11 @@ int run_fused_fwd_kernels(const ua_desc& d, const Layout& l, char* ws, void* O, 
 }
 
 template <class T>
-hipError_t finish_t(const Layout& l, const ua_desc& d, char* ws, const void* src, const void* dest, void* dk, void* dv,
-                    void* dq, void* dsrc, void* ddest, hipStream_t s) {
+hipError_t finish_t(const Layout& l, const ua_desc& d, char* ws, bool chunked, const void* src, const void* dest, void* dk,
+                    void* dv, void* dq, void* dsrc, void* ddest, hipStream_t s) {
   const int Z = l.Zq > l.Zk ? l.Zq : l.Zk;
   hipLaunchKernelGGL((ua::k_bwd_finish<T>), dim3((d.L + 3) / 4, Z), dim3(256), 0, s, (const float*)(ws + l.dKrow),
-                     (const float*)(ws + l.dVrow), (const float*)(ws + l.dKdacc), (const float*)(ws + l.dQacc),
+                     (const float*)(ws + l.dVrow), (const float*)(ws + l.dKdacc), chunked ? (const float*)(ws + l.dQacc) : nullptr,
                      (const float*)(ws + l.dsrc_raw), (const T*)(ws + l.Kp), (const T*)src, (const T*)dest, (T*)dk, (T*)dv,
                      (T*)dq, (T*)dsrc, (T*)ddest, l.Zk, l.Zq, d.L, l.Lp, l.D, d.d);
   return hipGetLastError();
@@ -233,7 +234,7 @@ hipError_t delta_t(const ua::RowsView& O, const ua::RowsView& dO, const ua::Rows
 
 int run_bwd_common(const ua_desc& d, const Layout& l, char* ws, bool chunked, const void* src, const void* dest, void* dkc,
                    void* dvc, void* dxq, void* dsrc, void* ddest, hipStream_t s) {
-  {
+  if (chunked) {
     UA_PROF("k_zero", s);
     UA_HIP(zero_fill(ws + l.dQacc, (size_t)l.Zq * l.Lp * l.D * 4, s));
     UA_HIP(zero_fill(ws + l.dKdacc, (size_t)l.Zk * l.Lp * l.D * 4, s));
@@ -242,17 +243,22 @@ int run_bwd_common(const ua_desc& d, const Layout& l, char* ws, bool chunked, co
   a.Kp = ws + l.Kp; a.Vp = ws + l.Vp; a.KT = ws + l.KT; a.Qp = ws + l.Qp; a.QT = ws + l.QT; a.dOp = ws + l.dOp;
   a.dOT = ws + l.dOT; a.lsrc = (const float*)(ws + l.lsrc); a.ldest = (const float*)(ws + l.ldest);
   a.lse2 = (const float*)(ws + l.lse2); a.delta = (const float*)(ws + l.delta); a.C = (const float*)(ws + l.C);
-  a.dQacc = (float*)(ws + l.dQacc); a.dKdacc = (float*)(ws + l.dKdacc); a.dKrow = (float*)(ws + l.dKrow);
+  a.dQacc = (float*)(ws + l.dQacc); a.dKdacc = (float*)(ws + l.dKdacc); a.Dsuf = (float*)(ws + l.Dsuf);
+  a.dKrow = (float*)(ws + l.dKrow);
   a.dVrow = (float*)(ws + l.dVrow); a.dsrc_raw = (float*)(ws + l.dsrc_raw);
   a.R = d.r; a.L = d.L; a.Lp = l.Lp; a.c = chunked ? d.chunk : 128; a.nch = l.nch; a.chunked = chunked ? 1 : 0;
   a.skip_masked = (d.flags & UA_FLAG_SKIP_MASKED) ? 1 : 0;
   {
     UA_PROF("k_bwd_keys", s);
-    UA_HIP(ua::launch_bwd_keys(d.dtype, l.D, a, l.Zk, s));
+    UA_HIP(ua::launch_bwd_keys(d.dtype, l.D, a, l.Zk, chunked ? 1 : 0, s));
+  }
+  if (!chunked) {
+    UA_PROF("k_bwd_queries", s);
+    UA_HIP(ua::launch_bwd_queries(d.dtype, l.D, a, dxq, d.d, l.Zk, s));
   }
   UA_PROF("k_bwd_finish", s);
-  if (d.dtype == UA_BF16) UA_HIP(finish_t<ua::bf16>(l, d, ws, src, dest, dkc, dvc, dxq, dsrc, ddest, s));
-  else UA_HIP(finish_t<float>(l, d, ws, src, dest, dkc, dvc, dxq, dsrc, ddest, s));
+  if (d.dtype == UA_BF16) UA_HIP(finish_t<ua::bf16>(l, d, ws, chunked, src, dest, dkc, dvc, dxq, dsrc, ddest, s));
+  else UA_HIP(finish_t<float>(l, d, ws, chunked, src, dest, dkc, dvc, dxq, dsrc, ddest, s));
   return UA_OK;
 }
 

@@ -100,6 +100,54 @@ __device__ __forceinline__ void stage_tile(T* __restrict__ lds, const T* __restr
 }
 
 // ---------------------------------------------------------------------------------
+// Asynchronous tile staging: global_load_lds_dwordx4 moves 16 bytes per lane from an arbitrary
+// global address straight into LDS at (wave-uniform base + 16*lane), without passing through
+// registers.  A padded LDS tile is therefore filled by NINSTR instructions of 1 KB each; the
+// lanes that fall on padding slots re-read a payload chunk.  Each wave issues instructions
+// w, w+NWAVES, ... and keeps the per-lane source offsets of its instructions in registers.
+// ---------------------------------------------------------------------------------
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+template <class T, int ROWS, int COLS> struct Tile {
+  static constexpr int STRIDE = COLS + kPad16 / (int)sizeof(T);        // elements per padded row
+  static constexpr int CPR = STRIDE * (int)sizeof(T) / 16;             // 16-byte chunks per padded row
+  static constexpr int CPP = COLS * (int)sizeof(T) / 16;               // payload chunks per row
+  static constexpr int NINSTR = (ROWS * CPR + 63) / 64;
+  static constexpr int BYTES = NINSTR * 1024;                          // LDS footprint
+};
+
+template <class TILE, int NWAVES> struct Stager {
+  static constexpr int PER = (TILE::NINSTR + NWAVES - 1) / NWAVES;
+  int off[PER];
+  // gstride_bytes: distance between consecutive rows of the tile in global memory
+  __device__ __forceinline__ void init(int w, int lane, long gstride_bytes, int rows) {
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int n = (w + k * NWAVES) * 64 + lane;
+      int row = n / TILE::CPR, c = n - row * TILE::CPR;
+      row = row < rows ? row : rows - 1;
+      c = c < TILE::CPP ? c : TILE::CPP - 1;
+      off[k] = (int)(row * gstride_bytes) + c * 16;
+    }
+  }
+  __device__ __forceinline__ void issue(void* lds_tile, const void* gtile, int w) const {
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int i = w + k * NWAVES;
+      if (i < TILE::NINSTR)
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const char*>(gtile) + off[k],
+                                         (lds_ptr_t)(reinterpret_cast<char*>(lds_tile) + i * 1024), 16, 0, 0);
+    }
+  }
+};
+__device__ __forceinline__ void wait_async_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// Column order of the transposed ([feature][position]) working tensors: inside every group of 16
+// positions bits 2 and 3 are swapped, so that the 8 k-values a lane needs for the permuted-t operand
+// (t = 16q + 8(e/4) + 4hi + e%4) are 8 CONSECUTIVE elements starting at 16q + 8hi.
+__host__ __device__ __forceinline__ constexpr int perm16(int t) { return (t & ~12) | ((t & 4) << 1) | ((t & 8) >> 1); }
+
+// ---------------------------------------------------------------------------------
 // lane exchanges (DPP within rows of 16 lanes, v_permlane{16,32}_swap across rows)
 // ---------------------------------------------------------------------------------
 __device__ __forceinline__ float xor_lane(float v, int mask) { return __shfl_xor(v, mask, 64); }

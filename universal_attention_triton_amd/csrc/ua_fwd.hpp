@@ -1,8 +1,4 @@
-// Forward kernels.
-//   k_carry        key-stationary pre-pass: per key s and per 32-query block tb the decay bias
-//                  accumulated over all queries before the block (log2 units).
-//   k_fwd_fused    query-stationary fused kernel: bias rebuilt per tile from the carries,
-//                  online softmax across key tiles, O and log-sum-exp written once.
+// Chunked forward kernel.
 //   k_fwd_chunked  key-chunk-stationary kernel producing the per-chunk partial outputs and
 //                  normalisers of the reference operator (universal_attention_autograd.py:9-38).
 #pragma once
@@ -13,176 +9,6 @@ namespace ua {
 // marker stored in the log2-unit normaliser buffer for a (query, chunk) pair with no visible key
 constexpr float kLseMasked = 3.0e38f;
 constexpr float kNegBig = -1.0e30f;
-
-// ---------------------------------------------------------------------------------------------
-// C[z][tb][s] = sum_{u < 32*tb, u > s} log2(1 - A[s,u])      for tb >= s/32
-// grid (Lp/128, Z_kv); 4 waves, wave w owns keys 32*(4*bx+w) .. +31 and sweeps query blocks.
-// ---------------------------------------------------------------------------------------------
-template <class T, int D>
-__global__ void __launch_bounds__(256) k_carry(const T* __restrict__ Kp, const float* __restrict__ lsrc,
-                                               const float* __restrict__ ldest, float* __restrict__ C, int Lp) {
-  extern __shared__ __align__(16) char smem[];
-  T* sKd = reinterpret_cast<T*>(smem);
-  constexpr int NQ = D / 16, LS = lds_stride<T>(D);
-  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 31, hi = lane >> 5;
-  const int z = blockIdx.y, nT = Lp / 32, sb = 4 * blockIdx.x + w;
-  Frag<T> ks[NQ];
-  {
-    const T* krow = Kp + ((long)z * Lp + 32 * sb + col) * D + 8 * hi;
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) ks[q] = ld8(krow + 16 * q);
-  }
-  const float la = lsrc[(long)z * Lp + 32 * sb + col];
-  float carry = 0.f;
-  float* Cz = C + (long)z * nT * Lp;
-  for (int tb = 4 * blockIdx.x; tb < nT; ++tb) {
-    __syncthreads();
-    stage_tile(sKd, Kp + ((long)z * Lp + 32 * tb) * D, 32, D, D, LS, tid, 256);
-    __syncthreads();
-    if (tb >= sb) {
-      f32x16 g = {0};
-#pragma unroll
-      for (int q = 0; q < NQ; ++q) mma(g, ld8(sKd + col * LS + 16 * q + 8 * hi), ks[q]);
-      float lb[16];
-      load_t16(ldest + (long)z * Lp + 32 * tb, hi, lb);
-      float tot = 0.f;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        float l2 = log2_one_minus(affinity(log2_relu(g[v]), la + lb[v]));
-        if (tb == sb && t_of(v, hi) <= col) l2 = 0.f;
-        tot += l2;
-      }
-      tot += xor_lane(tot, 32);
-      if (hi == 0) Cz[(long)tb * Lp + 32 * sb + col] = carry;
-      carry += tot;
-    }
-  }
-}
-
-// ---------------------------------------------------------------------------------------------
-// Fused forward.  grid (Lp/128, Z_q) ; 4 waves ; wave w owns queries 32*(4*jt+w) .. +31.
-// Per key tile of BS keys: G = K_t.K_s -> A -> log2(1-A) -> in-lane prefix + carry = bias,
-// S = Q_t.K_s, online softmax over keys, P^T through LDS, O += P^T V.
-// ---------------------------------------------------------------------------------------------
-template <class T, int D, int BS>
-__global__ void __launch_bounds__(256) k_fwd_fused(const T* __restrict__ Qp, const T* __restrict__ Kp,
-                                                   const T* __restrict__ VT, const float* __restrict__ lsrc,
-                                                   const float* __restrict__ ldest, const float* __restrict__ C,
-                                                   T* __restrict__ O, float* __restrict__ lse, float* __restrict__ lse2,
-                                                   int R, int L, int Lp, int d) {
-  extern __shared__ __align__(16) char smem[];
-  constexpr int NQ = D / 16, NB = D / 32, NSB = BS / 32, LS = lds_stride<T>(D), PS = lds_stride<T>(BS);
-  T* sKp = reinterpret_cast<T*>(smem);
-  T* sVT = sKp + BS * LS;
-  T* sP = sVT + D * PS;
-  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 31, hi = lane >> 5;
-  const int zq = blockIdx.y, zk = zq / R, nT = Lp / 32;
-  const int jt = gridDim.x - 1 - blockIdx.x, tb = 4 * jt + w;
-  T* sPw = sP + w * 32 * PS;
-
-  Frag<T> qf[NQ], kdf[NQ];
-  {
-    const T* qrow = Qp + ((long)zq * Lp + 32 * tb + col) * D + 8 * hi;
-    const T* krow = Kp + ((long)zk * Lp + 32 * tb + col) * D + 8 * hi;
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) { qf[q] = ld8(qrow + 16 * q); kdf[q] = ld8(krow + 16 * q); }
-  }
-  float lb[16];
-  load_t16(ldest + (long)zk * Lp + 32 * tb, hi, lb);
-  f32x16 o[NB];
-#pragma unroll
-  for (int n = 0; n < NB; ++n) o[n] = (f32x16){0};
-  float m[16], ls[16];
-#pragma unroll
-  for (int v = 0; v < 16; ++v) { m[v] = kNegBig; ls[v] = 0.f; }
-  const float* Crow = C + ((long)zk * nT + tb) * Lp;
-
-  const int n_kt = (128 * jt + 128) / BS;
-  for (int kt = 0; kt < n_kt; ++kt) {
-    __syncthreads();
-    stage_tile(sKp, Kp + ((long)zk * Lp + BS * kt) * D, BS, D, D, LS, tid, 256);
-    stage_tile(sVT, VT + (long)zk * D * Lp + BS * kt, D, BS, Lp, PS, tid, 256);
-    __syncthreads();
-    f32x16 s2[NSB];
-#pragma unroll
-    for (int j = 0; j < NSB; ++j) {
-      const int sbk = NSB * kt + j;
-      if (sbk <= tb) {
-        f32x16 g = {0};
-#pragma unroll
-        for (int q = 0; q < NQ; ++q) mma(g, kdf[q], ld8(sKp + (32 * j + col) * LS + 16 * q + 8 * hi));
-        const bool diag = (sbk == tb);
-        const float la = lsrc[(long)zk * Lp + 32 * sbk + col];
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          float l2 = log2_one_minus(affinity(log2_relu(g[v]), la + lb[v]));
-          g[v] = (diag && t_of(v, hi) <= col) ? 0.f : l2;
-        }
-        block_prefix(g, hi);
-        const float c = Crow[32 * sbk + col];
-        f32x16 sc = {0};
-#pragma unroll
-        for (int q = 0; q < NQ; ++q) mma(sc, qf[q], ld8(sKp + (32 * j + col) * LS + 16 * q + 8 * hi));
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          float x = __builtin_fmaf(sc[v], kLog2e, g[v] + c);
-          s2[j][v] = (diag && t_of(v, hi) < col) ? kNegBig : x;
-        }
-      } else {
-#pragma unroll
-        for (int v = 0; v < 16; ++v) s2[j][v] = kNegBig;
-      }
-    }
-    // online softmax over this tile's keys
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      float mx = s2[0][v];
-#pragma unroll
-      for (int j = 1; j < NSB; ++j) mx = fmaxf(mx, s2[j][v]);
-      mx = allmax32(mx);
-      const float mn = fmaxf(m[v], mx);
-      const float alpha = __builtin_amdgcn_exp2f(m[v] - mn);
-      m[v] = mn;
-      ls[v] *= alpha;
-#pragma unroll
-      for (int n = 0; n < NB; ++n) o[n][v] *= alpha;
-#pragma unroll
-      for (int j = 0; j < NSB; ++j) {
-        float p = __builtin_amdgcn_exp2f(s2[j][v] - mn);
-        ls[v] += p;
-        sPw[t_of(v, hi) * PS + 32 * j + col] = cvt<T>(p);
-      }
-    }
-    __syncthreads();
-#pragma unroll
-    for (int kq = 0; kq < BS / 16; ++kq) {
-      if (NSB * kt + kq / 2 <= tb) {
-        Frag<T> a = ld8(sPw + col * PS + 16 * kq + 8 * hi);
-#pragma unroll
-        for (int n = 0; n < NB; ++n) mma(o[n], a, ld8(sVT + (32 * n + col) * PS + 16 * kq + 8 * hi));
-      }
-    }
-  }
-  // epilogue
-#pragma unroll
-  for (int v = 0; v < 16; ++v) {
-    const float tot = allsum32(ls[v]);
-    const float inv = 1.0f / tot;
-    const int t = 32 * tb + t_of(v, hi);
-    if (t < L) {
-#pragma unroll
-      for (int n = 0; n < NB; ++n) {
-        const int dd = 32 * n + col;
-        if (dd < d) O[((long)zq * L + t) * d + dd] = cvt<T>(o[n][v] * inv);
-      }
-    }
-    if (col == 0) {
-      const float l2v = m[v] + __builtin_amdgcn_logf(tot);
-      lse2[(long)zq * Lp + t] = (t < L) ? l2v : 0.f;
-      if (t < L) lse[(long)zq * L + t] = l2v * kLn2;
-    }
-  }
-}
 
 // ---------------------------------------------------------------------------------------------
 // Chunked forward (reference operator semantics).  grid (n_chunks, Z_kv); NW = ceil(c/32) waves.
@@ -319,7 +145,7 @@ __global__ void __launch_bounds__(64 * NW) k_fwd_chunked(const T* __restrict__ Q
 #pragma unroll
         for (int ww = 1; ww < NW; ++ww) mm = fmaxf(mm, sM[ww * 32 + t_of(v, hi)]);
         m[v] = mm;
-        sP[t_of(v, hi) * PS + 32 * w + col] = cvt<T>(__builtin_amdgcn_exp2f(s2[v] - mm));
+        sP[t_of(v, hi) * PS + 32 * w + perm16(col)] = cvt<T>(__builtin_amdgcn_exp2f(s2[v] - mm));
       }
       __syncthreads();
       f32x16 osum = {0};

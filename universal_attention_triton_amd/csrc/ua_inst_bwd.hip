@@ -1,33 +1,67 @@
 // Instantiations and launcher of the key-stationary backward kernel.
 #include "ua_bwd.hpp"
+#include "ua_fused.hpp"
 #include "ua_internal.hpp"
 
 namespace ua {
 
-template <class T, int D, int NW>
-static hipError_t bwd_t(const BwdArgsV& v, int Zk, hipStream_t s) {
+template <class T>
+static BwdArgs<T> typed(const BwdArgsV& v) {
   BwdArgs<T> a;
   a.Kp = (const T*)v.Kp; a.Vp = (const T*)v.Vp; a.KT = (const T*)v.KT; a.Qp = (const T*)v.Qp; a.QT = (const T*)v.QT;
   a.dOp = (const T*)v.dOp; a.dOT = (const T*)v.dOT; a.lsrc = v.lsrc; a.ldest = v.ldest; a.lse2 = v.lse2; a.delta = v.delta;
   a.C = v.C;
-  a.dQacc = v.dQacc; a.dKdacc = v.dKdacc; a.dKrow = v.dKrow; a.dVrow = v.dVrow; a.dsrc_raw = v.dsrc_raw;
+  a.dQacc = v.dQacc; a.dKdacc = v.dKdacc; a.Dsuf = v.Dsuf; a.dKrow = v.dKrow; a.dVrow = v.dVrow; a.dsrc_raw = v.dsrc_raw;
   a.R = v.R; a.L = v.L; a.Lp = v.Lp; a.c = v.c; a.nch = v.nch; a.chunked = v.chunked; a.skip_masked = v.skip_masked;
+  return a;
+}
+
+template <class T, int D, int NW, bool COLS>
+static hipError_t bwd_t(const BwdArgsV& v, int Zk, hipStream_t s) {
+  const BwdArgs<T> a = typed<T>(v);
   constexpr int CP = 32 * NW;
   const size_t lds = (3 * 32 * lds_stride<T>(D) + 3 * D * lds_stride<T>(32) + 32 * lds_stride<T>(CP)) * sizeof(T) + 64 * sizeof(float);
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k_bwd_keys<T, D, NW>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k_bwd_keys<T, D, NW, COLS>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   const int groups = v.chunked ? v.nch * ((v.c + CP - 1) / CP) : v.Lp / CP;
-  hipLaunchKernelGGL((k_bwd_keys<T, D, NW>), dim3(groups, Zk), dim3(64 * NW), lds, s, a);
+  hipLaunchKernelGGL((k_bwd_keys<T, D, NW, COLS>), dim3(groups, Zk), dim3(64 * NW), lds, s, a);
+  return hipGetLastError();
+}
+template <class T, int D, int NST>
+static hipError_t bwd2_t(const BwdArgsV& v, int Zk, hipStream_t s) {
+  const BwdArgs<T> a = typed<T>(v);
+  const size_t lds = NST * (3 * Tile<T, 32, D>::BYTES + 3 * Tile<T, D, 32>::BYTES + 1024);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k_bwd_keys2<T, D, NST>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  hipLaunchKernelGGL((k_bwd_keys2<T, D, NST>), dim3(v.Lp / 128, Zk), dim3(256), lds, s, a);
   return hipGetLastError();
 }
 template <class T, int D>
-static hipError_t bwd_nw(const BwdArgsV& v, int Zk, hipStream_t s) {
-  if (!v.chunked || v.c >= 128) return bwd_t<T, D, 4>(v, Zk, s);
-  if (v.c > 32) return bwd_t<T, D, 2>(v, Zk, s);
-  return bwd_t<T, D, 1>(v, Zk, s);
+static hipError_t bwd_nw(const BwdArgsV& v, int Zk, int cols, hipStream_t s) {
+  if (!cols) return bwd2_t<T, D, (sizeof(T) == 2 ? 2 : 1)>(v, Zk, s);
+  if (!v.chunked || v.c >= 128) return bwd_t<T, D, 4, true>(v, Zk, s);
+  if (v.c > 32) return bwd_t<T, D, 2, true>(v, Zk, s);
+  return bwd_t<T, D, 1, true>(v, Zk, s);
 }
-hipError_t launch_bwd_keys(int dtype, int D, const BwdArgsV& a, int Zk, hipStream_t s) {
-  if (dtype == 1) return D == 64 ? bwd_nw<bf16, 64>(a, Zk, s) : bwd_nw<bf16, 128>(a, Zk, s);
-  return D == 64 ? bwd_nw<float, 64>(a, Zk, s) : bwd_nw<float, 128>(a, Zk, s);
+hipError_t launch_bwd_keys(int dtype, int D, const BwdArgsV& a, int Zk, int cols, hipStream_t s) {
+  if (dtype == 1) return D == 64 ? bwd_nw<bf16, 64>(a, Zk, cols, s) : bwd_nw<bf16, 128>(a, Zk, cols, s);
+  return D == 64 ? bwd_nw<float, 64>(a, Zk, cols, s) : bwd_nw<float, 128>(a, Zk, cols, s);
+}
+
+// explicit instantiations (the implicit ones are not emitted on the host side for this kernel)
+#define UA_INST(T, D, NST) template __global__ void k_bwd_queries2<T, D, NST>(BwdArgs<T>, T*, int);
+UA_INST(bf16, 64, 2) UA_INST(bf16, 128, 2) UA_INST(float, 64, 1) UA_INST(float, 128, 1)
+#undef UA_INST
+
+template <class T, int D, int NST>
+static hipError_t bwdq_t(const BwdArgsV& v, void* dq, int d, int Zk, hipStream_t s) {
+  const BwdArgs<T> a = typed<T>(v);
+  const size_t lds = NST * (4 * Tile<T, 32, D>::BYTES + 2 * Tile<T, D, 32>::BYTES + 4096) + 4 * 2 * 32 * lds_stride<T>(32) * sizeof(T);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k_bwd_queries2<T, D, NST>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  hipLaunchKernelGGL((k_bwd_queries2<T, D, NST>), dim3(v.Lp / 128, Zk), dim3(256), lds, s, a, (T*)dq, d);
+  return hipGetLastError();
+}
+hipError_t launch_bwd_queries(int dtype, int D, const BwdArgsV& a, void* dq, int d, int Zk, hipStream_t s) {
+  if (dtype == 1) return D == 64 ? bwdq_t<bf16, 64, 2>(a, dq, d, Zk, s) : bwdq_t<bf16, 128, 2>(a, dq, d, Zk, s);
+  return D == 64 ? bwdq_t<float, 64, 1>(a, dq, d, Zk, s) : bwdq_t<float, 128, 1>(a, dq, d, Zk, s);
 }
 
 }  // namespace ua

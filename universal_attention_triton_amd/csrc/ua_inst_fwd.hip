@@ -1,4 +1,5 @@
 // Instantiations and launchers of the forward kernels.
+#include "ua_fused.hpp"
 #include "ua_fwd.hpp"
 #include "ua_internal.hpp"
 
@@ -11,8 +12,10 @@ static void allow_lds(K kernel, size_t bytes) {
 
 template <class T, int D>
 static hipError_t carry_t(const void* Kp, const float* lsrc, const float* ldest, float* C, int Lp, int Zk, hipStream_t s) {
-  const size_t lds = 32 * lds_stride<T>(D) * sizeof(T);
-  hipLaunchKernelGGL((k_carry<T, D>), dim3(Lp / 128, Zk), dim3(256), lds, s, (const T*)Kp, lsrc, ldest, C, Lp);
+  constexpr int NST = 2;
+  const size_t lds = NST * (Tile<T, 32, D>::BYTES + 1024);
+  allow_lds(k_carry2<T, D, NST>, lds);
+  hipLaunchKernelGGL((k_carry2<T, D, NST>), dim3(Lp / 128, Zk), dim3(256), lds, s, (const T*)Kp, lsrc, ldest, C, Lp);
   return hipGetLastError();
 }
 hipError_t launch_carry(int dtype, int D, const void* Kp, const float* lsrc, const float* ldest, float* C, int Lp, int Zk,
@@ -21,26 +24,33 @@ hipError_t launch_carry(int dtype, int D, const void* Kp, const float* lsrc, con
   return D == 64 ? carry_t<float, 64>(Kp, lsrc, ldest, C, Lp, Zk, s) : carry_t<float, 128>(Kp, lsrc, ldest, C, Lp, Zk, s);
 }
 
-template <class T, int D, int BS>
+// explicit instantiations (the implicit ones are not emitted on the host side for these kernels)
+#define UA_INST(T, D, NST)                                                                                            \
+  template __global__ void k_fwd_fused2<T, D, NST>(const T*, const T*, const T*, const float*, const float*, const float*, \
+                                                   T*, float*, float*, int, int, int, int);
+UA_INST(bf16, 64, 1) UA_INST(bf16, 64, 2) UA_INST(bf16, 128, 1) UA_INST(bf16, 128, 2) UA_INST(float, 64, 1) UA_INST(float, 128, 1)
+#undef UA_INST
+
+template <class T, int D, int NST>
 static hipError_t fused_t(const void* Qp, const void* Kp, const void* VT, const float* lsrc, const float* ldest,
                           const float* C, void* O, float* lse, float* lse2, int R, int L, int Lp, int d, int Zq, hipStream_t s) {
-  const size_t lds = (BS * lds_stride<T>(D) + D * lds_stride<T>(BS) + 4 * 32 * lds_stride<T>(BS)) * sizeof(T);
-  allow_lds(k_fwd_fused<T, D, BS>, lds);
-  hipLaunchKernelGGL((k_fwd_fused<T, D, BS>), dim3(Lp / 128, Zq), dim3(256), lds, s, (const T*)Qp, (const T*)Kp,
+  const size_t lds = NST * (2 * Tile<T, 32, D>::BYTES + 2 * Tile<T, D, 32>::BYTES + 4096) + 4 * 32 * lds_stride<T>(64) * sizeof(T);
+  allow_lds(k_fwd_fused2<T, D, NST>, lds);
+  hipLaunchKernelGGL((k_fwd_fused2<T, D, NST>), dim3(Lp / 128, Zq), dim3(256), lds, s, (const T*)Qp, (const T*)Kp,
                      (const T*)VT, lsrc, ldest, C, (T*)O, lse, lse2, R, L, Lp, d);
   return hipGetLastError();
 }
-// variants: key-tile size per LDS stage
+// variants: 0 = double-buffered LDS stages, 1 = single stage (bf16 only; fp32 always runs single stage)
 int fwd_fused_variants(int dtype, int D) { (void)D; return dtype == 1 ? 2 : 1; }
 hipError_t launch_fwd_fused(int dtype, int D, int variant, const void* Qp, const void* Kp, const void* VT,
                             const float* lsrc, const float* ldest, const float* C, void* O, float* lse, float* lse2, int R,
                             int L, int Lp, int d, int Zq, hipStream_t s) {
 #define UA_ARGS Qp, Kp, VT, lsrc, ldest, C, O, lse, lse2, R, L, Lp, d, Zq, s
   if (dtype == 1) {
-    if (D == 64) return variant == 1 ? fused_t<bf16, 64, 128>(UA_ARGS) : fused_t<bf16, 64, 64>(UA_ARGS);
-    return variant == 1 ? fused_t<bf16, 128, 128>(UA_ARGS) : fused_t<bf16, 128, 64>(UA_ARGS);
+    if (D == 64) return variant == 1 ? fused_t<bf16, 64, 1>(UA_ARGS) : fused_t<bf16, 64, 2>(UA_ARGS);
+    return variant == 1 ? fused_t<bf16, 128, 1>(UA_ARGS) : fused_t<bf16, 128, 2>(UA_ARGS);
   }
-  return D == 64 ? fused_t<float, 64, 32>(UA_ARGS) : fused_t<float, 128, 32>(UA_ARGS);
+  return D == 64 ? fused_t<float, 64, 1>(UA_ARGS) : fused_t<float, 128, 1>(UA_ARGS);
 #undef UA_ARGS
 }
 

@@ -10,7 +10,7 @@ namespace ua {
 struct BwdArgsV {
   const void *Kp, *Vp, *KT, *Qp, *QT, *dOp, *dOT;
   const float *lsrc, *ldest, *lse2, *delta, *C;
-  float *dQacc, *dKdacc, *dKrow, *dVrow, *dsrc_raw;
+  float *dQacc, *dKdacc, *Dsuf, *dKrow, *dVrow, *dsrc_raw;
   int R, L, Lp, c, nch, chunked, skip_masked;
 };
 
@@ -24,6 +24,9 @@ hipError_t launch_fwd_fused(int dtype, int D, int variant, const void* Qp, const
 hipError_t launch_fwd_chunked(int dtype, int D, const void* Qp, const void* Kp, const void* VT, const float* lsrc,
                               const float* ldest, void* out, void* denom, float* lse2, long o_sz, long o_st, long o_sd,
                               long o_si, int R, int L, int Lp, int d, int c, int nch, int Zk, hipStream_t s);
-hipError_t launch_bwd_keys(int dtype, int D, const BwdArgsV& a, int Zk, hipStream_t s);
+// cols != 0: the kernel also produces dQ / dkcol through atomics (chunked mode); cols == 0: it records the
+// suffix carries and launch_bwd_queries finishes the query side.
+hipError_t launch_bwd_keys(int dtype, int D, const BwdArgsV& a, int Zk, int cols, hipStream_t s);
+hipError_t launch_bwd_queries(int dtype, int D, const BwdArgsV& a, void* dq, int d, int Zk, hipStream_t s);
 
 }  // namespace ua

@@ -21,6 +21,7 @@ __device__ __forceinline__ long rows_offset(const RowsView& v, int z, int row) {
 }
 
 // x (dtype T) -> nat [Z][Lp][D] and/or tr [Z][D][Lp], zero padded (rows >= L, cols >= d).
+// tr stores position t at column perm16(t).
 template <class T, int D>
 __global__ void __launch_bounds__(256) k_pack(RowsView x, T* __restrict__ nat, T* __restrict__ tr, int d, int L, int Lp) {
   __shared__ float tile[32][D + 1];
@@ -37,7 +38,7 @@ __global__ void __launch_bounds__(256) k_pack(RowsView x, T* __restrict__ nat, T
   __syncthreads();
   for (int i = tid; i < 32 * D; i += 256) {
     int dd = i >> 5, rr = i & 31;
-    tr[((long)z * D + dd) * Lp + row0 + rr] = cvt<T>(tile[rr][dd]);
+    tr[((long)z * D + dd) * Lp + row0 + rr] = cvt<T>(tile[perm16(rr)][dd]);
   }
 }
 
