@@ -21,6 +21,27 @@ __device__ __forceinline__ void issue_row(void* lds_base, const void* src_lane) 
 }
 
 // generic pipeline skeleton:  ISSUE(step, stage_base)  COMPUTE(step, stage_base)
+// UA_PIPE_RANGE runs steps [S0, S1) of a pipeline of NSTEPS steps whose step S0 has already been issued
+// (by UA_PIPE_START or by the previous range), so that consecutive ranges may use different COMPUTE bodies.
+#define UA_PIPE_START(NSTEPS, ISSUE)                                                       \
+  do {                                                                                     \
+    if ((NSTEPS) > 0) ISSUE(0, smem);                                                      \
+  } while (0)
+#define UA_PIPE_RANGE(S0, S1, NSTEPS, STAGE_BYTES, ISSUE, COMPUTE)                         \
+  do {                                                                                     \
+    const int nsteps_ = (NSTEPS), s1_ = (S1);                                              \
+    for (int step_ = (S0); step_ < s1_; ++step_) {                                         \
+      wait_async_loads();                                                                  \
+      __syncthreads();                                                                     \
+      char* cur_ = smem + (NST == 2 ? (step_ & 1) * (STAGE_BYTES) : 0);                    \
+      if (NST == 2 && step_ + 1 < nsteps_) ISSUE(step_ + 1, smem + ((step_ + 1) & 1) * (STAGE_BYTES)); \
+      COMPUTE(step_, cur_);                                                                \
+      if (NST == 1) {                                                                      \
+        __syncthreads();                                                                   \
+        if (step_ + 1 < nsteps_) ISSUE(step_ + 1, smem);                                   \
+      }                                                                                    \
+    }                                                                                      \
+  } while (0)
 #define UA_PIPELINE(NSTEPS, STAGE_BYTES, ISSUE, COMPUTE)                                   \
   do {                                                                                     \
     const int nsteps_ = (NSTEPS);                                                          \
@@ -253,8 +274,12 @@ __global__ void __launch_bounds__(256) k_fwd_fused2(const T* __restrict__ Qp, co
 // ---------------------------------------------------------------------------------------------
 // Key-stationary backward (fused mode).  grid (Lp/128, Zk); 4 waves; wave w owns keys 128g+32w..+31,
 // sweeps query blocks from the last one down to its own; one (query block, query group) per step.
+// MR = more than one query group per kv head (the decay state of a query block then lives across steps).
 // ---------------------------------------------------------------------------------------------
-template <class T, int D, int NST>
+struct TrueC { static constexpr bool value = true; };
+struct FalseC { static constexpr bool value = false; };
+
+template <class T, int D, int NST, bool MR>
 __global__ void __launch_bounds__(256) k_bwd_keys2(BwdArgs<T> a) {
   extern __shared__ __align__(16) char smem[];
   using TN = Tile<T, 32, D>;
@@ -263,7 +288,7 @@ __global__ void __launch_bounds__(256) k_bwd_keys2(BwdArgs<T> a) {
   constexpr int TILES = 3 * TN::BYTES + 3 * TT::BYTES, SB = TILES + 1024;
   // stats row of a stage: [lse2: 32f][delta: 32f][ldest: 32f][unused: 32f][forward carries of the 128 keys: 128f]
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 31, hi = lane >> 5;
-  const int zk = blockIdx.y, Lp = a.Lp, L = a.L, nT = Lp / 32, R = a.R;
+  const int zk = blockIdx.y, Lp = a.Lp, L = a.L, nT = Lp / 32, R = MR ? a.R : 1;
   const int g = gridDim.x - 1 - blockIdx.x, sb = 4 * g + w, spos = 32 * sb + col;
   const int nTr = (L + 31) / 32, first = 4 * g;
   if (first >= nTr) return;                      // every key of this workgroup is padding
@@ -283,116 +308,140 @@ __global__ void __launch_bounds__(256) k_bwd_keys2(BwdArgs<T> a) {
 #pragma unroll
   for (int n = 0; n < NB; ++n) { dVt[n] = (f32x16){0}; dKt[n] = (f32x16){0}; }
   float dsrc_acc = 0.f, dcar = 0.f;
-  f32x16 aff, bias, gk, dB;
-  float lab[16];
+  f32x16 aff_s, bias_s, gk_s, dB_s;              // state of the current query block (used when MR)
+  float lab_s[16];
   const T* Kz = a.Kp + (long)zk * Lp * D;
   const T* KTz = a.KT + (long)zk * D * Lp;
+  const float* ldz = a.ldest + (long)zk * Lp;
+  const float* Cz = a.C + (long)zk * nT * Lp + 128 * g;
+  float* Dz = a.Dsuf + (long)zk * nT * Lp + spos;
 
 #define UA_ISSUE(s, base)                                                                   \
   {                                                                                         \
     const int tb_ = nTr - 1 - (s) / R;                                                      \
     const long zq_ = (long)zk * R + (s) % R;                                                \
+    const long qo_ = (zq_ * Lp + 32 * tb_) * D, to_ = zq_ * D * Lp + 32 * tb_;              \
     stN.issue((base), Kz + (long)(32 * tb_) * D, w);                                        \
-    stN.issue((base) + TN::BYTES, a.Qp + (zq_ * Lp + 32 * tb_) * D, w);                     \
-    stN.issue((base) + 2 * TN::BYTES, a.dOp + (zq_ * Lp + 32 * tb_) * D, w);                \
+    stN.issue((base) + TN::BYTES, a.Qp + qo_, w);                                           \
+    stN.issue((base) + 2 * TN::BYTES, a.dOp + qo_, w);                                      \
     stT.issue((base) + 3 * TN::BYTES, KTz + 32 * tb_, w);                                   \
-    stT.issue((base) + 3 * TN::BYTES + TT::BYTES, a.QT + zq_ * D * Lp + 32 * tb_, w);       \
-    stT.issue((base) + 3 * TN::BYTES + 2 * TT::BYTES, a.dOT + zq_ * D * Lp + 32 * tb_, w);  \
+    stT.issue((base) + 3 * TN::BYTES + TT::BYTES, a.QT + to_, w);                           \
+    stT.issue((base) + 3 * TN::BYTES + 2 * TT::BYTES, a.dOT + to_, w);                      \
     if (w == 0) {                                                                           \
       const float* src_;                                                                    \
       if (lane < 8) src_ = a.lse2 + zq_ * Lp + 32 * tb_ + 4 * lane;                         \
       else if (lane < 16) src_ = a.delta + zq_ * Lp + 32 * tb_ + 4 * (lane - 8);            \
-      else if (lane < 32) src_ = a.ldest + (long)zk * Lp + 32 * tb_ + 4 * (lane & 7);       \
-      else src_ = a.C + ((long)zk * nT + tb_) * Lp + 128 * g + 4 * (lane - 32);             \
+      else if (lane < 32) src_ = ldz + 32 * tb_ + 4 * (lane & 7);                           \
+      else src_ = Cz + (long)tb_ * Lp + 4 * (lane - 32);                                    \
       issue_row((base) + TILES, src_);                                                      \
     }                                                                                       \
   }
-#define UA_COMPUTE(s, base) bwd_step((s), (base))
-  auto bwd_step = [&] __device__ (int s, const char* base) {
+#define UA_COMPUTE_FAST(s, base) bwd_step((s), (base), FalseC(), false)
+#define UA_COMPUTE_SLOW(s, base)                                                            \
+  {                                                                                         \
+    const int tb_ = nTr - 1 - (s) / R;                                                      \
+    if (tb_ >= sb) bwd_step((s), (base), TrueC(), tb_ == sb);                               \
+  }
+  // MASKED: the step may be this wave's diagonal block (run-time flag diag); otherwise every pair is visible
+  auto bwd_step = [&] __device__ (int s, const char* base, auto masked_c, const bool diag) {
+    constexpr bool DIAG = decltype(masked_c)::value;
     const int tb = nTr - 1 - s / R, r = s % R;
-    if (tb < sb) return;                         // this wave's keys lie after the whole query block
     const T* sKt = reinterpret_cast<const T*>(base);
     const T* sQ = reinterpret_cast<const T*>(base + TN::BYTES);
     const T* sdO = reinterpret_cast<const T*>(base + 2 * TN::BYTES);
     const T* sKT = reinterpret_cast<const T*>(base + 3 * TN::BYTES);
     const T* sQT = reinterpret_cast<const T*>(base + 3 * TN::BYTES + TT::BYTES);
     const T* sdOT = reinterpret_cast<const T*>(base + 3 * TN::BYTES + 2 * TT::BYTES);
-    const bool diag = (tb == sb);
     const float* stats = reinterpret_cast<const float*>(base + TILES);
-    float l2t[16], dlt[16];
-    load_t16(stats, hi, l2t);
-    load_t16(stats + 32, hi, dlt);
-    if (r == 0) {
+    f32x16 aff_l, bias_l, gk_l, dB_l;
+    float lab_l[16];
+    f32x16& aff = MR ? aff_s : aff_l;
+    f32x16& bias = MR ? bias_s : bias_l;
+    f32x16& gk = MR ? gk_s : gk_l;
+    f32x16& dB = MR ? dB_s : dB_l;
+    float (&lab)[16] = MR ? lab_s : lab_l;
+    if (!MR || r == 0) {
       const float cin = stats[128 + 32 * w + col];
       load_t16(stats + 64, hi, lab);
-      gk = (f32x16){0};
+      f32x16 acc = {0};
 #pragma unroll
-      for (int q = 0; q < NQ; ++q) mma(gk, ld8(sKt + col * LS + 16 * q + 8 * hi), kp[q]);
-      f32x16 x;
+      for (int q = 0; q < NQ; ++q) mma(acc, ld8(sKt + col * LS + 16 * q + 8 * hi), kp[q]);
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         lab[v] += la;
-        gk[v] = log2_relu(gk[v]);
+        gk[v] = log2_relu(acc[v]);
         aff[v] = affinity(gk[v], lab[v]);
         const float l2 = log2_one_minus(aff[v]);
-        x[v] = (diag && t_of(v, hi) <= col) ? 0.f : l2;
+        bias[v] = (DIAG && diag && t_of(v, hi) <= col) ? 0.f : l2;
       }
-      block_prefix(x, hi);
+      block_prefix(bias, hi);
 #pragma unroll
-      for (int v = 0; v < 16; ++v) { bias[v] = x[v] + cin; dB[v] = 0.f; }
+      for (int v = 0; v < 16; ++v) { bias[v] += cin; if (MR) dB[v] = 0.f; }
     }
     {
       f32x16 sc = {0}, dP = {0};
 #pragma unroll
-      for (int q = 0; q < NQ; ++q) {
-        mma(sc, ld8(sQ + col * LS + 16 * q + 8 * hi), kp[q]);
-        mma(dP, ld8(sdO + col * LS + 16 * q + 8 * hi), vf[q]);
-      }
-      f32x16 P, dS;
+      for (int q = 0; q < NQ; ++q) mma(sc, ld8(sQ + col * LS + 16 * q + 8 * hi), kp[q]);
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) mma(dP, ld8(sdO + col * LS + 16 * q + 8 * hi), vf[q]);
+      float l2t[16], dlt[16];
+      load_t16(stats, hi, l2t);
+      load_t16(stats + 32, hi, dlt);
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[v], kLog2e, bias[v]) - l2t[v]);
-        p = (diag && t_of(v, hi) < col) ? 0.f : p;
-        P[v] = p;
-        dS[v] = p * (dP[v] - dlt[v]);
-        dB[v] += dS[v];
+        if (DIAG) p = (diag && t_of(v, hi) < col) ? 0.f : p;
+        sc[v] = p;
+        dP[v] = p * (dP[v] - dlt[v]);
       }
 #pragma unroll
       for (int q2 = 0; q2 < 2; ++q2) {
-        const Frag<T> bp = as_operand<T>(P, q2), bs = as_operand<T>(dS, q2);
+        const Frag<T> bp = as_operand<T>(sc, q2);
 #pragma unroll
-        for (int n = 0; n < NB; ++n) {
-          mma(dVt[n], ld8(sdOT + (32 * n + col) * TS + 16 * q2 + 8 * hi), bp);
-          mma(dKt[n], ld8(sQT + (32 * n + col) * TS + 16 * q2 + 8 * hi), bs);
-        }
+        for (int n = 0; n < NB; ++n) mma(dVt[n], ld8(sdOT + (32 * n + col) * TS + 16 * q2 + 8 * hi), bp);
       }
+#pragma unroll
+      for (int q2 = 0; q2 < 2; ++q2) {
+        const Frag<T> bs = as_operand<T>(dP, q2);
+#pragma unroll
+        for (int n = 0; n < NB; ++n) mma(dKt[n], ld8(sQT + (32 * n + col) * TS + 16 * q2 + 8 * hi), bs);
+      }
+#pragma unroll
+      for (int v = 0; v < 16; ++v) dB[v] = MR ? dB[v] + dP[v] : dP[v];
     }
-    if (r == R - 1) {
-      if (hi == 0) a.Dsuf[((long)zk * nT + tb) * Lp + spos] = dcar;
+    if (!MR || r == R - 1) {
+      if (hi == 0) Dz[(long)tb * Lp] = dcar;
       const float tot = block_suffix(dB, hi);
-      f32x16 dg;
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const float dl = (diag && t_of(v, hi) <= col) ? 0.f : dB[v] + dcar;
+        float dl = dB[v] + dcar;
+        if (DIAG) dl = (diag && t_of(v, hi) <= col) ? 0.f : dl;
         const float av = aff[v];
-        const float den = fmaxf(fminf(av, kAMax), kAMinBwd) - 1.0f;
+        const float den = __builtin_amdgcn_fmed3f(av, kAMinBwd, kAMax) - 1.0f;
         const float dA = (av <= kAMax) ? dl * __builtin_amdgcn_rcpf(den) : 0.f;
-        dsrc_acc += dA * av;
+        dsrc_acc = __builtin_fmaf(dA, av, dsrc_acc);
         const float f = (2.0f / 3.0f) * __builtin_amdgcn_exp2f(__builtin_fmaf(gk[v], -1.0f / 3.0f, lab[v]));
-        dg[v] = (gk[v] > -1.0e30f) ? dA * f : 0.f;
+        dB[v] = (gk[v] > -1.0e30f) ? dA * f : 0.f;
       }
       dcar += tot;
 #pragma unroll
       for (int q2 = 0; q2 < 2; ++q2) {
-        const Frag<T> b = as_operand<T>(dg, q2);
+        const Frag<T> b = as_operand<T>(dB, q2);
 #pragma unroll
         for (int n = 0; n < NB; ++n) mma(dKt[n], ld8(sKT + (32 * n + col) * TS + 16 * q2 + 8 * hi), b);
       }
     }
   };
-  UA_PIPELINE((nTr - first) * R, SB, UA_ISSUE, UA_COMPUTE);
+  {
+    // the last four query blocks of the sweep hold the diagonal blocks of the four waves
+    const int nblk = nTr - first, total = nblk * R, nfast = (nblk > 4 ? nblk - 4 : 0) * R;
+    UA_PIPE_START(total, UA_ISSUE);
+    UA_PIPE_RANGE(0, nfast, total, SB, UA_ISSUE, UA_COMPUTE_FAST);
+    UA_PIPE_RANGE(nfast, total, total, SB, UA_ISSUE, UA_COMPUTE_SLOW);
+  }
 #undef UA_ISSUE
-#undef UA_COMPUTE
+#undef UA_COMPUTE_FAST
+#undef UA_COMPUTE_SLOW
   // epilogue
   float lo, up;
   swap32(dsrc_acc, lo, up);
@@ -566,5 +615,7 @@ __global__ void __launch_bounds__(256) k_bwd_queries2(BwdArgs<T> a, T* __restric
 }
 
 #undef UA_PIPELINE
+#undef UA_PIPE_RANGE
+#undef UA_PIPE_START
 
 }  // namespace ua

@@ -26,13 +26,23 @@ static hipError_t bwd_t(const BwdArgsV& v, int Zk, hipStream_t s) {
   hipLaunchKernelGGL((k_bwd_keys<T, D, NW, COLS>), dim3(groups, Zk), dim3(64 * NW), lds, s, a);
   return hipGetLastError();
 }
+// explicit instantiations (the implicit ones are not emitted on the host side for kernels holding lambdas)
+#define UA_INST(T, D, NST) \
+  template __global__ void k_bwd_keys2<T, D, NST, false>(BwdArgs<T>); template __global__ void k_bwd_keys2<T, D, NST, true>(BwdArgs<T>);
+UA_INST(bf16, 64, 2) UA_INST(bf16, 128, 2) UA_INST(float, 64, 1) UA_INST(float, 128, 1)
+#undef UA_INST
+
+template <class T, int D, int NST, bool MR>
+static hipError_t bwd2_mr(const BwdArgs<T>& a, int Lp, int Zk, hipStream_t s) {
+  const size_t lds = NST * (3 * Tile<T, 32, D>::BYTES + 3 * Tile<T, D, 32>::BYTES + 1024);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k_bwd_keys2<T, D, NST, MR>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  hipLaunchKernelGGL((k_bwd_keys2<T, D, NST, MR>), dim3(Lp / 128, Zk), dim3(256), lds, s, a);
+  return hipGetLastError();
+}
 template <class T, int D, int NST>
 static hipError_t bwd2_t(const BwdArgsV& v, int Zk, hipStream_t s) {
   const BwdArgs<T> a = typed<T>(v);
-  const size_t lds = NST * (3 * Tile<T, 32, D>::BYTES + 3 * Tile<T, D, 32>::BYTES + 1024);
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k_bwd_keys2<T, D, NST>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-  hipLaunchKernelGGL((k_bwd_keys2<T, D, NST>), dim3(v.Lp / 128, Zk), dim3(256), lds, s, a);
-  return hipGetLastError();
+  return v.R > 1 ? bwd2_mr<T, D, NST, true>(a, v.Lp, Zk, s) : bwd2_mr<T, D, NST, false>(a, v.Lp, Zk, s);
 }
 template <class T, int D>
 static hipError_t bwd_nw(const BwdArgsV& v, int Zk, int cols, hipStream_t s) {
