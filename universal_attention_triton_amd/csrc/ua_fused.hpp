@@ -20,44 +20,52 @@ __device__ __forceinline__ void issue_row(void* lds_base, const void* src_lane) 
   __builtin_amdgcn_global_load_lds(src_lane, (lds_ptr_t)lds_base, 16, 0, 0);
 }
 
-// generic pipeline skeleton:  ISSUE(step, stage_base)  COMPUTE(step, stage_base)
+// Pipeline skeleton.  Every kernel declares two STATIC LDS arrays stage0 / stage1 (distinct objects, so the
+// compiler can prove that the asynchronous loads filling one stage do not alias the reads of the other and
+// does not wait for them) and provides ISSUE(step, stage) and COMPUTE(step, stage).
 // UA_PIPE_RANGE runs steps [S0, S1) of a pipeline of NSTEPS steps whose step S0 has already been issued
 // (by UA_PIPE_START or by the previous range), so that consecutive ranges may use different COMPUTE bodies.
 #define UA_PIPE_START(NSTEPS, ISSUE)                                                       \
   do {                                                                                     \
-    if ((NSTEPS) > 0) ISSUE(0, smem);                                                      \
+    if ((NSTEPS) > 0) ISSUE(0, stage0);                                                    \
   } while (0)
-#define UA_PIPE_RANGE(S0, S1, NSTEPS, STAGE_BYTES, ISSUE, COMPUTE)                         \
+#define UA_STEP2_(STEP, NSTEPS, CUR, NXT, ISSUE, COMPUTE)                                  \
+  {                                                                                        \
+    wait_async_loads();                                                                    \
+    __syncthreads();                                                                       \
+    if ((STEP) + 1 < (NSTEPS)) ISSUE((STEP) + 1, NXT);                                     \
+    COMPUTE((STEP), CUR);                                                                  \
+  }
+// With two stages S0 must be even (even steps live in stage0); the loop is unrolled by two so that both
+// stage roles are compile-time constants on a straight-line path.
+#define UA_PIPE_RANGE(S0, S1, NSTEPS, ISSUE, COMPUTE)                                      \
   do {                                                                                     \
     const int nsteps_ = (NSTEPS), s1_ = (S1);                                              \
-    for (int step_ = (S0); step_ < s1_; ++step_) {                                         \
-      wait_async_loads();                                                                  \
-      __syncthreads();                                                                     \
-      char* cur_ = smem + (NST == 2 ? (step_ & 1) * (STAGE_BYTES) : 0);                    \
-      if (NST == 2 && step_ + 1 < nsteps_) ISSUE(step_ + 1, smem + ((step_ + 1) & 1) * (STAGE_BYTES)); \
-      COMPUTE(step_, cur_);                                                                \
-      if (NST == 1) {                                                                      \
+    int step_ = (S0);                                                                      \
+    if constexpr (NST == 2) {                                                              \
+      for (; step_ + 1 < s1_; step_ += 2) {                                                \
+        UA_STEP2_(step_, nsteps_, stage0, stage1, ISSUE, COMPUTE)                          \
+        UA_STEP2_(step_ + 1, nsteps_, stage1, stage0, ISSUE, COMPUTE)                      \
+      }                                                                                    \
+      if (step_ < s1_) UA_STEP2_(step_, nsteps_, stage0, stage1, ISSUE, COMPUTE)           \
+    } else {                                                                               \
+      for (; step_ < s1_; ++step_) {                                                       \
+        wait_async_loads();                                                                \
         __syncthreads();                                                                   \
-        if (step_ + 1 < nsteps_) ISSUE(step_ + 1, smem);                                   \
+        COMPUTE(step_, stage0);                                                            \
+        __syncthreads();                                                                   \
+        if (step_ + 1 < nsteps_) ISSUE(step_ + 1, stage0);                                 \
       }                                                                                    \
     }                                                                                      \
   } while (0)
-#define UA_PIPELINE(NSTEPS, STAGE_BYTES, ISSUE, COMPUTE)                                   \
+#define UA_PIPELINE(NSTEPS, ISSUE, COMPUTE)                                                \
   do {                                                                                     \
-    const int nsteps_ = (NSTEPS);                                                          \
-    if (nsteps_ > 0) ISSUE(0, smem);                                                       \
-    for (int step_ = 0; step_ < nsteps_; ++step_) {                                        \
-      wait_async_loads();                                                                  \
-      __syncthreads();                                                                     \
-      char* cur_ = smem + (NST == 2 ? (step_ & 1) * (STAGE_BYTES) : 0);                    \
-      if (NST == 2 && step_ + 1 < nsteps_) ISSUE(step_ + 1, smem + ((step_ + 1) & 1) * (STAGE_BYTES)); \
-      COMPUTE(step_, cur_);                                                                \
-      if (NST == 1) {                                                                      \
-        __syncthreads();                                                                   \
-        if (step_ + 1 < nsteps_) ISSUE(step_ + 1, smem);                                   \
-      }                                                                                    \
-    }                                                                                      \
+    UA_PIPE_START(NSTEPS, ISSUE);                                                          \
+    UA_PIPE_RANGE(0, NSTEPS, NSTEPS, ISSUE, COMPUTE);                                      \
   } while (0)
+#define UA_STAGES(BYTES)                                                                   \
+  __shared__ __attribute__((aligned(1024))) char stage0[BYTES];                            \
+  __shared__ __attribute__((aligned(1024))) char stage1[NST == 2 ? (BYTES) : 1024]
 
 // ---------------------------------------------------------------------------------------------
 // C[z][tb][s] = sum_{u < 32*tb, u > s} log2(1 - A[s,u])   (tb >= s/32).  grid (Lp/128, Zk), 4 waves.
@@ -65,9 +73,9 @@ __device__ __forceinline__ void issue_row(void* lds_base, const void* src_lane) 
 template <class T, int D, int NST>
 __global__ void __launch_bounds__(256) k_carry2(const T* __restrict__ Kp, const float* __restrict__ lsrc,
                                                 const float* __restrict__ ldest, float* __restrict__ C, int Lp) {
-  extern __shared__ __align__(16) char smem[];
   using TN = Tile<T, 32, D>;
   constexpr int NQ = D / 16, LS = TN::STRIDE, SB = TN::BYTES + 1024;   // tile + [ldest of the block: 32 floats]
+  UA_STAGES(SB);
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 31, hi = lane >> 5;
   const int z = blockIdx.y, nT = Lp / 32, sb = 4 * blockIdx.x + w, first = 4 * blockIdx.x;
   Stager<TN, 4> st;
@@ -108,7 +116,7 @@ __global__ void __launch_bounds__(256) k_carry2(const T* __restrict__ Kp, const 
       carry += lo + up;                                                                     \
     }                                                                                       \
   }
-  UA_PIPELINE(nT - first, SB, UA_ISSUE, UA_COMPUTE);
+  UA_PIPELINE(nT - first, UA_ISSUE, UA_COMPUTE);
 #undef UA_ISSUE
 #undef UA_COMPUTE
 }
@@ -122,15 +130,16 @@ __global__ void __launch_bounds__(256) k_fwd_fused2(const T* __restrict__ Qp, co
                                                     const float* __restrict__ ldest, const float* __restrict__ C,
                                                     T* __restrict__ O, float* __restrict__ lse, float* __restrict__ lse2,
                                                     int R, int L, int Lp, int d) {
-  extern __shared__ __align__(16) char smem[];
   using TN = Tile<T, 32, D>;
   using TT = Tile<T, D, 32>;
   constexpr int NQ = D / 16, NB = D / 32, LS = TN::STRIDE, TS = TT::STRIDE, PS = lds_stride<T>(64);
   constexpr int TILES = 2 * TN::BYTES + 2 * TT::BYTES, SB = TILES + 4 * 1024;   // + per wave [C row: 64f][lsrc: 64f]
+  UA_STAGES(SB);
+  __shared__ __attribute__((aligned(16))) T sPbuf[4 * 32 * PS];
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 31, hi = lane >> 5;
   const int zq = blockIdx.y, zk = zq / R, nT = Lp / 32;
   const int jt = gridDim.x - 1 - blockIdx.x, tb = 4 * jt + w;
-  T* sPw = reinterpret_cast<T*>(smem + NST * SB) + w * 32 * PS;
+  T* sPw = sPbuf + w * 32 * PS;
   const int pcol = perm16(col);
   Stager<TN, 4> stN;
   Stager<TT, 4> stT;
@@ -247,7 +256,7 @@ __global__ void __launch_bounds__(256) k_fwd_fused2(const T* __restrict__ Qp, co
       }
     }
   };
-  UA_PIPELINE(n_kt, SB, UA_ISSUE, UA_COMPUTE);
+  UA_PIPELINE(n_kt, UA_ISSUE, UA_COMPUTE);
 #undef UA_ISSUE
 #undef UA_COMPUTE
   // epilogue
@@ -281,11 +290,11 @@ struct FalseC { static constexpr bool value = false; };
 
 template <class T, int D, int NST, bool MR>
 __global__ void __launch_bounds__(256) k_bwd_keys2(BwdArgs<T> a) {
-  extern __shared__ __align__(16) char smem[];
   using TN = Tile<T, 32, D>;
   using TT = Tile<T, D, 32>;
   constexpr int NQ = D / 16, NB = D / 32, LS = TN::STRIDE, TS = TT::STRIDE;
   constexpr int TILES = 3 * TN::BYTES + 3 * TT::BYTES, SB = TILES + 1024;
+  UA_STAGES(SB);
   // stats row of a stage: [lse2: 32f][delta: 32f][ldest: 32f][unused: 32f][forward carries of the 128 keys: 128f]
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 31, hi = lane >> 5;
   const int zk = blockIdx.y, Lp = a.Lp, L = a.L, nT = Lp / 32, R = MR ? a.R : 1;
@@ -434,10 +443,10 @@ __global__ void __launch_bounds__(256) k_bwd_keys2(BwdArgs<T> a) {
   };
   {
     // the last four query blocks of the sweep hold the diagonal blocks of the four waves
-    const int nblk = nTr - first, total = nblk * R, nfast = (nblk > 4 ? nblk - 4 : 0) * R;
+    const int nblk = nTr - first, total = nblk * R, nfast = ((nblk > 4 ? nblk - 4 : 0) * R) & ~1;
     UA_PIPE_START(total, UA_ISSUE);
-    UA_PIPE_RANGE(0, nfast, total, SB, UA_ISSUE, UA_COMPUTE_FAST);
-    UA_PIPE_RANGE(nfast, total, total, SB, UA_ISSUE, UA_COMPUTE_SLOW);
+    UA_PIPE_RANGE(0, nfast, total, UA_ISSUE, UA_COMPUTE_FAST);
+    UA_PIPE_RANGE(nfast, total, total, UA_ISSUE, UA_COMPUTE_SLOW);
   }
 #undef UA_ISSUE
 #undef UA_COMPUTE_FAST
@@ -463,15 +472,16 @@ __global__ void __launch_bounds__(256) k_bwd_keys2(BwdArgs<T> a) {
 // ---------------------------------------------------------------------------------------------
 template <class T, int D, int NST>
 __global__ void __launch_bounds__(256) k_bwd_queries2(BwdArgs<T> a, T* __restrict__ dq, int d) {
-  extern __shared__ __align__(16) char smem[];
   using TN = Tile<T, 32, D>;
   using TT = Tile<T, D, 32>;
   constexpr int NQ = D / 16, NB = D / 32, LS = TN::STRIDE, TS = TT::STRIDE, SS = lds_stride<T>(32);
   constexpr int TILES = 4 * TN::BYTES + 2 * TT::BYTES, SB = TILES + 4 * 1024;   // + per wave [C: 64f][lsrc: 64f][Dsuf: 64f]
+  UA_STAGES(SB);
+  __shared__ __attribute__((aligned(16))) T sXbuf[4 * 2 * 32 * SS];
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 31, hi = lane >> 5;
   const int zk = blockIdx.y, Lp = a.Lp, L = a.L, nT = Lp / 32, R = a.R;
   const int jt = gridDim.x - 1 - blockIdx.x, tb = 4 * jt + w;
-  T* sXs = reinterpret_cast<T*>(smem + NST * SB) + w * 2 * 32 * SS;
+  T* sXs = sXbuf + w * 2 * 32 * SS;
   T* sXg = sXs + 32 * SS;
   const int pcol = perm16(col);
   Stager<TN, 4> stN;
@@ -590,7 +600,7 @@ __global__ void __launch_bounds__(256) k_bwd_queries2(BwdArgs<T> a, T* __restric
         }
       }
     };
-    UA_PIPELINE(n_kt, SB, UA_ISSUE, UA_COMPUTE);
+    UA_PIPELINE(n_kt, UA_ISSUE, UA_COMPUTE);
 #undef UA_ISSUE
 #undef UA_COMPUTE
     __syncthreads();   // the next group's prologue reuses stage 0
@@ -617,5 +627,7 @@ __global__ void __launch_bounds__(256) k_bwd_queries2(BwdArgs<T> a, T* __restric
 #undef UA_PIPELINE
 #undef UA_PIPE_RANGE
 #undef UA_PIPE_START
+#undef UA_STEP2_
+#undef UA_STAGES
 
 }  // namespace ua

@@ -34,9 +34,7 @@ UA_INST(bf16, 64, 2) UA_INST(bf16, 128, 2) UA_INST(float, 64, 1) UA_INST(float, 
 
 template <class T, int D, int NST, bool MR>
 static hipError_t bwd2_mr(const BwdArgs<T>& a, int Lp, int Zk, hipStream_t s) {
-  const size_t lds = NST * (3 * Tile<T, 32, D>::BYTES + 3 * Tile<T, D, 32>::BYTES + 1024);
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k_bwd_keys2<T, D, NST, MR>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-  hipLaunchKernelGGL((k_bwd_keys2<T, D, NST, MR>), dim3(Lp / 128, Zk), dim3(256), lds, s, a);
+  hipLaunchKernelGGL((k_bwd_keys2<T, D, NST, MR>), dim3(Lp / 128, Zk), dim3(256), 0, s, a);
   return hipGetLastError();
 }
 template <class T, int D, int NST>
@@ -64,9 +62,7 @@ UA_INST(bf16, 64, 2) UA_INST(bf16, 128, 2) UA_INST(float, 64, 1) UA_INST(float, 
 template <class T, int D, int NST>
 static hipError_t bwdq_t(const BwdArgsV& v, void* dq, int d, int Zk, hipStream_t s) {
   const BwdArgs<T> a = typed<T>(v);
-  const size_t lds = NST * (4 * Tile<T, 32, D>::BYTES + 2 * Tile<T, D, 32>::BYTES + 4096) + 4 * 2 * 32 * lds_stride<T>(32) * sizeof(T);
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k_bwd_queries2<T, D, NST>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-  hipLaunchKernelGGL((k_bwd_queries2<T, D, NST>), dim3(v.Lp / 128, Zk), dim3(256), lds, s, a, (T*)dq, d);
+  hipLaunchKernelGGL((k_bwd_queries2<T, D, NST>), dim3(v.Lp / 128, Zk), dim3(256), 0, s, a, (T*)dq, d);
   return hipGetLastError();
 }
 hipError_t launch_bwd_queries(int dtype, int D, const BwdArgsV& a, void* dq, int d, int Zk, hipStream_t s) {
