@@ -122,7 +122,7 @@ __global__ void __launch_bounds__(64 * NW) k_bwd_keys(BwdArgs<T> a) {
         x[v] = (valid && tpos > spos) ? l2 : 0.f;
       }
       block_prefix(x, hi);
-      const float cin = a.C[((long)zk * nT + tb) * Lp + min(spos, Lp - 1)];
+      const float cin = a.C[((long)zk * (Lp / 16) + 2 * tb) * Lp + min(spos, Lp - 1)];   // carries are kept per 16-query tile
 #pragma unroll
       for (int v = 0; v < 16; ++v) bias[v] = x[v] + cin;
     }

@@ -58,7 +58,7 @@ Layout make_layout(const ua_desc& d, bool chunked) {
   Layout l{};
   l.D = d.d <= 64 ? 64 : 128;
   l.Lp = (int)align_up((size_t)d.L, 128);
-  l.nT = l.Lp / 32;
+  l.nT = l.Lp / 16;     // carries are kept per 16-query tile
   l.nch = chunked ? d.L / d.chunk : 1;
   l.Zk = d.b * d.h;
   l.Zq = l.Zk * d.r;
@@ -109,13 +109,15 @@ ua::RowsView chunked_view(const ua_chunked& c, int nch) {
 ua::RowsView null_view() { ua::RowsView v{}; v.inner = 1; v.H = v.R = v.N = 1; return v; }
 
 template <class T>
-hipError_t pack_t(int D, const ua::RowsView& x, void* nat, void* tr, int d, int L, int Lp, int Z, hipStream_t s) {
-  if (D == 64) hipLaunchKernelGGL((ua::k_pack<T, 64>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp);
-  else hipLaunchKernelGGL((ua::k_pack<T, 128>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp);
+hipError_t pack_t(int D, const ua::RowsView& x, void* nat, void* tr, int d, int L, int Lp, int Z, int tr_mode, hipStream_t s) {
+  if (D == 64) hipLaunchKernelGGL((ua::k_pack<T, 64>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp, tr_mode);
+  else hipLaunchKernelGGL((ua::k_pack<T, 128>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp, tr_mode);
   return hipGetLastError();
 }
-hipError_t pack(int dtype, int D, const ua::RowsView& x, void* nat, void* tr, int d, int L, int Lp, int Z, hipStream_t s) {
-  return dtype == UA_BF16 ? pack_t<ua::bf16>(D, x, nat, tr, d, L, Lp, Z, s) : pack_t<float>(D, x, nat, tr, d, L, Lp, Z, s);
+// tr_mode: column order of the transposed copy inside each group of 32 positions
+enum { TR_PERM16 = 0, TR_PERM32 = 1, TR_NATURAL = 2 };
+hipError_t pack(int dtype, int D, const ua::RowsView& x, void* nat, void* tr, int d, int L, int Lp, int Z, int tr_mode, hipStream_t s) {
+  return dtype == UA_BF16 ? pack_t<ua::bf16>(D, x, nat, tr, d, L, Lp, Z, tr_mode, s) : pack_t<float>(D, x, nat, tr, d, L, Lp, Z, tr_mode, s);
 }
 
 // ---- optional per-kernel timing (hipEvents on the launch stream) ---------------------------
@@ -163,13 +165,15 @@ hipError_t zero_fill(void* p, size_t bytes, hipStream_t s) {   // bytes is a mul
 }
 
 // packs K, V and Q in both orientations and the log-gates
-int pack_inputs(const ua_desc& d, const Layout& l, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* src,
-                const void* dest, char* ws, hipStream_t s) {
+int pack_inputs(const ua_desc& d, const Layout& l, bool chunked, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq,
+                const void* src, const void* dest, char* ws, hipStream_t s) {
   UA_PROF("pack_inputs", s);
   const ua::RowsView K = rows_view(*kc, d.h, 1), V = rows_view(*vc, d.h, 1), Q = rows_view(*xq, d.h, d.r);
-  UA_HIP(pack(d.dtype, l.D, K, ws + l.Kp, ws + l.KT, d.d, d.L, l.Lp, l.Zk, s));
-  UA_HIP(pack(d.dtype, l.D, V, ws + l.Vp, ws + l.VT, d.d, d.L, l.Lp, l.Zk, s));
-  UA_HIP(pack(d.dtype, l.D, Q, ws + l.Qp, ws + l.QT, d.d, d.L, l.Lp, l.Zq, s));
+  // the chunked kernels work on 32x32 tiles, the fused ones on 16x16 tiles (and read V^T in natural order)
+  const int mode = chunked ? TR_PERM16 : TR_PERM32;
+  UA_HIP(pack(d.dtype, l.D, K, ws + l.Kp, ws + l.KT, d.d, d.L, l.Lp, l.Zk, mode, s));
+  UA_HIP(pack(d.dtype, l.D, V, ws + l.Vp, ws + l.VT, d.d, d.L, l.Lp, l.Zk, chunked ? TR_PERM16 : TR_NATURAL, s));
+  UA_HIP(pack(d.dtype, l.D, Q, ws + l.Qp, ws + l.QT, d.d, d.L, l.Lp, l.Zq, mode, s));
   const dim3 grid((l.Lp + 255) / 256, l.Zk);
   if (d.dtype == UA_BF16)
     hipLaunchKernelGGL((ua::k_gates<ua::bf16>), grid, dim3(256), 0, s, (const ua::bf16*)src, (const ua::bf16*)dest,
@@ -285,7 +289,7 @@ int ua_fused_fwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, cons
   if (!O || !lse) return fail(UA_EINVAL, "null output tensor");
   char* w = (char*)ws;
   hipStream_t s = (hipStream_t)stream;
-  if (int e = pack_inputs(*desc, l, kc, vc, xq, static_src, static_dest, w, s)) return e;
+  if (int e = pack_inputs(*desc, l, false, kc, vc, xq, static_src, static_dest, w, s)) return e;
   return run_fused_fwd_kernels(*desc, l, w, O, lse, tuned_variant(*desc, UA_OP_FUSED_FWD), s);
 }
 
@@ -300,7 +304,7 @@ int ua_fused_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, cons
   hipStream_t s = (hipStream_t)stream;
   const ua_desc& d = *desc;
   if (!ws_has_fwd) {
-    if (int e = pack_inputs(d, l, kc, vc, xq, static_src, static_dest, w, s)) return e;
+    if (int e = pack_inputs(d, l, false, kc, vc, xq, static_src, static_dest, w, s)) return e;
     UA_HIP(ua::launch_carry(d.dtype, l.D, w + l.Kp, (const float*)(w + l.lsrc), (const float*)(w + l.ldest),
                             (float*)(w + l.C), l.Lp, l.Zk, s));
   }
@@ -309,7 +313,7 @@ int ua_fused_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, cons
   const ua::RowsView lsev = contiguous_view(lse, d.L, 1), none = null_view();
   {
     UA_PROF("pack_dO+delta", s);
-    UA_HIP(pack(d.dtype, l.D, dOv, w + l.dOp, w + l.dOT, d.d, d.L, l.Lp, l.Zq, s));
+    UA_HIP(pack(d.dtype, l.D, dOv, w + l.dOp, w + l.dOT, d.d, d.L, l.Lp, l.Zq, TR_PERM32, s));
   }
   if (d.dtype == UA_BF16) UA_HIP(delta_t<ua::bf16>(Ov, dOv, none, lsev, (float*)(w + l.delta), (float*)(w + l.lse2), d.d, d.L, l.Lp, l.Zq, s));
   else UA_HIP(delta_t<float>(Ov, dOv, none, lsev, (float*)(w + l.delta), (float*)(w + l.lse2), d.d, d.L, l.Lp, l.Zq, s));
@@ -325,7 +329,7 @@ int ua_fwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
   char* w = (char*)ws;
   hipStream_t s = (hipStream_t)stream;
   const ua_desc& d = *desc;
-  if (int e = pack_inputs(d, l, kc, vc, xq, static_src, static_dest, w, s)) return e;
+  if (int e = pack_inputs(d, l, true, kc, vc, xq, static_src, static_dest, w, s)) return e;
   UA_PROF("k_fwd_chunked", s);
   UA_HIP(ua::launch_fwd_chunked(d.dtype, l.D, w + l.Qp, w + l.Kp, w + l.VT, (const float*)(w + l.lsrc),
                                 (const float*)(w + l.ldest), out->ptr, denom, (float*)(w + l.lse2), out->stride_z, out->stride_t, out->stride_d, out->stride_i, d.r, d.L,
@@ -346,7 +350,7 @@ int ua_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
   const ua_desc& d = *desc;
   if (!ws_has_fwd) {
     // recompute the per-chunk normalisers (the partial outputs themselves are passed in)
-    if (int e = pack_inputs(d, l, kc, vc, xq, static_src, static_dest, w, s)) return e;
+    if (int e = pack_inputs(d, l, true, kc, vc, xq, static_src, static_dest, w, s)) return e;
     UA_HIP(ua::launch_fwd_chunked(d.dtype, l.D, w + l.Qp, w + l.Kp, w + l.VT, (const float*)(w + l.lsrc),
                                   (const float*)(w + l.ldest), nullptr, nullptr, (float*)(w + l.lse2), 0, 0, 0, 0, d.r, d.L, l.Lp, d.d, d.chunk, l.nch, l.Zk, s));
   }
@@ -359,7 +363,7 @@ int ua_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
   ua::RowsView gdv;
   gdv.p = g_denom; gdv.sb = (long)d.L * l.nch; gdv.sh = 0; gdv.sr = 0; gdv.sn = 1; gdv.so = 0; gdv.si = l.nch; gdv.sc = 1;
   gdv.inner = 1 << 30; gdv.H = 1; gdv.R = 1; gdv.N = l.nch;
-  UA_HIP(pack(d.dtype, l.D, gv, w + l.dOp, w + l.dOT, d.d, d.L, l.Lp, l.Zq * l.nch, s));
+  UA_HIP(pack(d.dtype, l.D, gv, w + l.dOp, w + l.dOT, d.d, d.L, l.Lp, l.Zq * l.nch, TR_PERM16, s));
   if (d.dtype == UA_BF16) UA_HIP(delta_t<ua::bf16>(outv, gv, gdv, none, (float*)(w + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s));
   else UA_HIP(delta_t<float>(outv, gv, gdv, none, (float*)(w + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s));
   return run_bwd_common(d, l, w, true, static_src, static_dest, dkc, dvc, dxq, dsrc, ddest, s);

@@ -48,6 +48,18 @@ __device__ __forceinline__ void mma(f32x16& c, const Frag<float>& a, const Frag<
   for (int e = 0; e < 8; ++e) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a.v[e], b.v[e], c, 0, 0, 0);
 }
 
+// 16x16 tiles (v_mfma_f32_16x16x32_bf16 / 16x16x4_f32): A lane l = row l%16, k-values 8*(l/16)..+7 of a
+// 32-wide k-step; B lane l = column l%16, same k-values; result f32x4: lane <-> column l%16, register v <->
+// row 4*(l/16) + v.  In the [t, s] orientation a lane therefore owns one key and 4 of the 16 queries of a tile.
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+__device__ __forceinline__ void mma16(f32x4& c, const Frag<bf16>& a, const Frag<bf16>& b) {
+  c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ void mma16(f32x4& c, const Frag<float>& a, const Frag<float>& b) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e) c = __builtin_amdgcn_mfma_f32_16x16x4f32(a.v[e], b.v[e], c, 0, 0, 0);
+}
+
 template <class T> __device__ __forceinline__ T cvt(float x);
 template <> __device__ __forceinline__ float cvt<float>(float x) { return x; }
 template <> __device__ __forceinline__ bf16 cvt<bf16>(float x) { return (bf16)x; }
@@ -59,6 +71,18 @@ template <class T> __device__ __forceinline__ Frag<T> as_operand(const f32x16& c
   for (int e = 0; e < 8; ++e) f.v[e] = cvt<T>(c[8 * q + e]);
   return f;
 }
+
+// two 16x16 result tiles covering 32 consecutive queries (tile i: t = 16i + 4g + v) as ONE B operand of a
+// product contracting over those 32 queries: element e of lane group g is query 16*(e/4) + 4g + e%4
+template <class T> __device__ __forceinline__ Frag<T> as_operand16(const f32x4& x0, const f32x4& x1) {
+  Frag<T> f;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) { f.v[e] = cvt<T>(x0[e]); f.v[4 + e] = cvt<T>(x1[e]); }
+  return f;
+}
+// column of position t (inside its group of 32) in the transposed working tensors read by such products:
+// the 8 k-values of lane group g are then 8 CONSECUTIVE elements starting at 8g
+__host__ __device__ __forceinline__ constexpr int perm32(int t) { return (t & ~31) | (((t >> 2) & 3) << 3) | (((t >> 4) & 1) << 2) | (t & 3); }
 
 // 8 contiguous elements (global or LDS); p must be 16-byte aligned
 template <class T> __device__ __forceinline__ Frag<T> ld8(const T* p) {
@@ -216,6 +240,64 @@ __device__ __forceinline__ float block_suffix(f32x16& x, int hi) {
     run += lo + up;
   }
   return run;
+}
+
+// ---- scans over the 32 queries of two 16x16 tiles (lane = key l%16, lane group g = l/16 holds t = 4g+v) ----
+struct GroupMasks { float g1, g2, n1, n2; };    // g1 = g&1, g2 = g>>1 as floats, n* their complements
+__device__ __forceinline__ GroupMasks group_masks(int lane) {
+  const int g = lane >> 4;
+  GroupMasks m;
+  m.g1 = (g & 1) ? 1.f : 0.f; m.g2 = (g & 2) ? 1.f : 0.f; m.n1 = 1.f - m.g1; m.n2 = 1.f - m.g2;
+  return m;
+}
+// s = per-lane sum of its 4 queries; before = sum over lane groups holding EARLIER queries, after = LATER ones,
+// total = all four groups
+__device__ __forceinline__ void group_scan(float s, const GroupMasks& m, float& before, float& after, float& total) {
+  float a, b;
+  swap16(s, a, b);                   // a: group with g&1 == 0 of the pair, b: the other
+  float lo, up;
+  swap32(a + b, lo, up);             // lo: groups {0,1}, up: groups {2,3}
+  before = __builtin_fmaf(m.g1, a, m.g2 * lo);
+  after = __builtin_fmaf(m.n1, b, m.n2 * up);
+  total = lo + up;
+}
+// inclusive prefix over t = 0..31 (x0: queries 0..15, x1: 16..31); returns the total
+__device__ __forceinline__ float prefix32(f32x4& x0, f32x4& x1, const GroupMasks& m) {
+  x0[1] += x0[0]; x0[2] += x0[1]; x0[3] += x0[2];
+  x1[1] += x1[0]; x1[2] += x1[1]; x1[3] += x1[2];
+  float b0, a0, t0, b1, a1, t1;
+  group_scan(x0[3], m, b0, a0, t0);
+  group_scan(x1[3], m, b1, a1, t1);
+  b1 += t0;
+#pragma unroll
+  for (int v = 0; v < 4; ++v) { x0[v] += b0; x1[v] += b1; }
+  return t0 + t1;
+}
+// inclusive suffix: x[t] = sum_{t' >= t}; returns the total, t1 = total of the second tile (queries 16..31)
+__device__ __forceinline__ float suffix32(f32x4& x0, f32x4& x1, const GroupMasks& m, float& t1) {
+  x0[2] += x0[3]; x0[1] += x0[2]; x0[0] += x0[1];
+  x1[2] += x1[3]; x1[1] += x1[2]; x1[0] += x1[1];
+  float b0, a0, t0, b1, a1;
+  group_scan(x0[0], m, b0, a0, t0);
+  group_scan(x1[0], m, b1, a1, t1);
+  a0 += t1;
+#pragma unroll
+  for (int v = 0; v < 4; ++v) { x0[v] += a0; x1[v] += a1; }
+  return t0 + t1;
+}
+// the 4 per-query values of lane group g inside a 16-query tile, from a float array indexed by query
+__device__ __forceinline__ f32x4 load_t4(const float* __restrict__ p16, int g) {
+  const float4 x = *reinterpret_cast<const float4*>(p16 + 4 * g);
+  return (f32x4){x.x, x.y, x.z, x.w};
+}
+// all-reduce over the 16 lanes of a lane group (the 16 keys of a tile)
+__device__ __forceinline__ float allmax16(float v) {
+  v = fmaxf(v, dpp<kDppXor1>(v)); v = fmaxf(v, dpp<kDppXor2>(v)); v = fmaxf(v, dpp<kDppRor4>(v)); v = fmaxf(v, dpp<kDppRor8>(v));
+  return v;
+}
+__device__ __forceinline__ float allsum16(float v) {
+  v += dpp<kDppXor1>(v); v += dpp<kDppXor2>(v); v += dpp<kDppRor4>(v); v += dpp<kDppRor8>(v);
+  return v;
 }
 
 // ---------------------------------------------------------------------------------

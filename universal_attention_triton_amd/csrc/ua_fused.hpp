@@ -68,100 +68,127 @@ __device__ __forceinline__ void issue_row(void* lds_base, const void* src_lane) 
   __shared__ __attribute__((aligned(1024))) char stage1[NST == 2 ? (BYTES) : 1024]
 
 // ---------------------------------------------------------------------------------------------
-// C[z][tb][s] = sum_{u < 32*tb, u > s} log2(1 - A[s,u])   (tb >= s/32).  grid (Lp/128, Zk), 4 waves.
+// The fused-path kernels tile with v_mfma_f32_16x16x32: a wave owns 16 stationary rows (keys in the
+// key-stationary kernels, queries in the query-stationary ones), which halves its operand strips and
+// accumulators so that two waves fit per SIMD; workgroups have 8 waves and share the staged tiles.
+// Carries are kept per 16-query tile:
+//   C[z][t16][s]    = sum_{u < 16*t16, u > s} log2(1 - A[s,u])        (t16 >= s/16 ... any t16 with 16*t16+15 >= s)
+//   Dsuf[z][t16][s] = sum_{t >= 16*(t16+1)} dBias[s,t]
 // ---------------------------------------------------------------------------------------------
+struct TrueC { static constexpr bool value = true; };
+struct FalseC { static constexpr bool value = false; };
+
+// grid (Lp/128, Zk), 8 waves; wave w owns keys 16*(8*bx+w)..+15 and sweeps the 32-query blocks from its own on.
 template <class T, int D, int NST>
-__global__ void __launch_bounds__(256) k_carry2(const T* __restrict__ Kp, const float* __restrict__ lsrc,
+__global__ void __launch_bounds__(512) k_carry2(const T* __restrict__ Kp, const float* __restrict__ lsrc,
                                                 const float* __restrict__ ldest, float* __restrict__ C, int Lp) {
   using TN = Tile<T, 32, D>;
-  constexpr int NQ = D / 16, LS = TN::STRIDE, SB = TN::BYTES + 1024;   // tile + [ldest of the block: 32 floats]
+  constexpr int NK = D / 32, LS = TN::STRIDE, SB = TN::BYTES + 1024;   // tile + [ldest of the block: 32 floats]
   UA_STAGES(SB);
-  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 31, hi = lane >> 5;
-  const int z = blockIdx.y, nT = Lp / 32, sb = 4 * blockIdx.x + w, first = 4 * blockIdx.x;
-  Stager<TN, 4> st;
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
+  const int z = blockIdx.y, nT = Lp / 32, nT16 = Lp / 16, sb16 = 8 * blockIdx.x + w, first = 4 * blockIdx.x;
+  const int spos = 16 * sb16 + col;
+  const GroupMasks gm = group_masks(lane);
+  Stager<TN, 8> st;
   st.init(w, lane, D * (long)sizeof(T), 32);
-  Frag<T> ks[NQ];
+  Frag<T> ks[NK];
   {
-    const T* krow = Kp + ((long)z * Lp + 32 * sb + col) * D + 8 * hi;
+    const T* krow = Kp + ((long)z * Lp + spos) * D + 8 * g;
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) ks[q] = ld8(krow + 16 * q);
+    for (int q = 0; q < NK; ++q) ks[q] = ld8(krow + 32 * q);
   }
-  const float la = lsrc[(long)z * Lp + 32 * sb + col];
+  const float la = lsrc[(long)z * Lp + spos];
   float carry = 0.f;
-  float* Cz = C + (long)z * nT * Lp;
+  float* Cz = C + (long)z * nT16 * Lp + spos;
   const T* Kz = Kp + (long)z * Lp * D;
 #define UA_ISSUE(s, base)                                                                   \
   {                                                                                         \
     st.issue((base), Kz + (long)32 * (first + (s)) * D, w);                                 \
     if (w == 0) issue_row((base) + TN::BYTES, ldest + (long)z * Lp + 32 * (first + (s)) + 4 * (lane & 7)); \
   }
-#define UA_COMPUTE(s, base)                                                                 \
+#define UA_COMPUTE_FAST(s, base) carry_step((s), (base), FalseC())
+#define UA_COMPUTE_SLOW(s, base)                                                            \
   {                                                                                         \
-    const int tb = first + (s);                                                             \
-    const T* sK = reinterpret_cast<const T*>(base);                                         \
-    if (tb >= sb) {                                                                         \
-      float lb[16];                                                                         \
-      load_t16(reinterpret_cast<const float*>((base) + TN::BYTES), hi, lb);                 \
-      f32x16 g = {0};                                                                       \
-      _Pragma("unroll") for (int q = 0; q < NQ; ++q) mma(g, ld8(sK + col * LS + 16 * q + 8 * hi), ks[q]); \
-      float tot = 0.f;                                                                      \
-      _Pragma("unroll") for (int v = 0; v < 16; ++v) {                                      \
-        float l2 = log2_one_minus(affinity(log2_relu(g[v]), la + lb[v]));                   \
-        if (tb == sb && t_of(v, hi) <= col) l2 = 0.f;                                       \
-        tot += l2;                                                                          \
-      }                                                                                     \
-      float lo, up;                                                                         \
-      swap32(tot, lo, up);                                                                  \
-      if (hi == 0) Cz[(long)tb * Lp + 32 * sb + col] = carry;                               \
-      carry += lo + up;                                                                     \
-    }                                                                                       \
+    if (first + (s) >= (sb16 >> 1)) carry_step((s), (base), TrueC());                       \
   }
-  UA_PIPELINE(nT - first, UA_ISSUE, UA_COMPUTE);
+  auto carry_step = [&] __device__ (int s, const char* base, auto masked_c) {
+    constexpr bool MASKED = decltype(masked_c)::value;
+    const int tb = first + s;
+    const T* sK = reinterpret_cast<const T*>(base);
+    const float* stats = reinterpret_cast<const float*>(base + TN::BYTES);
+    f32x4 x[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      f32x4 acc = {0, 0, 0, 0};
+#pragma unroll
+      for (int q = 0; q < NK; ++q) mma16(acc, ld8(sK + (16 * i + col) * LS + 32 * q + 8 * g), ks[q]);
+      const f32x4 lb = load_t4(stats + 16 * i, g);
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        float l2 = log2_one_minus(affinity(log2_relu(acc[v]), la + lb[v]));
+        if (MASKED) l2 = (32 * tb + 16 * i + 4 * g + v <= spos) ? 0.f : l2;
+        x[i][v] = l2;
+      }
+    }
+    float b0, a0, t0, b1, a1, t1;
+    group_scan((x[0][0] + x[0][1]) + (x[0][2] + x[0][3]), gm, b0, a0, t0);
+    group_scan((x[1][0] + x[1][1]) + (x[1][2] + x[1][3]), gm, b1, a1, t1);
+    if (g == 0) {
+      Cz[(long)(2 * tb) * Lp] = carry;
+      Cz[(long)(2 * tb + 1) * Lp] = carry + t0;
+    }
+    carry += t0 + t1;
+  };
+  {
+    const int total = nT - first, nslow = total < 4 ? total : 4;   // the first four blocks hold the diagonals
+    UA_PIPE_START(total, UA_ISSUE);
+    UA_PIPE_RANGE(0, nslow, total, UA_ISSUE, UA_COMPUTE_SLOW);
+    UA_PIPE_RANGE(nslow, total, total, UA_ISSUE, UA_COMPUTE_FAST);
+  }
 #undef UA_ISSUE
-#undef UA_COMPUTE
+#undef UA_COMPUTE_FAST
+#undef UA_COMPUTE_SLOW
 }
 
 // ---------------------------------------------------------------------------------------------
-// Fused forward.  grid (Lp/128, Zq); 4 waves; wave w owns queries 32*(4*jt+w)..+31; 64 keys per step.
+// Fused forward.  grid (Lp/128, Zq); 8 waves; wave w owns queries 16*(8*jt+w)..+15; 64 keys per step,
+// key tiles visited from the diagonal backwards.
 // ---------------------------------------------------------------------------------------------
 template <class T, int D, int NST>
-__global__ void __launch_bounds__(256) k_fwd_fused2(const T* __restrict__ Qp, const T* __restrict__ Kp,
+__global__ void __launch_bounds__(512) k_fwd_fused2(const T* __restrict__ Qp, const T* __restrict__ Kp,
                                                     const T* __restrict__ VT, const float* __restrict__ lsrc,
                                                     const float* __restrict__ ldest, const float* __restrict__ C,
                                                     T* __restrict__ O, float* __restrict__ lse, float* __restrict__ lse2,
                                                     int R, int L, int Lp, int d) {
   using TN = Tile<T, 32, D>;
   using TT = Tile<T, D, 32>;
-  constexpr int NQ = D / 16, NB = D / 32, LS = TN::STRIDE, TS = TT::STRIDE, PS = lds_stride<T>(64);
-  constexpr int TILES = 2 * TN::BYTES + 2 * TT::BYTES, SB = TILES + 4 * 1024;   // + per wave [C row: 64f][lsrc: 64f]
+  constexpr int NK = D / 32, ND = D / 16, LS = TN::STRIDE, TS = TT::STRIDE, PS = lds_stride<T>(64);
+  constexpr int TILES = 2 * TN::BYTES + 2 * TT::BYTES, SB = TILES + 8 * 1024;   // + per wave [C row: 64f][lsrc: 64f]
   UA_STAGES(SB);
-  __shared__ __attribute__((aligned(16))) T sPbuf[4 * 32 * PS];
-  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 31, hi = lane >> 5;
-  const int zq = blockIdx.y, zk = zq / R, nT = Lp / 32;
-  const int jt = gridDim.x - 1 - blockIdx.x, tb = 4 * jt + w;
-  T* sPw = sPbuf + w * 32 * PS;
-  const int pcol = perm16(col);
-  Stager<TN, 4> stN;
-  Stager<TT, 4> stT;
+  __shared__ __attribute__((aligned(16))) T sPbuf[8 * 16 * PS];
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
+  const int zq = blockIdx.y, zk = zq / R, nT16 = Lp / 16;
+  const int jt = gridDim.x - 1 - blockIdx.x, tq = 8 * jt + w;       // 16-query tile of this wave
+  T* sPw = sPbuf + w * 16 * PS;
+  const GroupMasks gm = group_masks(lane);
+  Stager<TN, 8> stN;
+  Stager<TT, 8> stT;
   stN.init(w, lane, D * (long)sizeof(T), 32);
   stT.init(w, lane, Lp * (long)sizeof(T), D);
 
-  Frag<T> qf[NQ], kf[NQ];
+  Frag<T> qf[NK], kf[NK];
   {
-    const T* qrow = Qp + ((long)zq * Lp + 32 * tb + col) * D + 8 * hi;
-    const T* krow = Kp + ((long)zk * Lp + 32 * tb + col) * D + 8 * hi;
+    const T* qrow = Qp + ((long)zq * Lp + 16 * tq + col) * D + 8 * g;
+    const T* krow = Kp + ((long)zk * Lp + 16 * tq + col) * D + 8 * g;
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) { qf[q] = ld8(qrow + 16 * q); kf[q] = ld8(krow + 16 * q); }
+    for (int q = 0; q < NK; ++q) { qf[q] = ld8(qrow + 32 * q); kf[q] = ld8(krow + 32 * q); }
   }
-  float lb[16];
-  load_t16(ldest + (long)zk * Lp + 32 * tb, hi, lb);
-  f32x16 o[NB];
+  const f32x4 lb = load_t4(ldest + (long)zk * Lp + 16 * tq, g);
+  f32x4 o[ND];
 #pragma unroll
-  for (int n = 0; n < NB; ++n) o[n] = (f32x16){0};
-  float m[16], ls[16];
-#pragma unroll
-  for (int v = 0; v < 16; ++v) { m[v] = -1.0e30f; ls[v] = 0.f; }
-  const float* Crow = C + ((long)zk * nT + tb) * Lp;
+  for (int n = 0; n < ND; ++n) o[n] = (f32x4){0, 0, 0, 0};
+  f32x4 m = {-1.0e30f, -1.0e30f, -1.0e30f, -1.0e30f}, ls = {0, 0, 0, 0};
+  const float* Crow = C + ((long)zk * nT16 + tq) * Lp;
   const float* lsz = lsrc + (long)zk * Lp;
   const T* Kz = Kp + (long)zk * Lp * D;
   const T* Vz = VT + (long)zk * D * Lp;
@@ -176,99 +203,103 @@ __global__ void __launch_bounds__(256) k_fwd_fused2(const T* __restrict__ Qp, co
     stT.issue((base) + 2 * TN::BYTES + TT::BYTES, Vz + 64 * kt_ + 32, w);                   \
     issue_row((base) + TILES + w * 1024, ((lane & 16) ? lsz : Crow) + 64 * kt_ + 4 * (lane & 15)); \
   }
-#define UA_COMPUTE(s, base)                                                                 \
-  {                                                                                         \
-    const int kt_ = n_kt - 1 - (s);                                                         \
-    fwd_tile(kt_, base);                                                                    \
-  }
-  auto fwd_tile = [&] __device__ (int kt, const char* base) {
-    f32x16 s2[2];
+#define UA_COMPUTE_FAST(s, base) fwd_tile(n_kt - 1 - (s), (base), FalseC())
+#define UA_COMPUTE_SLOW(s, base) fwd_tile(n_kt - 1 - (s), (base), TrueC())
+  auto fwd_tile = [&] __device__ (int kt, const char* base, auto masked_c) {
+    constexpr bool MASKED = decltype(masked_c)::value;
+    const float* stats = reinterpret_cast<const float*>(base + TILES + w * 1024);
+    f32x4 s2[4];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int sbk = 2 * kt + j;
-      const T* sK = reinterpret_cast<const T*>(base + j * TN::BYTES);
-      if (sbk <= tb) {
-        const float* stats = reinterpret_cast<const float*>(base + TILES + w * 1024);
-        const float c = stats[32 * j + col];
-        const float la = stats[64 + 32 * j + col];
-        f32x16 g = {0}, sc = {0};
+    for (int j = 0; j < 4; ++j) {
+      const int sbk = 4 * kt + j;                      // 16-key tile
+      const T* sK = reinterpret_cast<const T*>(base + (j >> 1) * TN::BYTES) + (16 * (j & 1) + col) * LS + 8 * g;
+      if (!MASKED || sbk <= tq) {
+        const float c = stats[16 * j + col];
+        const float la = stats[64 + 16 * j + col];
+        f32x4 gt = {0, 0, 0, 0}, sc = {0, 0, 0, 0};
 #pragma unroll
-        for (int q = 0; q < NQ; ++q) {
-          const Frag<T> kb = ld8(sK + col * LS + 16 * q + 8 * hi);
-          mma(g, kf[q], kb);
-          mma(sc, qf[q], kb);
+        for (int q = 0; q < NK; ++q) {
+          const Frag<T> kb = ld8(sK + 32 * q);
+          mma16(gt, kf[q], kb);
+          mma16(sc, qf[q], kb);
         }
-        const bool diag = (sbk == tb);
+        const bool diag = MASKED && (sbk == tq);
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const float l2 = log2_one_minus(affinity(log2_relu(g[v]), la + lb[v]));
-          g[v] = (diag && t_of(v, hi) <= col) ? 0.f : l2;
+        for (int v = 0; v < 4; ++v) {
+          const float l2 = log2_one_minus(affinity(log2_relu(gt[v]), la + lb[v]));
+          gt[v] = (MASKED && diag && 4 * g + v <= col) ? 0.f : l2;
         }
-        block_prefix(g, hi);
+        // inclusive prefix over the 16 queries of this wave
+        gt[1] += gt[0]; gt[2] += gt[1]; gt[3] += gt[2];
+        float before, after, tot;
+        group_scan(gt[3], gm, before, after, tot);
+        before += c;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const float x = __builtin_fmaf(sc[v], kLog2e, g[v] + c);
-          s2[j][v] = (diag && t_of(v, hi) < col) ? -1.0e30f : x;
+        for (int v = 0; v < 4; ++v) {
+          const float x = __builtin_fmaf(sc[v], kLog2e, gt[v] + before);
+          s2[j][v] = (MASKED && diag && 4 * g + v < col) ? -1.0e30f : x;
         }
       } else {
-#pragma unroll
-        for (int v = 0; v < 16; ++v) s2[j][v] = -1.0e30f;
+        s2[j] = (f32x4){-1.0e30f, -1.0e30f, -1.0e30f, -1.0e30f};
       }
     }
     // online softmax: rescale only when some query of this wave raises its maximum
-    float mx[16];
+    f32x4 mx;
     bool grow = false;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      mx[v] = allmax32(fmaxf(s2[0][v], s2[1][v]));
+    for (int v = 0; v < 4; ++v) {
+      mx[v] = allmax16(fmaxf(fmaxf(s2[0][v], s2[1][v]), fmaxf(s2[2][v], s2[3][v])));
       grow |= (mx[v] > m[v]);
     }
     if (__builtin_amdgcn_ballot_w64(grow) != 0) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
+      for (int v = 0; v < 4; ++v) {
         const float mn = fmaxf(m[v], mx[v]);
         const float alpha = __builtin_amdgcn_exp2f(m[v] - mn);
         m[v] = mn;
         ls[v] *= alpha;
 #pragma unroll
-        for (int n = 0; n < NB; ++n) o[n][v] *= alpha;
+        for (int n = 0; n < ND; ++n) o[n][v] *= alpha;
       }
     }
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
+    for (int j = 0; j < 4; ++j) {
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int v = 0; v < 4; ++v) {
         const float p = __builtin_amdgcn_exp2f(s2[j][v] - m[v]);
         ls[v] += p;
-        sPw[t_of(v, hi) * PS + 32 * j + pcol] = cvt<T>(p);
+        sPw[(4 * g + v) * PS + 16 * j + col] = cvt<T>(p);
       }
     }
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      if (2 * kt + j <= tb) {
-        const T* sV = reinterpret_cast<const T*>(base + 2 * TN::BYTES + j * TT::BYTES);
+    for (int kq = 0; kq < 2; ++kq) {                   // 32 keys per k-step
+      if (!MASKED || 4 * kt + 2 * kq <= tq) {
+        const T* sV = reinterpret_cast<const T*>(base + 2 * TN::BYTES + kq * TT::BYTES);
+        const Frag<T> pa = ld8(sPw + col * PS + 32 * kq + 8 * g);
 #pragma unroll
-        for (int kq = 0; kq < 2; ++kq) {
-          const Frag<T> pa = ld8(sPw + col * PS + 32 * j + 16 * kq + 8 * hi);
-#pragma unroll
-          for (int n = 0; n < NB; ++n) mma(o[n], pa, ld8(sV + (32 * n + col) * TS + 16 * kq + 8 * hi));
-        }
+        for (int n = 0; n < ND; ++n) mma16(o[n], pa, ld8(sV + (16 * n + col) * TS + 8 * g));
       }
     }
   };
-  UA_PIPELINE(n_kt, UA_ISSUE, UA_COMPUTE);
+  {
+    // the first two key tiles (visited first) hold the diagonal blocks of the eight waves
+    UA_PIPE_START(n_kt, UA_ISSUE);
+    UA_PIPE_RANGE(0, 2, n_kt, UA_ISSUE, UA_COMPUTE_SLOW);
+    UA_PIPE_RANGE(2, n_kt, n_kt, UA_ISSUE, UA_COMPUTE_FAST);
+  }
 #undef UA_ISSUE
-#undef UA_COMPUTE
+#undef UA_COMPUTE_FAST
+#undef UA_COMPUTE_SLOW
   // epilogue
 #pragma unroll
-  for (int v = 0; v < 16; ++v) {
-    const float tot = allsum32(ls[v]);
+  for (int v = 0; v < 4; ++v) {
+    const float tot = allsum16(ls[v]);
     const float inv = 1.0f / tot;
-    const int t = 32 * tb + t_of(v, hi);
+    const int t = 16 * tq + 4 * g + v;
     if (t < L) {
 #pragma unroll
-      for (int n = 0; n < NB; ++n) {
-        const int dd = 32 * n + col;
+      for (int n = 0; n < ND; ++n) {
+        const int dd = 16 * n + col;
         if (dd < d) O[((long)zq * L + t) * d + dd] = cvt<T>(o[n][v] * inv);
       }
     }
@@ -281,49 +312,46 @@ __global__ void __launch_bounds__(256) k_fwd_fused2(const T* __restrict__ Qp, co
 }
 
 // ---------------------------------------------------------------------------------------------
-// Key-stationary backward (fused mode).  grid (Lp/128, Zk); 4 waves; wave w owns keys 128g+32w..+31,
-// sweeps query blocks from the last one down to its own; one (query block, query group) per step.
+// Key-stationary backward (fused mode).  grid (Lp/128, Zk); 8 waves; wave w owns keys 128g+16w..+15 and
+// sweeps the 32-query blocks from the last one down to its own; one (query block, query group) per step.
 // MR = more than one query group per kv head (the decay state of a query block then lives across steps).
 // ---------------------------------------------------------------------------------------------
-struct TrueC { static constexpr bool value = true; };
-struct FalseC { static constexpr bool value = false; };
-
 template <class T, int D, int NST, bool MR>
-__global__ void __launch_bounds__(256) k_bwd_keys2(BwdArgs<T> a) {
+__global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   using TN = Tile<T, 32, D>;
   using TT = Tile<T, D, 32>;
-  constexpr int NQ = D / 16, NB = D / 32, LS = TN::STRIDE, TS = TT::STRIDE;
+  constexpr int NK = D / 32, ND = D / 16, LS = TN::STRIDE, TS = TT::STRIDE;
   constexpr int TILES = 3 * TN::BYTES + 3 * TT::BYTES, SB = TILES + 1024;
-  UA_STAGES(SB);
   // stats row of a stage: [lse2: 32f][delta: 32f][ldest: 32f][unused: 32f][forward carries of the 128 keys: 128f]
-  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 31, hi = lane >> 5;
-  const int zk = blockIdx.y, Lp = a.Lp, L = a.L, nT = Lp / 32, R = MR ? a.R : 1;
-  const int g = gridDim.x - 1 - blockIdx.x, sb = 4 * g + w, spos = 32 * sb + col;
-  const int nTr = (L + 31) / 32, first = 4 * g;
+  UA_STAGES(SB);
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
+  const int zk = blockIdx.y, Lp = a.Lp, L = a.L, nT16 = Lp / 16, R = MR ? a.R : 1;
+  const int kg = gridDim.x - 1 - blockIdx.x, sb16 = 8 * kg + w, spos = 16 * sb16 + col;
+  const int nTr = (L + 31) / 32, first = 4 * kg;
   if (first >= nTr) return;                      // every key of this workgroup is padding
-  Stager<TN, 4> stN;
-  Stager<TT, 4> stT;
+  const GroupMasks gm = group_masks(lane);
+  Stager<TN, 8> stN;
+  Stager<TT, 8> stT;
   stN.init(w, lane, D * (long)sizeof(T), 32);
   stT.init(w, lane, Lp * (long)sizeof(T), D);
 
-  Frag<T> kp[NQ], vf[NQ];
+  Frag<T> kp[NK], vf[NK];
   {
-    const long ro = ((long)zk * Lp + spos) * D + 8 * hi;
+    const long ro = ((long)zk * Lp + spos) * D + 8 * g;
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) { kp[q] = ld8(a.Kp + ro + 16 * q); vf[q] = ld8(a.Vp + ro + 16 * q); }
+    for (int q = 0; q < NK; ++q) { kp[q] = ld8(a.Kp + ro + 32 * q); vf[q] = ld8(a.Vp + ro + 32 * q); }
   }
   const float la = a.lsrc[(long)zk * Lp + spos];
-  f32x16 dVt[NB], dKt[NB];
+  f32x4 dVt[ND], dKt[ND];
 #pragma unroll
-  for (int n = 0; n < NB; ++n) { dVt[n] = (f32x16){0}; dKt[n] = (f32x16){0}; }
+  for (int n = 0; n < ND; ++n) { dVt[n] = (f32x4){0, 0, 0, 0}; dKt[n] = (f32x4){0, 0, 0, 0}; }
   float dsrc_acc = 0.f, dcar = 0.f;
-  f32x16 aff_s, bias_s, gk_s, dB_s;              // state of the current query block (used when MR)
-  float lab_s[16];
+  f32x4 aff_s[2], bias_s[2], gk_s[2], dB_s[2], lab_s[2];     // state of the current query block (used when MR)
   const T* Kz = a.Kp + (long)zk * Lp * D;
   const T* KTz = a.KT + (long)zk * D * Lp;
   const float* ldz = a.ldest + (long)zk * Lp;
-  const float* Cz = a.C + (long)zk * nT * Lp + 128 * g;
-  float* Dz = a.Dsuf + (long)zk * nT * Lp + spos;
+  const float* Cz = a.C + (long)zk * nT16 * Lp + 128 * kg;
+  float* Dz = a.Dsuf + (long)zk * nT16 * Lp + spos;
 
 #define UA_ISSUE(s, base)                                                                   \
   {                                                                                         \
@@ -341,7 +369,7 @@ __global__ void __launch_bounds__(256) k_bwd_keys2(BwdArgs<T> a) {
       if (lane < 8) src_ = a.lse2 + zq_ * Lp + 32 * tb_ + 4 * lane;                         \
       else if (lane < 16) src_ = a.delta + zq_ * Lp + 32 * tb_ + 4 * (lane - 8);            \
       else if (lane < 32) src_ = ldz + 32 * tb_ + 4 * (lane & 7);                           \
-      else src_ = Cz + (long)tb_ * Lp + 4 * (lane - 32);                                    \
+      else src_ = Cz + (long)(2 * tb_) * Lp + 4 * (lane - 32);                              \
       issue_row((base) + TILES, src_);                                                      \
     }                                                                                       \
   }
@@ -349,11 +377,11 @@ __global__ void __launch_bounds__(256) k_bwd_keys2(BwdArgs<T> a) {
 #define UA_COMPUTE_SLOW(s, base)                                                            \
   {                                                                                         \
     const int tb_ = nTr - 1 - (s) / R;                                                      \
-    if (tb_ >= sb) bwd_step((s), (base), TrueC(), tb_ == sb);                               \
+    if (tb_ >= (sb16 >> 1)) bwd_step((s), (base), TrueC(), tb_ == (sb16 >> 1));             \
   }
-  // MASKED: the step may be this wave's diagonal block (run-time flag diag); otherwise every pair is visible
+  // MASKED: the step may be the query block that holds this wave's own keys (run-time flag diag)
   auto bwd_step = [&] __device__ (int s, const char* base, auto masked_c, const bool diag) {
-    constexpr bool DIAG = decltype(masked_c)::value;
+    constexpr bool MASKED = decltype(masked_c)::value;
     const int tb = nTr - 1 - s / R, r = s % R;
     const T* sKt = reinterpret_cast<const T*>(base);
     const T* sQ = reinterpret_cast<const T*>(base + TN::BYTES);
@@ -362,87 +390,93 @@ __global__ void __launch_bounds__(256) k_bwd_keys2(BwdArgs<T> a) {
     const T* sQT = reinterpret_cast<const T*>(base + 3 * TN::BYTES + TT::BYTES);
     const T* sdOT = reinterpret_cast<const T*>(base + 3 * TN::BYTES + 2 * TT::BYTES);
     const float* stats = reinterpret_cast<const float*>(base + TILES);
-    f32x16 aff_l, bias_l, gk_l, dB_l;
-    float lab_l[16];
-    f32x16& aff = MR ? aff_s : aff_l;
-    f32x16& bias = MR ? bias_s : bias_l;
-    f32x16& gk = MR ? gk_s : gk_l;
-    f32x16& dB = MR ? dB_s : dB_l;
-    float (&lab)[16] = MR ? lab_s : lab_l;
+    f32x4 aff_l[2], bias_l[2], gk_l[2], dB_l[2], lab_l[2];
+    f32x4 (&aff)[2] = MR ? aff_s : aff_l;
+    f32x4 (&bias)[2] = MR ? bias_s : bias_l;
+    f32x4 (&gk)[2] = MR ? gk_s : gk_l;
+    f32x4 (&dB)[2] = MR ? dB_s : dB_l;
+    f32x4 (&lab)[2] = MR ? lab_s : lab_l;
+    const int tl0 = 32 * tb + 4 * g - spos;        // query position minus key position for (tile 0, v = 0)
     if (!MR || r == 0) {
-      const float cin = stats[128 + 32 * w + col];
-      load_t16(stats + 64, hi, lab);
-      f32x16 acc = {0};
+      const float cin = stats[128 + 16 * w + col];
 #pragma unroll
-      for (int q = 0; q < NQ; ++q) mma(acc, ld8(sKt + col * LS + 16 * q + 8 * hi), kp[q]);
+      for (int i = 0; i < 2; ++i) {
+        f32x4 acc = {0, 0, 0, 0};
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        lab[v] += la;
-        gk[v] = log2_relu(acc[v]);
-        aff[v] = affinity(gk[v], lab[v]);
-        const float l2 = log2_one_minus(aff[v]);
-        bias[v] = (DIAG && diag && t_of(v, hi) <= col) ? 0.f : l2;
+        for (int q = 0; q < NK; ++q) mma16(acc, ld8(sKt + (16 * i + col) * LS + 32 * q + 8 * g), kp[q]);
+        lab[i] = load_t4(stats + 64 + 16 * i, g);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          lab[i][v] += la;
+          gk[i][v] = log2_relu(acc[v]);
+          aff[i][v] = affinity(gk[i][v], lab[i][v]);
+          const float l2 = log2_one_minus(aff[i][v]);
+          bias[i][v] = (MASKED && diag && tl0 + 16 * i + v <= 0) ? 0.f : l2;
+        }
       }
-      block_prefix(bias, hi);
+      prefix32(bias[0], bias[1], gm);
 #pragma unroll
-      for (int v = 0; v < 16; ++v) { bias[v] += cin; if (MR) dB[v] = 0.f; }
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) { bias[i][v] += cin; if (MR) dB[i][v] = 0.f; }
     }
     {
-      f32x16 sc = {0}, dP = {0};
+      f32x4 P[2], dS[2];
 #pragma unroll
-      for (int q = 0; q < NQ; ++q) mma(sc, ld8(sQ + col * LS + 16 * q + 8 * hi), kp[q]);
+      for (int i = 0; i < 2; ++i) {
+        f32x4 sc = {0, 0, 0, 0}, dP = {0, 0, 0, 0};
 #pragma unroll
-      for (int q = 0; q < NQ; ++q) mma(dP, ld8(sdO + col * LS + 16 * q + 8 * hi), vf[q]);
-      float l2t[16], dlt[16];
-      load_t16(stats, hi, l2t);
-      load_t16(stats + 32, hi, dlt);
+        for (int q = 0; q < NK; ++q) mma16(sc, ld8(sQ + (16 * i + col) * LS + 32 * q + 8 * g), kp[q]);
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[v], kLog2e, bias[v]) - l2t[v]);
-        if (DIAG) p = (diag && t_of(v, hi) < col) ? 0.f : p;
-        sc[v] = p;
-        dP[v] = p * (dP[v] - dlt[v]);
+        for (int q = 0; q < NK; ++q) mma16(dP, ld8(sdO + (16 * i + col) * LS + 32 * q + 8 * g), vf[q]);
+        const f32x4 l2t = load_t4(stats + 16 * i, g), dlt = load_t4(stats + 32 + 16 * i, g);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[v], kLog2e, bias[i][v]) - l2t[v]);
+          if (MASKED) p = (diag && tl0 + 16 * i + v < 0) ? 0.f : p;
+          P[i][v] = p;
+          dS[i][v] = p * (dP[v] - dlt[v]);
+        }
       }
+      const Frag<T> bp = as_operand16<T>(P[0], P[1]), bs = as_operand16<T>(dS[0], dS[1]);
 #pragma unroll
-      for (int q2 = 0; q2 < 2; ++q2) {
-        const Frag<T> bp = as_operand<T>(sc, q2);
+      for (int n = 0; n < ND; ++n) mma16(dVt[n], ld8(sdOT + (16 * n + col) * TS + 8 * g), bp);
 #pragma unroll
-        for (int n = 0; n < NB; ++n) mma(dVt[n], ld8(sdOT + (32 * n + col) * TS + 16 * q2 + 8 * hi), bp);
-      }
+      for (int n = 0; n < ND; ++n) mma16(dKt[n], ld8(sQT + (16 * n + col) * TS + 8 * g), bs);
 #pragma unroll
-      for (int q2 = 0; q2 < 2; ++q2) {
-        const Frag<T> bs = as_operand<T>(dP, q2);
+      for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int n = 0; n < NB; ++n) mma(dKt[n], ld8(sQT + (32 * n + col) * TS + 16 * q2 + 8 * hi), bs);
-      }
-#pragma unroll
-      for (int v = 0; v < 16; ++v) dB[v] = MR ? dB[v] + dP[v] : dP[v];
+        for (int v = 0; v < 4; ++v) dB[i][v] = MR ? dB[i][v] + dS[i][v] : dS[i][v];
     }
     if (!MR || r == R - 1) {
-      if (hi == 0) Dz[(long)tb * Lp] = dcar;
-      const float tot = block_suffix(dB, hi);
+      float t1;
+      const float tot = suffix32(dB[0], dB[1], gm, t1);
+      if (g == 0) {
+        Dz[(long)(2 * tb + 1) * Lp] = dcar;
+        Dz[(long)(2 * tb) * Lp] = dcar + t1;
+      }
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        float dl = dB[v] + dcar;
-        if (DIAG) dl = (diag && t_of(v, hi) <= col) ? 0.f : dl;
-        const float av = aff[v];
-        const float den = __builtin_amdgcn_fmed3f(av, kAMinBwd, kAMax) - 1.0f;
-        const float dA = (av <= kAMax) ? dl * __builtin_amdgcn_rcpf(den) : 0.f;
-        dsrc_acc = __builtin_fmaf(dA, av, dsrc_acc);
-        const float f = (2.0f / 3.0f) * __builtin_amdgcn_exp2f(__builtin_fmaf(gk[v], -1.0f / 3.0f, lab[v]));
-        dB[v] = (gk[v] > -1.0e30f) ? dA * f : 0.f;
+      for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          float dl = dB[i][v] + dcar;
+          if (MASKED) dl = (diag && tl0 + 16 * i + v <= 0) ? 0.f : dl;
+          const float av = aff[i][v];
+          const float den = __builtin_amdgcn_fmed3f(av, kAMinBwd, kAMax) - 1.0f;
+          const float dA = (av <= kAMax) ? dl * __builtin_amdgcn_rcpf(den) : 0.f;
+          dsrc_acc = __builtin_fmaf(dA, av, dsrc_acc);
+          const float f = (2.0f / 3.0f) * __builtin_amdgcn_exp2f(__builtin_fmaf(gk[i][v], -1.0f / 3.0f, lab[i][v]));
+          dB[i][v] = (gk[i][v] > -1.0e30f) ? dA * f : 0.f;
+        }
       }
       dcar += tot;
+      const Frag<T> b = as_operand16<T>(dB[0], dB[1]);
 #pragma unroll
-      for (int q2 = 0; q2 < 2; ++q2) {
-        const Frag<T> b = as_operand<T>(dB, q2);
-#pragma unroll
-        for (int n = 0; n < NB; ++n) mma(dKt[n], ld8(sKT + (32 * n + col) * TS + 16 * q2 + 8 * hi), b);
-      }
+      for (int n = 0; n < ND; ++n) mma16(dKt[n], ld8(sKT + (16 * n + col) * TS + 8 * g), b);
     }
   };
   {
-    // the last four query blocks of the sweep hold the diagonal blocks of the four waves
+    // the last four query blocks of the sweep hold the diagonal blocks of the eight waves
     const int nblk = nTr - first, total = nblk * R, nfast = ((nblk > 4 ? nblk - 4 : 0) * R) & ~1;
     UA_PIPE_START(total, UA_ISSUE);
     UA_PIPE_RANGE(0, nfast, total, UA_ISSUE, UA_COMPUTE_FAST);
@@ -452,77 +486,78 @@ __global__ void __launch_bounds__(256) k_bwd_keys2(BwdArgs<T> a) {
 #undef UA_COMPUTE_FAST
 #undef UA_COMPUTE_SLOW
   // epilogue
-  float lo, up;
-  swap32(dsrc_acc, lo, up);
-  if (hi == 0) a.dsrc_raw[(long)zk * Lp + spos] = lo + up;
+  {
+    float b, af, tot;
+    group_scan(dsrc_acc, gm, b, af, tot);
+    if (g == 0) a.dsrc_raw[(long)zk * Lp + spos] = tot;
+  }
 #pragma unroll
-  for (int n = 0; n < NB; ++n) {
-#pragma unroll
-    for (int gq = 0; gq < 4; ++gq) {
-      const long o = ((long)zk * Lp + spos) * D + 32 * n + 8 * gq + 4 * hi;
-      *reinterpret_cast<float4*>(a.dVrow + o) = make_float4(dVt[n][4 * gq], dVt[n][4 * gq + 1], dVt[n][4 * gq + 2], dVt[n][4 * gq + 3]);
-      *reinterpret_cast<float4*>(a.dKrow + o) = make_float4(dKt[n][4 * gq], dKt[n][4 * gq + 1], dKt[n][4 * gq + 2], dKt[n][4 * gq + 3]);
-    }
+  for (int n = 0; n < ND; ++n) {
+    const long o = ((long)zk * Lp + spos) * D + 16 * n + 4 * g;
+    *reinterpret_cast<float4*>(a.dVrow + o) = make_float4(dVt[n][0], dVt[n][1], dVt[n][2], dVt[n][3]);
+    *reinterpret_cast<float4*>(a.dKrow + o) = make_float4(dKt[n][0], dKt[n][1], dKt[n][2], dKt[n][3]);
   }
 }
 
 // ---------------------------------------------------------------------------------------------
 // Query-stationary backward (fused mode): dQ and the column side of dK, no atomics.
-// grid (Lp/128, Zk); 4 waves; wave w owns queries 32*(4*jt+w)..+31; 64 keys per step.
+// grid (Lp/128, Zk); 8 waves; wave w owns queries 16*(8*jt+w)..+15; 64 keys per step.
+//   dQ[t,:] += sum_s dS[s,t] k_s        dkcol[u,:] += sum_s dg[s,u] k_s
+// dS^T and dg^T pass through a wave-private LDS tile to become A operands.  With r query groups the sweep is
+// repeated per group; dg is linear in dBias, so the groups' contributions to dkcol add up (the cross-tile
+// suffix carry is added in the first group only).
 // ---------------------------------------------------------------------------------------------
 template <class T, int D, int NST>
-__global__ void __launch_bounds__(256) k_bwd_queries2(BwdArgs<T> a, T* __restrict__ dq, int d) {
+__global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restrict__ dq, int d) {
   using TN = Tile<T, 32, D>;
   using TT = Tile<T, D, 32>;
-  constexpr int NQ = D / 16, NB = D / 32, LS = TN::STRIDE, TS = TT::STRIDE, SS = lds_stride<T>(32);
-  constexpr int TILES = 4 * TN::BYTES + 2 * TT::BYTES, SB = TILES + 4 * 1024;   // + per wave [C: 64f][lsrc: 64f][Dsuf: 64f]
+  constexpr int NK = D / 32, ND = D / 16, LS = TN::STRIDE, TS = TT::STRIDE, XS = lds_stride<T>(64);
+  constexpr int TILES = 4 * TN::BYTES + 2 * TT::BYTES, SB = TILES + 8 * 1024;   // + per wave [C: 64f][lsrc: 64f][Dsuf: 64f]
   UA_STAGES(SB);
-  __shared__ __attribute__((aligned(16))) T sXbuf[4 * 2 * 32 * SS];
-  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 31, hi = lane >> 5;
-  const int zk = blockIdx.y, Lp = a.Lp, L = a.L, nT = Lp / 32, R = a.R;
-  const int jt = gridDim.x - 1 - blockIdx.x, tb = 4 * jt + w;
-  T* sXs = sXbuf + w * 2 * 32 * SS;
-  T* sXg = sXs + 32 * SS;
-  const int pcol = perm16(col);
-  Stager<TN, 4> stN;
-  Stager<TT, 4> stT;
+  __shared__ __attribute__((aligned(16))) T sXbuf[8 * 16 * XS];
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
+  const int zk = blockIdx.y, Lp = a.Lp, L = a.L, nT16 = Lp / 16, R = a.R;
+  const int jt = gridDim.x - 1 - blockIdx.x, tq = 8 * jt + w;
+  T* sX = sXbuf + w * 16 * XS;
+  const GroupMasks gm = group_masks(lane);
+  Stager<TN, 8> stN;
+  Stager<TT, 8> stT;
   stN.init(w, lane, D * (long)sizeof(T), 32);
   stT.init(w, lane, Lp * (long)sizeof(T), D);
 
-  Frag<T> kt[NQ];
+  Frag<T> kt[NK];
   {
-    const T* krow = a.Kp + ((long)zk * Lp + 32 * tb + col) * D + 8 * hi;
+    const T* krow = a.Kp + ((long)zk * Lp + 16 * tq + col) * D + 8 * g;
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) kt[q] = ld8(krow + 16 * q);
+    for (int q = 0; q < NK; ++q) kt[q] = ld8(krow + 32 * q);
   }
-  float lb[16];
-  load_t16(a.ldest + (long)zk * Lp + 32 * tb, hi, lb);
-  f32x16 dKc[NB];
+  const f32x4 lb = load_t4(a.ldest + (long)zk * Lp + 16 * tq, g);
+  f32x4 dKc[ND];
 #pragma unroll
-  for (int n = 0; n < NB; ++n) dKc[n] = (f32x16){0};
-  const float* Crow = a.C + ((long)zk * nT + tb) * Lp;
-  const float* Drow = a.Dsuf + ((long)zk * nT + tb) * Lp;
+  for (int n = 0; n < ND; ++n) dKc[n] = (f32x4){0, 0, 0, 0};
+  const float* Crow = a.C + ((long)zk * nT16 + tq) * Lp;
+  const float* Drow = a.Dsuf + ((long)zk * nT16 + tq) * Lp;
   const float* lsz = a.lsrc + (long)zk * Lp;
   const T* Kz = a.Kp + (long)zk * Lp * D;
   const T* Vz = a.Vp + (long)zk * Lp * D;
   const T* KTz = a.KT + (long)zk * D * Lp;
   const int n_kt = 2 * jt + 2;
+  // column of key (16*(j&1) + col) inside its 32-key group of the transposed key tile
+  const int pc0 = perm32(col), pc1 = perm32(16 + col);
 
   for (int r = 0; r < R; ++r) {
     const long zq = (long)zk * R + r;
-    Frag<T> qt[NQ], gt[NQ];
+    Frag<T> qt[NK], gt[NK];
     {
-      const T* qrow = a.Qp + (zq * Lp + 32 * tb + col) * D + 8 * hi;
-      const T* grow = a.dOp + (zq * Lp + 32 * tb + col) * D + 8 * hi;
+      const T* qrow = a.Qp + (zq * Lp + 16 * tq + col) * D + 8 * g;
+      const T* grow = a.dOp + (zq * Lp + 16 * tq + col) * D + 8 * g;
 #pragma unroll
-      for (int q = 0; q < NQ; ++q) { qt[q] = ld8(qrow + 16 * q); gt[q] = ld8(grow + 16 * q); }
+      for (int q = 0; q < NK; ++q) { qt[q] = ld8(qrow + 32 * q); gt[q] = ld8(grow + 32 * q); }
     }
-    float l2t[16], dlt[16];
-    load_t16(a.lse2 + zq * Lp + 32 * tb, hi, l2t);
-    load_t16(a.delta + zq * Lp + 32 * tb, hi, dlt);
-    f32x16 dQ[NB];
+    const f32x4 l2t = load_t4(a.lse2 + zq * Lp + 16 * tq, g), dlt = load_t4(a.delta + zq * Lp + 16 * tq, g);
+    f32x4 dQ[ND];
 #pragma unroll
-    for (int n = 0; n < NB; ++n) dQ[n] = (f32x16){0};
+    for (int n = 0; n < ND; ++n) dQ[n] = (f32x4){0, 0, 0, 0};
 
 #define UA_ISSUE(s, base)                                                                   \
   {                                                                                         \
@@ -536,91 +571,117 @@ __global__ void __launch_bounds__(256) k_bwd_queries2(BwdArgs<T> a, T* __restric
     issue_row((base) + TILES + w * 1024,                                                    \
               (lane < 16 ? Crow : (lane < 32 ? lsz : Drow)) + k0_ + 4 * (lane & 15));       \
   }
-#define UA_COMPUTE(s, base) bq_step((s), (base))
-    auto bq_step = [&] __device__ (int kti, const char* base) {
+#define UA_COMPUTE_FAST(s, base) bq_step((s), (base), FalseC())
+#define UA_COMPUTE_SLOW(s, base) bq_step((s), (base), TrueC())
+    auto bq_step = [&] __device__ (int kti, const char* base, auto masked_c) {
+      constexpr bool MASKED = decltype(masked_c)::value;
+      const float* stats = reinterpret_cast<const float*>(base + TILES + w * 1024);
+      // the 64 keys of the step are handled as two halves of 32 (= one contraction step of the column products);
+      // sX holds [16 queries][dS of the half: 32][dg of the half: 32]
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const int sbk = 2 * kti + j;
-        if (sbk > tb) continue;
-        const T* sK = reinterpret_cast<const T*>(base + j * TN::BYTES);
-        const T* sV = reinterpret_cast<const T*>(base + (2 + j) * TN::BYTES);
-        const T* sKT = reinterpret_cast<const T*>(base + 4 * TN::BYTES + j * TT::BYTES);
-        const bool diag = (sbk == tb);
-        const float* stats = reinterpret_cast<const float*>(base + TILES + w * 1024);
-        const float cin = stats[32 * j + col];
-        const float la = stats[64 + 32 * j + col];
-        const float din = (r == 0) ? stats[128 + 32 * j + col] : 0.f;
-        f32x16 gk = {0}, sc = {0}, dP = {0};
+      for (int kq = 0; kq < 2; ++kq) {
+        if (MASKED && 4 * kti + 2 * kq > tq) continue;     // wave-uniform: the whole half lies after this wave's queries
 #pragma unroll
-        for (int q = 0; q < NQ; ++q) {
-          const Frag<T> kb = ld8(sK + col * LS + 16 * q + 8 * hi);
-          mma(gk, kt[q], kb);
-          mma(sc, qt[q], kb);
-          mma(dP, gt[q], ld8(sV + col * LS + 16 * q + 8 * hi));
-        }
-        f32x16 aff, x;
-        float lab[16];
+        for (int jj = 0; jj < 2; ++jj) {
+          const int j = 2 * kq + jj, sbk = 4 * kti + j;
+          const bool live = !MASKED || sbk <= tq;
+          const bool diag = MASKED && (sbk == tq);
+          f32x4 dS = {0, 0, 0, 0}, dg = {0, 0, 0, 0};
+          if (live) {
+            const T* sK = reinterpret_cast<const T*>(base + kq * TN::BYTES) + (16 * jj + col) * LS + 8 * g;
+            const T* sV = reinterpret_cast<const T*>(base + (2 + kq) * TN::BYTES) + (16 * jj + col) * LS + 8 * g;
+            const float cin = stats[16 * j + col];
+            const float la = stats[64 + 16 * j + col];
+            const float din = (r == 0) ? stats[128 + 16 * j + col] : 0.f;
+            f32x4 acc = {0, 0, 0, 0}, sc = {0, 0, 0, 0}, dP = {0, 0, 0, 0};
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          lab[v] = la + lb[v];
-          gk[v] = log2_relu(gk[v]);
-          aff[v] = affinity(gk[v], lab[v]);
-          const float l2 = log2_one_minus(aff[v]);
-          x[v] = (diag && t_of(v, hi) <= col) ? 0.f : l2;
-        }
-        block_prefix(x, hi);
-        f32x16 dS;
+            for (int q = 0; q < NK; ++q) {
+              const Frag<T> kb = ld8(sK + 32 * q);
+              mma16(acc, kt[q], kb);
+              mma16(sc, qt[q], kb);
+              mma16(dP, gt[q], ld8(sV + 32 * q));
+            }
+            f32x4 x, gk, aff, lab;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[v], kLog2e, x[v] + cin) - l2t[v]);
-          p = (diag && t_of(v, hi) < col) ? 0.f : p;
-          dS[v] = p * (dP[v] - dlt[v]);
-          sXs[t_of(v, hi) * SS + pcol] = cvt<T>(dS[v]);
-        }
-        block_suffix(dS, hi);
+            for (int v = 0; v < 4; ++v) {
+              lab[v] = la + lb[v];
+              gk[v] = log2_relu(acc[v]);
+              aff[v] = affinity(gk[v], lab[v]);
+              const float l2 = log2_one_minus(aff[v]);
+              x[v] = (MASKED && diag && 4 * g + v <= col) ? 0.f : l2;
+            }
+            x[1] += x[0]; x[2] += x[1]; x[3] += x[2];
+            float before, after, tot;
+            group_scan(x[3], gm, before, after, tot);
+            before += cin;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const float dl = (diag && t_of(v, hi) <= col) ? 0.f : dS[v] + din;
-          const float av = aff[v];
-          const float den = fmaxf(fminf(av, kAMax), kAMinBwd) - 1.0f;
-          const float dA = (av <= kAMax) ? dl * __builtin_amdgcn_rcpf(den) : 0.f;
-          const float f = (2.0f / 3.0f) * __builtin_amdgcn_exp2f(__builtin_fmaf(gk[v], -1.0f / 3.0f, lab[v]));
-          const float dg = (gk[v] > -1.0e30f) ? dA * f : 0.f;
-          sXg[t_of(v, hi) * SS + pcol] = cvt<T>(dg);
-        }
+            for (int v = 0; v < 4; ++v) {
+              float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[v], kLog2e, x[v] + before) - l2t[v]);
+              if (MASKED) p = (diag && 4 * g + v < col) ? 0.f : p;
+              dS[v] = p * (dP[v] - dlt[v]);
+            }
+            // decay part: suffix over this wave's 16 queries + carry of the later tiles
+            f32x4 y = dS;
+            y[2] += y[3]; y[1] += y[2]; y[0] += y[1];
+            group_scan(y[0], gm, before, after, tot);
+            after += din;
 #pragma unroll
-        for (int kq = 0; kq < 2; ++kq) {
-          const Frag<T> as = ld8(sXs + col * SS + 16 * kq + 8 * hi), ag = ld8(sXg + col * SS + 16 * kq + 8 * hi);
-#pragma unroll
-          for (int n = 0; n < NB; ++n) {
-            const Frag<T> kb = ld8(sKT + (32 * n + col) * TS + 16 * kq + 8 * hi);
-            mma(dQ[n], as, kb);
-            mma(dKc[n], ag, kb);
+            for (int v = 0; v < 4; ++v) {
+              float dl = y[v] + after;
+              if (MASKED) dl = (diag && 4 * g + v <= col) ? 0.f : dl;
+              const float av = aff[v];
+              const float den = __builtin_amdgcn_fmed3f(av, kAMinBwd, kAMax) - 1.0f;
+              const float dA = (av <= kAMax) ? dl * __builtin_amdgcn_rcpf(den) : 0.f;
+              const float f = (2.0f / 3.0f) * __builtin_amdgcn_exp2f(__builtin_fmaf(gk[v], -1.0f / 3.0f, lab[v]));
+              dg[v] = (gk[v] > -1.0e30f) ? dA * f : 0.f;
+            }
           }
+          const int pc = jj ? pc1 : pc0;
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            sX[(4 * g + v) * XS + pc] = cvt<T>(dS[v]);
+            sX[(4 * g + v) * XS + 32 + pc] = cvt<T>(dg[v]);
+          }
+        }
+        // dQ += dS^T K,  dkcol += dg^T K   (contraction over the 32 keys of the half)
+        const T* sKT = reinterpret_cast<const T*>(base + 4 * TN::BYTES + kq * TT::BYTES);
+        const Frag<T> as = ld8(sX + col * XS + 8 * g), ag = ld8(sX + col * XS + 32 + 8 * g);
+#pragma unroll
+        for (int n = 0; n < ND; ++n) {
+          const Frag<T> kb = ld8(sKT + (16 * n + col) * TS + 8 * g);
+          mma16(dQ[n], as, kb);
+          mma16(dKc[n], ag, kb);
         }
       }
     };
-    UA_PIPELINE(n_kt, UA_ISSUE, UA_COMPUTE);
+    {
+      // the last two key tiles hold the diagonal blocks of the eight waves
+      const int nfast = n_kt - 2;
+      UA_PIPE_START(n_kt, UA_ISSUE);
+      UA_PIPE_RANGE(0, nfast, n_kt, UA_ISSUE, UA_COMPUTE_FAST);
+      UA_PIPE_RANGE(nfast, n_kt, n_kt, UA_ISSUE, UA_COMPUTE_SLOW);
+    }
 #undef UA_ISSUE
-#undef UA_COMPUTE
-    __syncthreads();   // the next group's prologue reuses stage 0
+#undef UA_COMPUTE_FAST
+#undef UA_COMPUTE_SLOW
+    __syncthreads();   // the next group's prologue refills stage 0
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int t = 32 * tb + t_of(v, hi);
+    for (int v = 0; v < 4; ++v) {
+      const int t = 16 * tq + 4 * g + v;
       if (t < L) {
 #pragma unroll
-        for (int n = 0; n < NB; ++n) {
-          const int dd = 32 * n + col;
+        for (int n = 0; n < ND; ++n) {
+          const int dd = 16 * n + col;
           if (dd < d) dq[(zq * L + t) * d + dd] = cvt<T>(dQ[n][v]);
         }
       }
     }
   }
 #pragma unroll
-  for (int v = 0; v < 16; ++v) {
-    const int t = 32 * tb + t_of(v, hi);
+  for (int v = 0; v < 4; ++v) {
+    const int t = 16 * tq + 4 * g + v;
 #pragma unroll
-    for (int n = 0; n < NB; ++n) a.dKdacc[((long)zk * Lp + t) * D + 32 * n + col] = dKc[n][v];
+    for (int n = 0; n < ND; ++n) a.dKdacc[((long)zk * Lp + t) * D + 16 * n + col] = dKc[n][v];
   }
 }
 

@@ -34,7 +34,7 @@ UA_INST(bf16, 64, 2) UA_INST(bf16, 128, 2) UA_INST(float, 64, 1) UA_INST(float, 
 
 template <class T, int D, int NST, bool MR>
 static hipError_t bwd2_mr(const BwdArgs<T>& a, int Lp, int Zk, hipStream_t s) {
-  hipLaunchKernelGGL((k_bwd_keys2<T, D, NST, MR>), dim3(Lp / 128, Zk), dim3(256), 0, s, a);
+  hipLaunchKernelGGL((k_bwd_keys2<T, D, NST, MR>), dim3(Lp / 128, Zk), dim3(512), 0, s, a);
   return hipGetLastError();
 }
 template <class T, int D, int NST>
@@ -62,7 +62,7 @@ UA_INST(bf16, 64, 2) UA_INST(bf16, 128, 2) UA_INST(float, 64, 1) UA_INST(float, 
 template <class T, int D, int NST>
 static hipError_t bwdq_t(const BwdArgsV& v, void* dq, int d, int Zk, hipStream_t s) {
   const BwdArgs<T> a = typed<T>(v);
-  hipLaunchKernelGGL((k_bwd_queries2<T, D, NST>), dim3(v.Lp / 128, Zk), dim3(256), 0, s, a, (T*)dq, d);
+  hipLaunchKernelGGL((k_bwd_queries2<T, D, NST>), dim3(v.Lp / 128, Zk), dim3(512), 0, s, a, (T*)dq, d);
   return hipGetLastError();
 }
 hipError_t launch_bwd_queries(int dtype, int D, const BwdArgsV& a, void* dq, int d, int Zk, hipStream_t s) {

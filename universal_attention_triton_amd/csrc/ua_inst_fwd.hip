@@ -13,7 +13,7 @@ static void allow_lds(K kernel, size_t bytes) {
 template <class T, int D>
 static hipError_t carry_t(const void* Kp, const float* lsrc, const float* ldest, float* C, int Lp, int Zk, hipStream_t s) {
   constexpr int NST = 2;
-  hipLaunchKernelGGL((k_carry2<T, D, NST>), dim3(Lp / 128, Zk), dim3(256), 0, s, (const T*)Kp, lsrc, ldest, C, Lp);
+  hipLaunchKernelGGL((k_carry2<T, D, NST>), dim3(Lp / 128, Zk), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, C, Lp);
   return hipGetLastError();
 }
 hipError_t launch_carry(int dtype, int D, const void* Kp, const float* lsrc, const float* ldest, float* C, int Lp, int Zk,
@@ -32,7 +32,7 @@ UA_INST(bf16, 64, 1) UA_INST(bf16, 64, 2) UA_INST(bf16, 128, 1) UA_INST(bf16, 12
 template <class T, int D, int NST>
 static hipError_t fused_t(const void* Qp, const void* Kp, const void* VT, const float* lsrc, const float* ldest,
                           const float* C, void* O, float* lse, float* lse2, int R, int L, int Lp, int d, int Zq, hipStream_t s) {
-  hipLaunchKernelGGL((k_fwd_fused2<T, D, NST>), dim3(Lp / 128, Zq), dim3(256), 0, s, (const T*)Qp, (const T*)Kp,
+  hipLaunchKernelGGL((k_fwd_fused2<T, D, NST>), dim3(Lp / 128, Zq), dim3(512), 0, s, (const T*)Qp, (const T*)Kp,
                      (const T*)VT, lsrc, ldest, C, (T*)O, lse, lse2, R, L, Lp, d);
   return hipGetLastError();
 }

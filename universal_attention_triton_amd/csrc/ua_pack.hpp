@@ -21,9 +21,10 @@ __device__ __forceinline__ long rows_offset(const RowsView& v, int z, int row) {
 }
 
 // x (dtype T) -> nat [Z][Lp][D] and/or tr [Z][D][Lp], zero padded (rows >= L, cols >= d).
-// tr stores position t at column perm16(t).
+// tr stores position t at column perm16(t) (tr_mode 0), perm32(t) (1) or t (2).
 template <class T, int D>
-__global__ void __launch_bounds__(256) k_pack(RowsView x, T* __restrict__ nat, T* __restrict__ tr, int d, int L, int Lp) {
+__global__ void __launch_bounds__(256) k_pack(RowsView x, T* __restrict__ nat, T* __restrict__ tr, int d, int L, int Lp,
+                                              int tr_mode) {
   __shared__ float tile[32][D + 1];
   const int z = blockIdx.y, row0 = blockIdx.x * 32, tid = threadIdx.x;
   const T* xp = reinterpret_cast<const T*>(x.p);
@@ -38,7 +39,9 @@ __global__ void __launch_bounds__(256) k_pack(RowsView x, T* __restrict__ nat, T
   __syncthreads();
   for (int i = tid; i < 32 * D; i += 256) {
     int dd = i >> 5, rr = i & 31;
-    tr[((long)z * D + dd) * Lp + row0 + rr] = cvt<T>(tile[perm16(rr)][dd]);
+    // perm16 and perm32 are involutions / bijections of 0..31: column rr holds the position that maps onto it
+    const int src = tr_mode == 0 ? perm16(rr) : (tr_mode == 1 ? (((rr >> 3) & 3) << 2 | ((rr >> 2) & 1) << 4 | (rr & 3)) : rr);
+    tr[((long)z * D + dd) * Lp + row0 + rr] = cvt<T>(tile[src][dd]);
   }
 }
 
