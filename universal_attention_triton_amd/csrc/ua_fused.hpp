@@ -121,7 +121,7 @@ __global__ void __launch_bounds__(512) k_carry2(const T* __restrict__ Kp, const 
     for (int i = 0; i < 2; ++i) {
       f32x4 acc = {0, 0, 0, 0};
 #pragma unroll
-      for (int q = 0; q < NK; ++q) mma16(acc, ld8(sK + (16 * i + col) * LS + 32 * q + 8 * g), ks[q]);
+      for (int q = 0; q < NK; ++q) mma16(acc, ld8(sK + TN::at(i, col, q, g)), ks[q]);
       const f32x4 lb = load_t4(stats + 16 * i, g);
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
@@ -212,14 +212,14 @@ __global__ void __launch_bounds__(512) k_fwd_fused2(const T* __restrict__ Qp, co
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int sbk = 4 * kt + j;                      // 16-key tile
-      const T* sK = reinterpret_cast<const T*>(base + (j >> 1) * TN::BYTES) + (16 * (j & 1) + col) * LS + 8 * g;
+      const T* sK = reinterpret_cast<const T*>(base + (j >> 1) * TN::BYTES);
       if (!MASKED || sbk <= tq) {
         const float c = stats[16 * j + col];
         const float la = stats[64 + 16 * j + col];
         f32x4 gt = {0, 0, 0, 0}, sc = {0, 0, 0, 0};
 #pragma unroll
         for (int q = 0; q < NK; ++q) {
-          const Frag<T> kb = ld8(sK + 32 * q);
+          const Frag<T> kb = ld8(sK + TN::at(j & 1, col, q, g));
           mma16(gt, kf[q], kb);
           mma16(sc, qf[q], kb);
         }
@@ -277,7 +277,7 @@ __global__ void __launch_bounds__(512) k_fwd_fused2(const T* __restrict__ Qp, co
         const T* sV = reinterpret_cast<const T*>(base + 2 * TN::BYTES + kq * TT::BYTES);
         const Frag<T> pa = ld8(sPw + col * PS + 32 * kq + 8 * g);
 #pragma unroll
-        for (int n = 0; n < ND; ++n) mma16(o[n], pa, ld8(sV + (16 * n + col) * TS + 8 * g));
+        for (int n = 0; n < ND; ++n) mma16(o[n], pa, ld8(sV + TT::at(n, col, 0, g)));
       }
     }
   };
@@ -403,7 +403,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
       for (int i = 0; i < 2; ++i) {
         f32x4 acc = {0, 0, 0, 0};
 #pragma unroll
-        for (int q = 0; q < NK; ++q) mma16(acc, ld8(sKt + (16 * i + col) * LS + 32 * q + 8 * g), kp[q]);
+        for (int q = 0; q < NK; ++q) mma16(acc, ld8(sKt + TN::at(i, col, q, g)), kp[q]);
         lab[i] = load_t4(stats + 64 + 16 * i, g);
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
@@ -426,9 +426,9 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
       for (int i = 0; i < 2; ++i) {
         f32x4 sc = {0, 0, 0, 0}, dP = {0, 0, 0, 0};
 #pragma unroll
-        for (int q = 0; q < NK; ++q) mma16(sc, ld8(sQ + (16 * i + col) * LS + 32 * q + 8 * g), kp[q]);
+        for (int q = 0; q < NK; ++q) mma16(sc, ld8(sQ + TN::at(i, col, q, g)), kp[q]);
 #pragma unroll
-        for (int q = 0; q < NK; ++q) mma16(dP, ld8(sdO + (16 * i + col) * LS + 32 * q + 8 * g), vf[q]);
+        for (int q = 0; q < NK; ++q) mma16(dP, ld8(sdO + TN::at(i, col, q, g)), vf[q]);
         const f32x4 l2t = load_t4(stats + 16 * i, g), dlt = load_t4(stats + 32 + 16 * i, g);
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
@@ -440,9 +440,9 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
       }
       const Frag<T> bp = as_operand16<T>(P[0], P[1]), bs = as_operand16<T>(dS[0], dS[1]);
 #pragma unroll
-      for (int n = 0; n < ND; ++n) mma16(dVt[n], ld8(sdOT + (16 * n + col) * TS + 8 * g), bp);
+      for (int n = 0; n < ND; ++n) mma16(dVt[n], ld8(sdOT + TT::at(n, col, 0, g)), bp);
 #pragma unroll
-      for (int n = 0; n < ND; ++n) mma16(dKt[n], ld8(sQT + (16 * n + col) * TS + 8 * g), bs);
+      for (int n = 0; n < ND; ++n) mma16(dKt[n], ld8(sQT + TT::at(n, col, 0, g)), bs);
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -472,7 +472,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
       dcar += tot;
       const Frag<T> b = as_operand16<T>(dB[0], dB[1]);
 #pragma unroll
-      for (int n = 0; n < ND; ++n) mma16(dKt[n], ld8(sKT + (16 * n + col) * TS + 8 * g), b);
+      for (int n = 0; n < ND; ++n) mma16(dKt[n], ld8(sKT + TT::at(n, col, 0, g)), b);
     }
   };
   {
@@ -588,18 +588,19 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
           const bool diag = MASKED && (sbk == tq);
           f32x4 dS = {0, 0, 0, 0}, dg = {0, 0, 0, 0};
           if (live) {
-            const T* sK = reinterpret_cast<const T*>(base + kq * TN::BYTES) + (16 * jj + col) * LS + 8 * g;
-            const T* sV = reinterpret_cast<const T*>(base + (2 + kq) * TN::BYTES) + (16 * jj + col) * LS + 8 * g;
+            const T* sK = reinterpret_cast<const T*>(base + kq * TN::BYTES);
+            const T* sV = reinterpret_cast<const T*>(base + (2 + kq) * TN::BYTES);
             const float cin = stats[16 * j + col];
             const float la = stats[64 + 16 * j + col];
             const float din = (r == 0) ? stats[128 + 16 * j + col] : 0.f;
             f32x4 acc = {0, 0, 0, 0}, sc = {0, 0, 0, 0}, dP = {0, 0, 0, 0};
 #pragma unroll
             for (int q = 0; q < NK; ++q) {
-              const Frag<T> kb = ld8(sK + 32 * q);
+              const int o = TN::at(jj, col, q, g);
+              const Frag<T> kb = ld8(sK + o);
               mma16(acc, kt[q], kb);
               mma16(sc, qt[q], kb);
-              mma16(dP, gt[q], ld8(sV + 32 * q));
+              mma16(dP, gt[q], ld8(sV + o));
             }
             f32x4 x, gk, aff, lab;
 #pragma unroll
@@ -648,7 +649,7 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
         const Frag<T> as = ld8(sX + col * XS + 8 * g), ag = ld8(sX + col * XS + 32 + 8 * g);
 #pragma unroll
         for (int n = 0; n < ND; ++n) {
-          const Frag<T> kb = ld8(sKT + (16 * n + col) * TS + 8 * g);
+          const Frag<T> kb = ld8(sKT + TT::at(n, col, 0, g));
           mma16(dQ[n], as, kb);
           mma16(dKc[n], ag, kb);
         }
