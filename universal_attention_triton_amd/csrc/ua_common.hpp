@@ -133,10 +133,11 @@ __device__ __forceinline__ void stage_tile(T* __restrict__ lds, const T* __restr
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 // A [ROWS][COLS] operand tile in LDS, filled by asynchronous global->LDS loads in units of 16-byte chunks.
-// ds_read_b128 serves 16 lanes per cycle in the groups {0-7, 24-31}, {8-15, 16-23}, {32-39, 56-63}, {40-47, 48-55};
-// an MFMA operand read (lane = row l%16, chunk l/16 of a 32-wide k-step) is conflict-free when those 16 chunks
-// fall on distinct banks.  bf16 tiles get that without padding by storing payload chunk c of row r at position
-// c ^ swz(r); fp32 tiles keep one padding chunk per row.
+// ds_read_b128 serves 16 lanes per cycle (256 bytes over 64 banks).  An MFMA operand read (lane = row l%16,
+// chunk l/16 of a 32-wide k-step) from rows padded by one chunk takes 8 cycles instead of 4 on this part; storing
+// payload chunk c of row r at position c ^ swz(r) in UNPADDED rows was measured conflict-free for rows of 16 and
+// 8 chunks with swz = r mod chunks-per-row, and for rows of 4 chunks with swz = (r >> 1) & 3.  bf16 tiles use
+// that; fp32 tiles keep one padding chunk per row.
 template <class T, int ROWS, int COLS> struct Tile {
   static constexpr bool SWZ = sizeof(T) == 2;
   static constexpr int STRIDE = SWZ ? COLS : COLS + kPad16 / (int)sizeof(T);   // elements per row
@@ -145,12 +146,12 @@ template <class T, int ROWS, int COLS> struct Tile {
   static constexpr int NINSTR = (ROWS * CPR + 63) / 64;
   static constexpr int BYTES = NINSTR * 1024;                          // LDS footprint
   static_assert(!SWZ || CPP == 4 || CPP == 8 || CPP == 16, "swizzle is defined for rows of 4, 8 or 16 chunks");
-  __host__ __device__ static constexpr int swz(int r) { return CPP >= 8 ? (r & (CPP - 1)) : ((r >> 2) & (CPP - 1)); }
+  __host__ __device__ static constexpr int swz(int r) { return CPP >= 8 ? (r & (CPP - 1)) : ((r >> 1) & (CPP - 1)); }
   // element offset of the 8 k-values [32q + 8g, 32q + 8g + 8) of row 16*blk + col  (col = lane & 15, g = lane >> 4)
   __device__ __forceinline__ static int at(int blk, int col, int q, int g) {
     if constexpr (SWZ) {
       if constexpr (CPP >= 8) return (16 * blk + col) * STRIDE + (((4 * q + g) ^ (col & (CPP - 1))) << 3);
-      else return (16 * blk + col) * STRIDE + (((g ^ (col >> 2)) & 3) << 3);          // 32-wide rows: q == 0
+      else return (16 * blk + col) * STRIDE + (((g ^ (col >> 1)) & 3) << 3);          // 32-wide rows: q == 0
     } else {
       return (16 * blk + col) * STRIDE + 32 * q + 8 * g;
     }
