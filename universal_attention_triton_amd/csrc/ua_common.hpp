@@ -177,12 +177,24 @@ template <class TILE, int NWAVES> struct Stager {
 #pragma unroll
     for (int k = 0; k < PER; ++k) {
       const int i = w + k * NWAVES;
-      if (i < TILE::NINSTR)
+      if (TILE::NINSTR % NWAVES == 0 || i < TILE::NINSTR)
         __builtin_amdgcn_global_load_lds(reinterpret_cast<const char*>(gtile) + off[k],
                                          (lds_ptr_t)(reinterpret_cast<char*>(lds_tile) + i * 1024), 16, 0, 0);
     }
   }
 };
+// Workgroups go to the 8 XCDs round-robin in dispatch order (x fastest).  This map hands every XCD whole heads
+// (grid y), in the same x order, so that the tiles which all workgroups of a head stream hit in that XCD's L2
+// instead of being fetched once per XCD.  Falls back to the identity when the head count is not a multiple of 8.
+__device__ __forceinline__ void xcd_map(int& bx, int& by) {
+  const int gx = gridDim.x, gy = gridDim.y;
+  bx = blockIdx.x; by = blockIdx.y;
+  if ((gy & 7) == 0) {
+    const int n = bx + gx * by, slot = n >> 3;
+    by = (n & 7) + 8 * (slot / gx);
+    bx = slot % gx;
+  }
+}
 __device__ __forceinline__ void wait_async_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // Column order of the transposed ([feature][position]) working tensors: inside every group of 16
@@ -326,6 +338,14 @@ __device__ __forceinline__ float allsum16(float v) {
 __device__ __forceinline__ float log2_relu(float g) { return __builtin_amdgcn_logf(fmaxf(g, 0.f)); }
 __device__ __forceinline__ float affinity(float lg, float lab) {
   return __builtin_amdgcn_exp2f(__builtin_fmaf(lg, 2.0f / 3.0f, lab));
+}
+// dG from the gradient dl of l = log2(1 - A) (log2 units folded by the caller):
+//   dA = dl / (clamp(A, 1e-6, 1-1e-6) - 1), zero where A exceeds the clamp;  dG = dA (2/3) A / G
+// as ONE reciprocal of (3/2)(clamp(A) - 1) G.  grelu = relu(G); where it is 0, A is 0 and so is the result.
+__device__ __forceinline__ float decay_grad(float dl, float a, float grelu) {
+  const float den15 = __builtin_fmaf(__builtin_amdgcn_fmed3f(a, kAMinBwd, kAMax), 1.5f, -1.5f);
+  const float r = __builtin_amdgcn_rcpf(den15 * fmaxf(grelu, 1.0e-30f));
+  return (a <= kAMax) ? (dl * a) * r : 0.f;
 }
 __device__ __forceinline__ float log2_one_minus(float a) { return __builtin_amdgcn_logf(1.0f - fminf(a, kAMax)); }
 constexpr float kGatePad = -1.0e4f;   // log-gate of padded rows: makes their affinity exactly 0

@@ -86,7 +86,9 @@ __global__ void __launch_bounds__(512) k_carry2(const T* __restrict__ Kp, const 
   constexpr int NK = D / 32, LS = TN::STRIDE, SB = TN::BYTES + 1024;   // tile + [ldest of the block: 32 floats]
   UA_STAGES(SB);
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
-  const int z = blockIdx.y, nT = Lp / 32, nT16 = Lp / 16, sb16 = 8 * blockIdx.x + w, first = 4 * blockIdx.x;
+  int bx, z;
+  xcd_map(bx, z);
+  const int nT = Lp / 32, nT16 = Lp / 16, sb16 = 8 * bx + w, first = 4 * bx;
   const int spos = 16 * sb16 + col;
   const GroupMasks gm = group_masks(lane);
   Stager<TN, 8> st;
@@ -167,8 +169,10 @@ __global__ void __launch_bounds__(512) k_fwd_fused2(const T* __restrict__ Qp, co
   UA_STAGES(SB);
   __shared__ __attribute__((aligned(16))) T sPbuf[8 * 16 * PS];
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
-  const int zq = blockIdx.y, zk = zq / R, nT16 = Lp / 16;
-  const int jt = gridDim.x - 1 - blockIdx.x, tq = 8 * jt + w;       // 16-query tile of this wave
+  int bx, zq;
+  xcd_map(bx, zq);
+  const int zk = zq / R, nT16 = Lp / 16;
+  const int jt = gridDim.x - 1 - bx, tq = 8 * jt + w;       // 16-query tile of this wave
   T* sPw = sPbuf + w * 16 * PS;
   const GroupMasks gm = group_masks(lane);
   Stager<TN, 8> stN;
@@ -325,8 +329,10 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   // stats row of a stage: [lse2: 32f][delta: 32f][ldest: 32f][unused: 32f][forward carries of the 128 keys: 128f]
   UA_STAGES(SB);
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
-  const int zk = blockIdx.y, Lp = a.Lp, L = a.L, nT16 = Lp / 16, R = MR ? a.R : 1;
-  const int kg = gridDim.x - 1 - blockIdx.x, sb16 = 8 * kg + w, spos = 16 * sb16 + col;
+  int bx, zk;
+  xcd_map(bx, zk);
+  const int Lp = a.Lp, L = a.L, nT16 = Lp / 16, R = MR ? a.R : 1;
+  const int kg = gridDim.x - 1 - bx, sb16 = 8 * kg + w, spos = 16 * sb16 + col;
   const int nTr = (L + 31) / 32, first = 4 * kg;
   if (first >= nTr) return;                      // every key of this workgroup is padding
   const GroupMasks gm = group_masks(lane);
@@ -346,7 +352,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
 #pragma unroll
   for (int n = 0; n < ND; ++n) { dVt[n] = (f32x4){0, 0, 0, 0}; dKt[n] = (f32x4){0, 0, 0, 0}; }
   float dsrc_acc = 0.f, dcar = 0.f;
-  f32x4 aff_s[2], bias_s[2], gk_s[2], dB_s[2], lab_s[2];     // state of the current query block (used when MR)
+  f32x4 aff_s[2], bias_s[2], gk_s[2], dB_s[2];     // state of the current query block (used when MR); gk = relu(G)
   const T* Kz = a.Kp + (long)zk * Lp * D;
   const T* KTz = a.KT + (long)zk * D * Lp;
   const float* ldz = a.ldest + (long)zk * Lp;
@@ -390,12 +396,11 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
     const T* sQT = reinterpret_cast<const T*>(base + 3 * TN::BYTES + TT::BYTES);
     const T* sdOT = reinterpret_cast<const T*>(base + 3 * TN::BYTES + 2 * TT::BYTES);
     const float* stats = reinterpret_cast<const float*>(base + TILES);
-    f32x4 aff_l[2], bias_l[2], gk_l[2], dB_l[2], lab_l[2];
+    f32x4 aff_l[2], bias_l[2], gk_l[2], dB_l[2];
     f32x4 (&aff)[2] = MR ? aff_s : aff_l;
     f32x4 (&bias)[2] = MR ? bias_s : bias_l;
     f32x4 (&gk)[2] = MR ? gk_s : gk_l;
     f32x4 (&dB)[2] = MR ? dB_s : dB_l;
-    f32x4 (&lab)[2] = MR ? lab_s : lab_l;
     const int tl0 = 32 * tb + 4 * g - spos;        // query position minus key position for (tile 0, v = 0)
     if (!MR || r == 0) {
       const float cin = stats[128 + 16 * w + col];
@@ -404,12 +409,11 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
         f32x4 acc = {0, 0, 0, 0};
 #pragma unroll
         for (int q = 0; q < NK; ++q) mma16(acc, ld8(sKt + TN::at(i, col, q, g)), kp[q]);
-        lab[i] = load_t4(stats + 64 + 16 * i, g);
+        const f32x4 lab = load_t4(stats + 64 + 16 * i, g);
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
-          lab[i][v] += la;
-          gk[i][v] = log2_relu(acc[v]);
-          aff[i][v] = affinity(gk[i][v], lab[i][v]);
+          gk[i][v] = fmaxf(acc[v], 0.f);
+          aff[i][v] = affinity(__builtin_amdgcn_logf(gk[i][v]), lab[v] + la);
           const float l2 = log2_one_minus(aff[i][v]);
           bias[i][v] = (MASKED && diag && tl0 + 16 * i + v <= 0) ? 0.f : l2;
         }
@@ -461,12 +465,8 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
         for (int v = 0; v < 4; ++v) {
           float dl = dB[i][v] + dcar;
           if (MASKED) dl = (diag && tl0 + 16 * i + v <= 0) ? 0.f : dl;
-          const float av = aff[i][v];
-          const float den = __builtin_amdgcn_fmed3f(av, kAMinBwd, kAMax) - 1.0f;
-          const float dA = (av <= kAMax) ? dl * __builtin_amdgcn_rcpf(den) : 0.f;
-          dsrc_acc = __builtin_fmaf(dA, av, dsrc_acc);
-          const float f = (2.0f / 3.0f) * __builtin_amdgcn_exp2f(__builtin_fmaf(gk[i][v], -1.0f / 3.0f, lab[i][v]));
-          dB[i][v] = (gk[i][v] > -1.0e30f) ? dA * f : 0.f;
+          dB[i][v] = decay_grad(dl, aff[i][v], gk[i][v]);
+          dsrc_acc = __builtin_fmaf(dB[i][v], gk[i][v], dsrc_acc);
         }
       }
       dcar += tot;
@@ -489,7 +489,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   {
     float b, af, tot;
     group_scan(dsrc_acc, gm, b, af, tot);
-    if (g == 0) a.dsrc_raw[(long)zk * Lp + spos] = tot;
+    if (g == 0) a.dsrc_raw[(long)zk * Lp + spos] = 1.5f * tot;    // sum dA A = 3/2 sum dG G
   }
 #pragma unroll
   for (int n = 0; n < ND; ++n) {
@@ -516,8 +516,10 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
   UA_STAGES(SB);
   __shared__ __attribute__((aligned(16))) T sXbuf[8 * 16 * XS];
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
-  const int zk = blockIdx.y, Lp = a.Lp, L = a.L, nT16 = Lp / 16, R = a.R;
-  const int jt = gridDim.x - 1 - blockIdx.x, tq = 8 * jt + w;
+  int bx, zk;
+  xcd_map(bx, zk);
+  const int Lp = a.Lp, L = a.L, nT16 = Lp / 16, R = a.R;
+  const int jt = gridDim.x - 1 - bx, tq = 8 * jt + w;
   T* sX = sXbuf + w * 16 * XS;
   const GroupMasks gm = group_masks(lane);
   Stager<TN, 8> stN;
@@ -602,12 +604,11 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
               mma16(sc, qt[q], kb);
               mma16(dP, gt[q], ld8(sV + o));
             }
-            f32x4 x, gk, aff, lab;
+            f32x4 x, gk, aff;
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
-              lab[v] = la + lb[v];
-              gk[v] = log2_relu(acc[v]);
-              aff[v] = affinity(gk[v], lab[v]);
+              gk[v] = fmaxf(acc[v], 0.f);
+              aff[v] = affinity(__builtin_amdgcn_logf(gk[v]), la + lb[v]);
               const float l2 = log2_one_minus(aff[v]);
               x[v] = (MASKED && diag && 4 * g + v <= col) ? 0.f : l2;
             }
@@ -630,11 +631,7 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
             for (int v = 0; v < 4; ++v) {
               float dl = y[v] + after;
               if (MASKED) dl = (diag && 4 * g + v <= col) ? 0.f : dl;
-              const float av = aff[v];
-              const float den = __builtin_amdgcn_fmed3f(av, kAMinBwd, kAMax) - 1.0f;
-              const float dA = (av <= kAMax) ? dl * __builtin_amdgcn_rcpf(den) : 0.f;
-              const float f = (2.0f / 3.0f) * __builtin_amdgcn_exp2f(__builtin_fmaf(gk[v], -1.0f / 3.0f, lab[v]));
-              dg[v] = (gk[v] > -1.0e30f) ? dA * f : 0.f;
+              dg[v] = decay_grad(dl, aff[v], gk[v]);
             }
           }
           const int pc = jj ? pc1 : pc0;
