@@ -153,11 +153,11 @@ __global__ void __launch_bounds__(512) k_carry2(const T* __restrict__ Kp, const 
 }
 
 // ---------------------------------------------------------------------------------------------
-// Fused forward.  grid (Lp/128, Zq); 8 waves; wave w owns queries 16*(8*jt+w)..+15; 64 keys per step,
+// Fused forward.  grid (ceil(Lp/16/NW), Zq); NW waves; wave w owns queries 16*(NW*jt+w)..+15; 64 keys per step,
 // key tiles visited from the diagonal backwards.
 // ---------------------------------------------------------------------------------------------
-template <class T, int D, int NST>
-__global__ void __launch_bounds__(512) k_fwd_fused2(const T* __restrict__ Qp, const T* __restrict__ Kp,
+template <class T, int D, int NST, int NW>
+__global__ void __launch_bounds__(64 * NW) k_fwd_fused2(const T* __restrict__ Qp, const T* __restrict__ Kp,
                                                     const T* __restrict__ VT, const float* __restrict__ lsrc,
                                                     const float* __restrict__ ldest, const float* __restrict__ C,
                                                     T* __restrict__ O, float* __restrict__ lse, float* __restrict__ lse2,
@@ -165,18 +165,20 @@ __global__ void __launch_bounds__(512) k_fwd_fused2(const T* __restrict__ Qp, co
   using TN = Tile<T, 32, D>;
   using TT = Tile<T, D, 32>;
   constexpr int NK = D / 32, ND = D / 16, LS = TN::STRIDE, TS = TT::STRIDE, PS = lds_stride<T>(64);
-  constexpr int TILES = 2 * TN::BYTES + 2 * TT::BYTES, SB = TILES + 8 * 1024;   // + per wave [C row: 64f][lsrc: 64f]
+  constexpr int TILES = 2 * TN::BYTES + 2 * TT::BYTES, SB = TILES + NW * 1024;   // + per wave [C row: 64f][lsrc: 64f]
   UA_STAGES(SB);
-  __shared__ __attribute__((aligned(16))) T sPbuf[8 * 16 * PS];
+  __shared__ __attribute__((aligned(16))) T sPbuf[NW * 16 * PS];
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
   int bx, zq;
   xcd_map(bx, zq);
   const int zk = zq / R, nT16 = Lp / 16;
-  const int jt = gridDim.x - 1 - bx, tq = 8 * jt + w;       // 16-query tile of this wave
+  const int jt = gridDim.x - 1 - bx;
+  const bool live = NW * jt + w < nT16;                      // the last workgroup may hold waves past the end
+  const int tq = live ? NW * jt + w : nT16 - 1;             // 16-query tile of this wave
   T* sPw = sPbuf + w * 16 * PS;
   const GroupMasks gm = group_masks(lane);
-  Stager<TN, 8> stN;
-  Stager<TT, 8> stT;
+  Stager<TN, NW> stN;
+  Stager<TT, NW> stT;
   stN.init(w, lane, D * (long)sizeof(T), 32);
   stT.init(w, lane, Lp * (long)sizeof(T), D);
 
@@ -196,7 +198,8 @@ __global__ void __launch_bounds__(512) k_fwd_fused2(const T* __restrict__ Qp, co
   const float* lsz = lsrc + (long)zk * Lp;
   const T* Kz = Kp + (long)zk * Lp * D;
   const T* Vz = VT + (long)zk * D * Lp;
-  const int n_kt = 2 * jt + 2;   // key tiles of 64 covering s <= last query of the workgroup
+  const int tq_end = min(NW * (jt + 1), nT16);
+  const int n_kt = (tq_end + 3) / 4;   // key tiles of 64 covering s <= last query of the workgroup
 
 #define UA_ISSUE(s, base)                                                                   \
   {                                                                                         \
@@ -286,15 +289,17 @@ __global__ void __launch_bounds__(512) k_fwd_fused2(const T* __restrict__ Qp, co
     }
   };
   {
-    // the first two key tiles (visited first) hold the diagonal blocks of the eight waves
+    // the key tiles visited first hold the diagonal blocks of the waves
+    const int nslow = min(n_kt, (n_kt - (NW * jt) / 4 + 1) & ~1);
     UA_PIPE_START(n_kt, UA_ISSUE);
-    UA_PIPE_RANGE(0, 2, n_kt, UA_ISSUE, UA_COMPUTE_SLOW);
-    UA_PIPE_RANGE(2, n_kt, n_kt, UA_ISSUE, UA_COMPUTE_FAST);
+    UA_PIPE_RANGE(0, nslow, n_kt, UA_ISSUE, UA_COMPUTE_SLOW);
+    UA_PIPE_RANGE(nslow, n_kt, n_kt, UA_ISSUE, UA_COMPUTE_FAST);
   }
 #undef UA_ISSUE
 #undef UA_COMPUTE_FAST
 #undef UA_COMPUTE_SLOW
   // epilogue
+  if (!live) return;
 #pragma unroll
   for (int v = 0; v < 4; ++v) {
     const float tot = allsum16(ls[v]);

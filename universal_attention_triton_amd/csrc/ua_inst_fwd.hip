@@ -23,30 +23,42 @@ hipError_t launch_carry(int dtype, int D, const void* Kp, const float* lsrc, con
 }
 
 // explicit instantiations (the implicit ones are not emitted on the host side for these kernels)
-#define UA_INST(T, D, NST)                                                                                            \
-  template __global__ void k_fwd_fused2<T, D, NST>(const T*, const T*, const T*, const float*, const float*, const float*, \
-                                                   T*, float*, float*, int, int, int, int);
-UA_INST(bf16, 64, 1) UA_INST(bf16, 64, 2) UA_INST(bf16, 128, 1) UA_INST(bf16, 128, 2) UA_INST(float, 64, 1) UA_INST(float, 128, 1)
+#define UA_INST(T, D, NST, NW)                                                                                        \
+  template __global__ void k_fwd_fused2<T, D, NST, NW>(const T*, const T*, const T*, const float*, const float*,      \
+                                                       const float*, T*, float*, float*, int, int, int, int);
+UA_INST(bf16, 64, 1, 8) UA_INST(bf16, 64, 2, 8) UA_INST(bf16, 64, 2, 12) UA_INST(bf16, 64, 2, 16)
+UA_INST(bf16, 128, 1, 8) UA_INST(bf16, 128, 2, 8) UA_INST(bf16, 128, 2, 12) UA_INST(bf16, 128, 2, 16)
+UA_INST(float, 64, 1, 8) UA_INST(float, 128, 1, 8)
 #undef UA_INST
 
-template <class T, int D, int NST>
+template <class T, int D, int NST, int NW>
 static hipError_t fused_t(const void* Qp, const void* Kp, const void* VT, const float* lsrc, const float* ldest,
                           const float* C, void* O, float* lse, float* lse2, int R, int L, int Lp, int d, int Zq, hipStream_t s) {
-  hipLaunchKernelGGL((k_fwd_fused2<T, D, NST>), dim3(Lp / 128, Zq), dim3(512), 0, s, (const T*)Qp, (const T*)Kp,
-                     (const T*)VT, lsrc, ldest, C, (T*)O, lse, lse2, R, L, Lp, d);
+  hipLaunchKernelGGL((k_fwd_fused2<T, D, NST, NW>), dim3((Lp / 16 + NW - 1) / NW, Zq), dim3(64 * NW), 0, s, (const T*)Qp,
+                     (const T*)Kp, (const T*)VT, lsrc, ldest, C, (T*)O, lse, lse2, R, L, Lp, d);
   return hipGetLastError();
 }
-// variants: 0 = double-buffered LDS stages, 1 = single stage (bf16 only; fp32 always runs single stage)
-int fwd_fused_variants(int dtype, int D) { (void)D; return dtype == 1 ? 2 : 1; }
+// variants (bf16): 0 = 8 waves, double-buffered stages; 1 = 8 waves, single stage; 2 = 12 waves; 3 = 16 waves
+// (both double-buffered).  fp32 always runs 8 waves with a single stage.
+int fwd_fused_variants(int dtype, int D) { (void)D; return dtype == 1 ? 4 : 1; }
+template <class T, int D>
+static hipError_t fused_v(int variant, const void* Qp, const void* Kp, const void* VT, const float* lsrc, const float* ldest,
+                          const float* C, void* O, float* lse, float* lse2, int R, int L, int Lp, int d, int Zq, hipStream_t s) {
+#define UA_ARGS Qp, Kp, VT, lsrc, ldest, C, O, lse, lse2, R, L, Lp, d, Zq, s
+  switch (variant) {
+    case 1: return fused_t<T, D, 1, 8>(UA_ARGS);
+    case 2: return fused_t<T, D, 2, 12>(UA_ARGS);
+    case 3: return fused_t<T, D, 2, 16>(UA_ARGS);
+    default: return fused_t<T, D, 2, 8>(UA_ARGS);
+  }
+#undef UA_ARGS
+}
 hipError_t launch_fwd_fused(int dtype, int D, int variant, const void* Qp, const void* Kp, const void* VT,
                             const float* lsrc, const float* ldest, const float* C, void* O, float* lse, float* lse2, int R,
                             int L, int Lp, int d, int Zq, hipStream_t s) {
 #define UA_ARGS Qp, Kp, VT, lsrc, ldest, C, O, lse, lse2, R, L, Lp, d, Zq, s
-  if (dtype == 1) {
-    if (D == 64) return variant == 1 ? fused_t<bf16, 64, 1>(UA_ARGS) : fused_t<bf16, 64, 2>(UA_ARGS);
-    return variant == 1 ? fused_t<bf16, 128, 1>(UA_ARGS) : fused_t<bf16, 128, 2>(UA_ARGS);
-  }
-  return D == 64 ? fused_t<float, 64, 1>(UA_ARGS) : fused_t<float, 128, 1>(UA_ARGS);
+  if (dtype == 1) return D == 64 ? fused_v<bf16, 64>(variant, UA_ARGS) : fused_v<bf16, 128>(variant, UA_ARGS);
+  return D == 64 ? fused_t<float, 64, 1, 8>(UA_ARGS) : fused_t<float, 128, 1, 8>(UA_ARGS);
 #undef UA_ARGS
 }
 
