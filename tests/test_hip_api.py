@@ -1,0 +1,209 @@
+"""Drop-in interface on the GPU: the reference's module paths, class names, shapes, error behaviour and
+autograd wiring, the fused entry points, the tune table, and edge cases of the inputs."""
+import pytest
+import torch
+
+from oracle import ua_oracle as orc
+from tests.util import NAMES, TOL, dense_reference, load_golden, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def _leaves(t, dtype, names=NAMES):
+    return [t[k].to(dtype).cuda().requires_grad_() for k in names]
+
+
+@pytest.mark.parametrize("name", ["tiny_fp32", "tiny_bf16", "small_fp32", "small_bf16"])
+def test_reference_call_sequence_through_the_drop_in_modules(name):
+    """out, denom = UniversalAttention.apply(...); O = SMVecMatMul.apply(out, denom) (softmax inside); O.backward(dO)
+    (reference universal_attention_autograd.py:7-99, :278-297) against the vectors the reference produced."""
+    import universal_attention_autograd as ref_api
+    t, dtype, (b, h, r, l, d, c, seed) = load_golden(name)
+    print("case drop-in", name, flush=True)
+    leaves = _leaves(t, dtype)
+    out, denom = ref_api.UniversalAttention.apply(*leaves)
+    assert out.shape == (b, h, r, l, d, l // c) and denom.shape == (b, h, r, l, l // c)
+    assert out.dtype == dtype and denom.dtype == dtype
+    O = ref_api.SMVecMatMul.apply(out, denom)
+    grads = torch.autograd.grad(O, leaves, t["dO"].to(dtype).cuda())
+    tol = TOL[dtype]
+    assert rel_err(out, t["out"]) <= tol and rel_err(denom, t["denom"]) <= tol and rel_err(O, t["O"]) <= tol
+    for g, k in zip(grads, ("c_dkc", "c_dvc", "c_dxq", "c_dsrc", "c_ddest")):
+        assert g is not None and g.shape == leaves[("c_dkc", "c_dvc", "c_dxq", "c_dsrc", "c_ddest").index(k)].shape
+        bar = tol if k != "c_dkc" else max(tol, 4e-4)      # d/dk of relu(k.k)^(2/3): see test_hip_backward
+        assert rel_err(g, t[k]) <= bar, (k, rel_err(g, t[k]))
+
+
+@pytest.mark.parametrize("name", ["tiny_fp32", "tiny_bf16"])
+def test_two_dimensional_layout_and_triton_side_entry(name):
+    """UniversalAttention2 (autograd.py:102-276) and the Triton-backed entry (Universal_Attention/universal_attention.py:5-46)
+    take xq [b,h,r,_n,_c,d] and static_dest [b,h,_n,_c] and return the same values as the 1-D operator."""
+    import universal_attention_autograd as ref_api
+    from Universal_Attention.universal_attention import UniversalAttention as Entry
+    t, dtype, (b, h, r, l, d, c, seed) = load_golden(name)
+    kc, vc, xq, src, dest = [t[k].to(dtype).cuda() for k in NAMES]
+    for _c in (c, 2 * c):
+        xq2, dest2 = xq.view(b, h, r, l // _c, _c, d), dest.view(b, h, l // _c, _c)
+        for op in (ref_api.UniversalAttention2, Entry):
+            out, denom = op.apply(kc, vc, xq2, src, dest2)
+            assert out.shape == (b, h, r, l, d, l // c)
+            assert rel_err(out, t["out"]) <= TOL[dtype] and rel_err(denom, t["denom"]) <= TOL[dtype]
+
+
+def test_entry_point_error_behaviour():
+    """AssertionError on a shape mismatch, ValueError on a wrong rank (universal_attention.py:8-13)."""
+    from Universal_Attention.universal_attention import UniversalAttention as Entry
+    inp = orc.make_inputs(1, 2, 1, 64, 16, 16, dtype=torch.float32, seed=3)
+    kc, vc, xq, src, dest = [inp[k].cuda() for k in NAMES]
+    xq2, dest2 = xq.view(1, 2, 1, 4, 16, 16), dest.view(1, 2, 4, 16)
+    with pytest.raises(AssertionError):
+        Entry.apply(kc, vc[:, :1], xq2, src, dest2)
+    with pytest.raises(AssertionError):
+        Entry.apply(kc, vc, xq2, src[..., :8], dest2)
+    with pytest.raises(ValueError):
+        Entry.apply(kc, vc, xq, src, dest2)            # 1-D xq where the 2-D layout is required
+    with pytest.raises(ValueError):
+        Entry.apply(kc.view(1, 2, 64, 16), vc, xq2, src, dest2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_fused_operator_autograd_and_strided_inputs(dtype):
+    """universal_attention(): 1-D and 2-D query layouts, gates arriving as permuted views (the model passes
+    [b,l,h] tensors transposed, reference main.py:29-31), keys/values as non-contiguous slices."""
+    from universal_attention_triton_amd.universal_attention import universal_attention
+    b, h, r, L, d, c = 2, 3, 2, 192, 64, 32
+    inp = orc.make_inputs(b, h, r, L, d, c, dtype=dtype, seed=31)
+    O_ref, lse_ref, g_ref = dense_reference(inp)
+    dev = {k: v.cuda() for k, v in inp.items()}
+    # strided variants holding the same values
+    src_v = dev["static_src"].reshape(b, h, L).transpose(1, 2).contiguous().transpose(1, 2).view(b, h, L // c, c)
+    dest_v = dev["static_dest"].transpose(1, 2).contiguous().transpose(1, 2)
+    kbig = torch.zeros(b, h, L // c, c, 2 * d, dtype=dtype, device="cuda")
+    kbig[..., :d] = dev["kc"]
+    leaves = [kbig[..., :d].detach().requires_grad_(), dev["vc"].detach().requires_grad_(), dev["xq"].detach().requires_grad_(),
+              src_v.detach().requires_grad_(), dest_v.detach().requires_grad_()]
+    assert not leaves[0].is_contiguous() and not leaves[3].is_contiguous() and not leaves[4].is_contiguous()
+    O = universal_attention(*leaves)
+    grads = torch.autograd.grad(O, leaves, dev["dO"].view(O.shape))
+    assert rel_err(O, O_ref) <= TOL[dtype]
+    for k, g, gr in zip(NAMES, grads, g_ref):
+        assert rel_err(g, gr) <= (TOL[dtype] if k != "kc" else max(TOL[dtype], 4e-4)), (k, rel_err(g, gr))
+    # 2-D query layout gives the same result in xq's shape
+    xq2 = dev["xq"].view(b, h, r, L // 64, 64, d)
+    O2, lse = universal_attention(dev["kc"], dev["vc"], xq2, dev["static_src"], dev["static_dest"].view(b, h, L // 64, 64), return_lse=True)
+    assert O2.shape == xq2.shape and rel_err(O2.reshape(O.shape), O_ref) <= TOL[dtype]
+    assert float((lse.cpu().double() - lse_ref).abs().max()) <= (1e-4 if dtype == torch.float32 else 2e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_second_generation_calling_convention(dtype):
+    """attention(q, k, v, causal, sm_scale, static_src, static_dest): query head j uses kv head j % H_kv and the
+    scale argument is not applied (universal_attention_kernel_opt.py:142, :84-85); head dim 80 is padded inside."""
+    from universal_attention_triton_amd.universal_attention import attention
+    B, Hkv, r, L, d = 1, 2, 3, 128, 80
+    inp = orc.make_inputs(B, Hkv, r, L, d, 32, dtype=dtype, seed=41)
+    O_ref, _, _ = dense_reference(inp)                                   # [B, Hkv, r, L, d]
+    k = inp["kc"].reshape(B, Hkv, L, d).cuda()
+    v = inp["vc"].reshape(B, Hkv, L, d).cuda()
+    q = inp["xq"].transpose(1, 2).reshape(B, r * Hkv, L, d).cuda()       # head j = rep * Hkv + kv
+    o = attention(q, k, v, True, 0.123, inp["static_src"].reshape(B, Hkv, L).cuda(), inp["static_dest"].cuda())
+    assert o.shape == (B, r * Hkv, L, d)
+    assert rel_err(o.view(B, r, Hkv, L, d).transpose(1, 2), O_ref) <= TOL[dtype]
+    with pytest.raises(AssertionError):
+        attention(q, k, v, False, 1.0, inp["static_src"].reshape(B, Hkv, L).cuda(), inp["static_dest"].cuda())
+
+
+def test_every_forward_variant_gives_the_same_result_and_autotune_records_one():
+    from universal_attention_triton_amd import ops
+    inp = orc.make_inputs(1, 2, 2, 1024 + 64, 128, 32, dtype=torch.bfloat16, seed=51)    # L not a multiple of 128/192/256
+    a = [inp[k].cuda() for k in NAMES]
+    O_ref, lse_ref, _ = dense_reference(inp)
+    n = ops.tune_variants(a[0], a[2])
+    assert n >= 2
+    results = []
+    for v in range(n):
+        ops.tune_set(a[0], a[2], v)
+        assert ops.tune_get(a[0], a[2]) == v
+        O, lse, _ = ops.fused_forward(*a)
+        torch.cuda.synchronize()
+        assert rel_err(O, O_ref) <= TOL[torch.bfloat16], (v, rel_err(O, O_ref))
+        assert float((lse.cpu().double() - lse_ref).abs().max()) <= 2e-2
+        results.append(O.float().cpu())
+    for v in range(1, n):
+        assert rel_err(results[v], results[0]) <= 2e-3, v            # same arithmetic, different summation order
+    best = ops.autotune(*a)
+    assert 0 <= best < n and ops.tune_get(a[0], a[2]) == best
+    O, _, _ = ops.fused_forward(*a)
+    assert rel_err(O, O_ref) <= TOL[torch.bfloat16]
+    ops.tune_set(a[0], a[2], 0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", ["L1", "L16", "L17_ragged", "gates_near_one", "gates_near_zero", "identical_keys", "orthogonal_keys"])
+def test_edge_cases_of_the_inputs(case, dtype):
+    """Shortest sequences, padding inside a 16-query tile, affinities at both clamps (A -> 1-1e-6 when all keys
+    coincide and the gates are 1; A = 0 when keys are orthogonal or gates vanish: then the bias is 0 and the
+    operator is causal softmax attention with scale 1)."""
+    from universal_attention_triton_amd import ops
+    b, h, r, L, d, c = 1, 2, 2, 96, 32, 32
+    gate_mean = 0.0
+    if case == "L1":
+        L, c = 1, 1
+    elif case == "L16":
+        L, c = 16, 16
+    elif case == "L17_ragged":
+        L, c = 17, 17
+    elif case == "orthogonal_keys":
+        d = 128                                                   # d >= L: every pair of keys is orthogonal
+    inp = orc.make_inputs(b, h, r, L, d, c, dtype=dtype, seed=61, gate_mean=gate_mean)
+    if case == "gates_near_one":
+        inp["static_src"].fill_(1.0); inp["static_dest"].fill_(1.0)
+    elif case == "gates_near_zero":
+        inp["static_src"].fill_(1e-30 if dtype == torch.float32 else 1e-30); inp["static_dest"].fill_(1e-30)
+    elif case == "identical_keys":
+        inp["kc"][:] = inp["kc"][:, :, :1, :1, :]
+        inp["static_src"].fill_(1.0); inp["static_dest"].fill_(1.0)
+    elif case == "orthogonal_keys":
+        k = torch.zeros(b, h, L, d)
+        k[:, :, torch.arange(L), torch.arange(L)] = 1.0
+        inp["kc"] = k.view(b, h, L // c, c, d).to(dtype)
+    print("case edge", case, dtype, flush=True)
+    O_ref, lse_ref, g_ref = dense_reference(inp)
+    dev = {k: v.cuda() for k, v in inp.items()}
+    a = [dev[k] for k in NAMES]
+    O, lse, ws = ops.fused_forward(*a, for_backward=True)
+    grads = ops.fused_backward(*a, O, lse, dev["dO"], ws=ws)
+    torch.cuda.synchronize()
+    tol = TOL[dtype]
+    assert torch.isfinite(O.float()).all() and all(torch.isfinite(g.float()).all() for g in grads)
+    assert rel_err(O, O_ref) <= tol, rel_err(O, O_ref)
+    if case in ("gates_near_zero", "orthogonal_keys"):
+        # textbook special case: no decay -> causal SDPA with scale 1
+        q = inp["xq"].double().reshape(b, h, r, L, d)
+        kk = inp["kc"].double().reshape(b, h, 1, L, d).expand(b, h, r, L, d)
+        vv = inp["vc"].double().reshape(b, h, 1, L, d).expand(b, h, r, L, d)
+        sdpa = torch.nn.functional.scaled_dot_product_attention(q, kk, vv, is_causal=True, scale=1.0)
+        assert rel_err(O, sdpa) <= tol
+    names = ("kc", "vc", "xq", "static_src", "static_dest")
+    for k, g, gr in zip(names, grads, g_ref):
+        if case == "identical_keys" and k in ("kc", "static_src", "static_dest"):
+            continue      # the affinity sits ON the clamp, where the reference's gradient convention (zero above the clamp) decides
+        if case == "orthogonal_keys" and k == "kc":
+            continue      # k.k = 0 exactly: d relu(g)^(2/3)/dg is inf * 0 in autograd (NaN); the kernels return 0
+        if float(gr.norm()) < 1e-10 * float(inp["dO"].double().norm()):
+            # zero in exact arithmetic (float64 leaves 1e-17): here terms such as dP - delta cancel only up to the
+            # summation order of fp32 dot products, and dS is rounded to the operand dtype before its products
+            assert float(g.float().norm()) <= 0.1 * tol * float(inp["dO"].float().norm()), (k, float(g.float().norm()))
+            continue
+        bar = tol if k != "kc" else max(tol, 4e-4)
+        assert rel_err(g.reshape(gr.shape), gr) <= bar, (case, k, rel_err(g.reshape(gr.shape), gr))
+
+
+def test_zero_upstream_gradient_gives_zero_gradients():
+    from universal_attention_triton_amd import ops
+    inp = orc.make_inputs(1, 2, 1, 256, 64, 64, dtype=torch.bfloat16, seed=71)
+    a = [inp[k].cuda() for k in NAMES]
+    O, lse, ws = ops.fused_forward(*a, for_backward=True)
+    grads = ops.fused_backward(*a, O, lse, torch.zeros_like(O), ws=ws)
+    for g in grads:
+        assert float(g.float().abs().max()) == 0.0

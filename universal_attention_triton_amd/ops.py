@@ -201,3 +201,27 @@ def merge_backward(mat, vec, g):
                                 d_vec.data_ptr(), _stream()), "ua_merge_bwd")
     d_mat = d4.unflatten(0, tuple(mat.shape[:-3])) if mat.dim() != 4 else d4
     return d_mat, d_vec.to(vec.dtype)
+
+
+def autotune(kc, vc, xq, static_src, static_dest, op=_lib.UA_OP_FUSED_FWD):
+    """Times the kernel variants of `op` for this problem on the current stream and records the fastest in the
+    library's table (what the reference's @triton.autotune does on first call).  Returns the variant id."""
+    kc, vc, xq, src, dest = _prep(kc, vc, xq, static_src, static_dest)
+    lib = _lib.load()
+    desc = _desc(kc, xq, op in (_lib.UA_OP_FWD, _lib.UA_OP_BWD))
+    ws = _workspace(desc, _lib.UA_OP_FUSED_BWD if op >= _lib.UA_OP_FUSED_FWD else _lib.UA_OP_BWD, xq.device)
+    v = lib.ua_autotune(ctypes.byref(desc), op, ws.data_ptr(), ws.numel(), _stream())
+    _lib.check(v, "ua_autotune")
+    return v
+
+
+def tune_variants(kc, xq, op=_lib.UA_OP_FUSED_FWD):
+    return _lib.load().ua_tune_variants(ctypes.byref(_desc(kc, xq, False)), op)
+
+
+def tune_set(kc, xq, variant, op=_lib.UA_OP_FUSED_FWD):
+    _lib.check(_lib.load().ua_tune_set(ctypes.byref(_desc(kc, xq, False)), op, variant), "ua_tune_set")
+
+
+def tune_get(kc, xq, op=_lib.UA_OP_FUSED_FWD):
+    return _lib.load().ua_tune_get(ctypes.byref(_desc(kc, xq, False)), op)
