@@ -1,0 +1,154 @@
+"""The BASELINE configurations at their full sizes on the GPU.
+
+The oracle (the reference's chunked torch operator restated, evaluated in float32 on the dtype-rounded inputs)
+checks single (batch, kv head) slices; the whole batch is covered by properties that do not depend on the size:
+  * sum_s dV[s,:] == sum_t dO[t,:] per head and query group, because every softmax row sums to one;
+  * the backward is linear in dO: doubling dO doubles every gradient bit for bit;
+  * heads holding identical inputs give bit-identical outputs and gradients (the fused path has no atomics);
+  * causality: the first T queries of a long sequence equal a run on the first T positions alone;
+  * the chunked operator followed by the merge equals the fused operator.
+"""
+import pytest
+import torch
+
+from oracle import ua_oracle as orc
+from tests.util import NAMES, TOL, rel_err
+
+pytestmark = pytest.mark.gpu
+BF16 = torch.bfloat16
+
+
+def _oracle_head(inp, z, with_backward, dtype=torch.float32):
+    """Oracle on head z = (batch index, kv head index) of `inp`: merged O and, optionally, the five gradients."""
+    bi, hi = z
+    one = [inp[k][bi:bi + 1, hi:hi + 1].to(dtype) for k in NAMES]
+    if not with_backward:
+        out, denom = orc.chunked_forward(*one)
+        return orc.merge(out, denom), None
+    leaves = [x.clone().requires_grad_() for x in one]
+    out, denom = orc.chunked_forward(*[x.detach() for x in leaves])
+    O = orc.merge(out, denom)
+    d_out, d_denom = orc.merge_backward(out, denom, inp["dO"][bi:bi + 1, hi:hi + 1].to(dtype))
+    grads = orc.chunked_backward(*[x.detach() for x in leaves], d_out, d_denom.float())
+    return O, grads
+
+
+def _run_fused(dev, backward=True, scale=1.0):
+    from universal_attention_triton_amd import ops
+    a = [dev[k] for k in NAMES]
+    O, lse, ws = ops.fused_forward(*a, for_backward=backward)
+    if not backward:
+        return O, lse, None
+    grads = ops.fused_backward(*a, O, lse, dev["dO"] * scale if scale != 1.0 else dev["dO"], ws=ws)
+    torch.cuda.synchronize()
+    return O, lse, grads
+
+
+def _check_head(O, grads, ref_O, ref_grads, z, tol):
+    bi, hi = z
+    assert rel_err(O[bi:bi + 1, hi:hi + 1], ref_O) <= tol, ("O", z, rel_err(O[bi:bi + 1, hi:hi + 1], ref_O))
+    if grads is None:
+        return
+    for k, g, gr in zip(NAMES, grads, ref_grads):
+        e = rel_err(g[bi:bi + 1, hi:hi + 1].reshape(gr.shape), gr)
+        assert e <= tol, (k, z, e)
+
+
+def _check_dv_identity(dev, grads, tol):
+    dv = grads[1].float().reshape(*dev["vc"].shape[:2], -1, dev["vc"].shape[-1]).sum(2)          # [b,h,d]
+    ref = dev["dO"].float().sum(dim=(2, 3))                                                       # over groups and queries
+    assert rel_err(dv, ref) <= tol, rel_err(dv, ref)
+
+
+def test_config1_bf16_forward_b2_h16_L2048_d64_chunk128():
+    from universal_attention_triton_amd import ops
+    inp = orc.make_inputs(2, 16, 1, 2048, 64, 128, dtype=BF16, seed=1001)
+    dev = {k: v.cuda() for k, v in inp.items()}
+    print("case cfg1 fused + chunked forward", flush=True)
+    O, lse, _ = _run_fused(dev, backward=False)
+    out, denom, _ = ops.chunked_forward(*[dev[k] for k in NAMES])
+    O2 = ops.merge_forward(out, denom)
+    torch.cuda.synchronize()
+    assert rel_err(O2, O) <= TOL[BF16]                      # chunked + merge == fused, every head
+    assert float(O.float().abs().amax()) <= float(inp["vc"].float().abs().amax()) * 1.01   # convex combinations of V
+    for z in ((0, 0), (1, 15)):
+        ref_O, _ = _oracle_head(inp, z, False)
+        _check_head(O, None, ref_O, None, z, TOL[BF16])
+        ref_out, ref_denom = orc.chunked_forward(*[inp[k][z[0]:z[0] + 1, z[1]:z[1] + 1].float() for k in NAMES])
+        assert rel_err(out[z[0]:z[0] + 1, z[1]:z[1] + 1], ref_out) <= TOL[BF16]
+        assert rel_err(denom[z[0]:z[0] + 1, z[1]:z[1] + 1], ref_denom) <= TOL[BF16]
+
+
+def test_config2_headline_bf16_forward_backward_h32_L8192_d128():
+    inp = orc.make_inputs(1, 32, 1, 8192, 128, 128, dtype=BF16, seed=1002)
+    # heads 30 and 31 are copies of heads 0 and 1: identical inputs must give identical bits
+    for k in list(NAMES) + ["dO"]:
+        inp[k][:, 30:32] = inp[k][:, 0:2]
+    dev = {k: v.cuda() for k, v in inp.items()}
+    print("case cfg2 fused forward + backward", flush=True)
+    O, lse, grads = _run_fused(dev)
+    for t in (O, lse) + tuple(grads):
+        assert torch.isfinite(t.float()).all()
+        assert torch.equal(t[:, 30:32], t[:, 0:2])
+    _check_dv_identity(dev, grads, TOL[BF16])
+    print("case cfg2 linearity", flush=True)
+    _, _, grads2 = _run_fused(dev, scale=2.0)
+    for g, g2 in zip(grads, grads2):
+        assert torch.equal(g2.float(), 2.0 * g.float())
+    print("case cfg2 oracle head", flush=True)
+    z = (0, 17)
+    ref_O, ref_grads = _oracle_head(inp, z, True)
+    _check_head(O, grads, ref_O, ref_grads, z, TOL[BF16])
+
+
+def test_config3_grouped_queries_h8_r4_L4096_d128():
+    inp = orc.make_inputs(1, 8, 4, 4096, 128, 128, dtype=BF16, seed=1003)
+    for k in list(NAMES) + ["dO"]:
+        inp[k][:, 7] = inp[k][:, 2]
+    dev = {k: v.cuda() for k, v in inp.items()}
+    print("case cfg3 fused forward + backward", flush=True)
+    O, lse, grads = _run_fused(dev)
+    for t in (O, lse) + tuple(grads):
+        assert torch.isfinite(t.float()).all()
+        assert torch.equal(t[:, 7], t[:, 2])
+    _check_dv_identity(dev, grads, TOL[BF16])
+    _, _, grads2 = _run_fused(dev, scale=2.0)
+    for g, g2 in zip(grads, grads2):
+        assert torch.equal(g2.float(), 2.0 * g.float())
+    print("case cfg3 oracle head", flush=True)
+    z = (0, 5)
+    ref_O, ref_grads = _oracle_head(inp, z, True)
+    _check_head(O, grads, ref_O, ref_grads, z, TOL[BF16])
+
+
+def test_config4_long_context_h8_L32768_d128_gates_near_one():
+    L, T = 32768, 4096
+    inp = orc.make_inputs(1, 8, 1, L, 128, 128, dtype=BF16, seed=1004, gate_mean=2.0)
+    for k in list(NAMES) + ["dO"]:
+        inp[k][:, 6] = inp[k][:, 1]
+    dev = {k: v.cuda() for k, v in inp.items()}
+    print("case cfg4 fused forward + backward", flush=True)
+    O, lse, grads = _run_fused(dev)
+    for t in (O, lse) + tuple(grads):
+        assert torch.isfinite(t.float()).all()
+        assert torch.equal(t[:, 6], t[:, 1])
+    _check_dv_identity(dev, grads, TOL[BF16])
+    # causality: queries < T see only keys < T
+    print("case cfg4 causal prefix", flush=True)
+    n = T // 128
+    short = {"kc": dev["kc"][:, :, :n].contiguous(), "vc": dev["vc"][:, :, :n].contiguous(), "xq": dev["xq"][:, :, :, :T].contiguous(),
+             "static_src": dev["static_src"][:, :, :n].contiguous(), "static_dest": dev["static_dest"][:, :, :T].contiguous(),
+             "dO": dev["dO"][:, :, :, :T].contiguous()}
+    Os, lses, _ = _run_fused(short, backward=False)
+    torch.cuda.synchronize()
+    assert torch.equal(Os, O[:, :, :, :T]) and torch.equal(lses, lse[:, :, :, :T])
+    # the reference operator on one head of the prefix, and of the whole sequence (forward)
+    print("case cfg4 oracle prefix head", flush=True)
+    z = (0, 3)
+    cpu_short = {k: v.cpu() for k, v in short.items()}
+    ref_O, ref_grads = _oracle_head(cpu_short, z, True)
+    _, _, gshort = _run_fused(short)
+    _check_head(Os, gshort, ref_O, ref_grads, z, TOL[BF16])
+    print("case cfg4 oracle full-length head, forward", flush=True)
+    ref_O, _ = _oracle_head(inp, z, False)
+    _check_head(O, None, ref_O, None, z, TOL[BF16])
