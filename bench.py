@@ -23,11 +23,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 CONFIGS = {  # BASELINE.json configs: b, h, r, L, d, chunk, dtype, gate_mean, passes
-    0: dict(b=1, h=4, r=1, L=512, d=64, c=64, dtype="fp32", mu=0.0),
-    1: dict(b=2, h=16, r=1, L=2048, d=64, c=128, dtype="bf16", mu=0.0),
-    2: dict(b=1, h=32, r=1, L=8192, d=128, c=128, dtype="bf16", mu=0.0),
-    3: dict(b=1, h=8, r=4, L=4096, d=128, c=128, dtype="bf16", mu=0.0),
-    4: dict(b=1, h=8, r=1, L=32768, d=128, c=128, dtype="bf16", mu=2.0),
+    0: dict(b=1, h=4, r=1, L=512, d=64, c=64, dtype="fp32", mu=0.0, bwd=False),
+    1: dict(b=2, h=16, r=1, L=2048, d=64, c=128, dtype="bf16", mu=0.0, bwd=False),
+    2: dict(b=1, h=32, r=1, L=8192, d=128, c=128, dtype="bf16", mu=0.0, bwd=True),
+    3: dict(b=1, h=8, r=4, L=4096, d=128, c=128, dtype="bf16", mu=0.0, bwd=True),
+    4: dict(b=1, h=8, r=1, L=32768, d=128, c=128, dtype="bf16", mu=2.0, bwd=True),
 }
 PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}   # MI355X dense MFMA peaks
 
@@ -58,17 +58,21 @@ def cpu_baseline(cfg, index, budget_s=10.0):
         t0 = time.time()
         out, denom = orc.chunked_forward(*[inp[k] for k in names])
         O = orc.merge(out, denom)
-        d_out, d_denom = orc.merge_backward(out, denom, inp["dO"])
-        orc.chunked_backward(*[inp[k] for k in names], d_out, d_denom.float())
+        if cfg["bwd"]:
+            d_out, d_denom = orc.merge_backward(out, denom, inp["dO"])
+            orc.chunked_backward(*[inp[k] for k in names], d_out, d_denom.float())
+            del d_out, d_denom
         spent += time.time() - t0
         heads += 1
-        del O, out, denom, d_out, d_denom
+        del O, out, denom
     f, bw = flops(dict(cfg, b=1, h=1))
+    if not cfg["bwd"]:
+        bw = 0
     return {"value": round(heads * (f + bw) / spent / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
             "kind": "port", "seconds": round(spent, 2), "ms_per_step_extrapolated": round(spent / heads * cfg["b"] * cfg["h"] * 1e3, 1),
-            "sample": "%d of %d kv heads of the workload (each b=1,h=1,r=%d,L=%d,d=%d,chunk=%d): chunked forward + merge + "
-                      "backward of the oracle, heads run one after the other"
-                      % (heads, cfg["b"] * cfg["h"], cfg["r"], cfg["L"], cfg["d"], cfg["c"])}
+            "sample": "%d of %d kv heads of the workload (each b=1,h=1,r=%d,L=%d,d=%d,chunk=%d): chunked forward + merge%s "
+                      "of the oracle, heads run one after the other"
+                      % (heads, cfg["b"] * cfg["h"], cfg["r"], cfg["L"], cfg["d"], cfg["c"], " + backward" if cfg["bwd"] else "")}
 
 
 def main():
@@ -97,9 +101,14 @@ def main():
     leaves = [inp[k].cuda().requires_grad_() for k in names]
     dO = inp["dO"].cuda()
 
-    def step():
-        O = universal_attention(*leaves)
-        return torch.autograd.grad(O, leaves, dO)
+    if cfg["bwd"]:
+        def step():
+            O = universal_attention(*leaves)
+            return torch.autograd.grad(O, leaves, dO)
+    else:
+        def step():
+            with torch.no_grad():
+                return universal_attention(*leaves)
 
     if args.calibrate_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").fill_(1.0)
@@ -122,19 +131,23 @@ def main():
     prof = _lib.prof_collect()
     ms = elapsed * 1e3 / args.steps
     f_fwd, f_bwd = flops(cfg)
+    if not cfg["bwd"]:
+        f_bwd = 0
+    dom = "k_bwd_keys" if cfg["bwd"] else "k_fwd_fused"
     kern = {k: round(v[1] / v[0], 4) for k, v in prof.items()}
-    dom_ms = prof["k_bwd_keys"][1] / prof["k_bwd_keys"][0]
+    dom_ms = prof[dom][1] / prof[dom][0]
     peak = PEAK_TFLOPS[cfg["dtype"]]
-    achieved = kernel_flops(cfg, "k_bwd_keys") / (dom_ms * 1e-3) / 1e12
+    achieved = kernel_flops(cfg, dom) / (dom_ms * 1e-3) / 1e12
     out = {
         "metric": "fwd+bwd ms and TFLOP/s (bf16, L=8192, d=128) on 1 MI355X; % MFMA peak", "value": round((f_fwd + f_bwd) / (ms * 1e-3) / 1e12, 2),
         "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": cfg["dtype"], "data": "synthetic",
-        "config": {"workload": "BASELINE config %d: fused fwd+bwd b=%d h=%d r=%d L=%d d=%d, upstream dO like the output"
-                               % (args.config, cfg["b"], cfg["h"], cfg["r"], cfg["L"], cfg["d"]),
+        "config": {"workload": "BASELINE config %d: fused %s b=%d h=%d r=%d L=%d d=%d%s"
+                               % (args.config, "fwd+bwd" if cfg["bwd"] else "fwd only", cfg["b"], cfg["h"], cfg["r"], cfg["L"], cfg["d"],
+                                  ", upstream dO like the output" if cfg["bwd"] else ""),
                    "pct_of_mfma_peak": round(100 * (f_fwd + f_bwd) / (ms * 1e-3) / 1e12 / peak, 2),
                    "kernel_ms": kern},
-        "roofline": {"bound": "mfma", "kernel": "k_bwd_keys", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
+        "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
                      "frac": round(achieved / peak, 4), "traffic": None},
     }
     if not args.no_cpu:
