@@ -273,6 +273,50 @@ __device__ __forceinline__ float block_suffix(f32x16& x, int hi) {
   return run;
 }
 
+// ---------------------------------------------------------------------------------
+// Wave-private staging of a [32 keys][16 queries] tile: written from result-tile registers (lane = key, its 4
+// consecutive queries: ONE store) and read back transposed as the A operand (row = query, k = the 32 keys) of a
+// product contracting over those keys.  bf16 uses ds_read_tr16_b64 (two reads per operand); fp32 has no
+// transposing read and keeps a [16 queries][32 keys] tile written element by element.
+// ---------------------------------------------------------------------------------
+typedef short v4s16 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) v4s16* lds_v4s16_t;
+template <class T> struct StageT;
+template <> struct StageT<bf16> {
+  static constexpr int BYTES = 1024;
+  // 32-byte rows (one per key); the two 128-byte halves of odd 256-byte blocks are swapped so that the
+  // transposing reads of lane groups 0 and 1 (keys 0-3 and 8-11) fall on different banks
+  __device__ __forceinline__ static int addr(int row, int byte) { return (row * 32 + byte) ^ (((row >> 3) & 1) << 7); }
+  // x[v] = value at (query 4g + v, key `row`)
+  __device__ __forceinline__ static void put(char* base, int row, int g, const f32x4& x) {
+    typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+    bf16x4 p;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) p[v] = (bf16)x[v];
+    *reinterpret_cast<bf16x4*>(base + addr(row, 8 * g)) = p;
+  }
+  __device__ __forceinline__ static Frag<bf16> get(char* base, int lane) {
+    const int i = lane & 15, G = lane >> 4;
+    const v4s16 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s16_t)(base + addr(8 * G + (i >> 2), 8 * (i & 3))));
+    const v4s16 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s16_t)(base + addr(8 * G + 4 + (i >> 2), 8 * (i & 3))));
+    Frag<bf16> f;
+    reinterpret_cast<v4s16*>(&f)[0] = lo;
+    reinterpret_cast<v4s16*>(&f)[1] = hi;
+    return f;
+  }
+};
+template <> struct StageT<float> {
+  static constexpr int STRIDE = 36, BYTES = 16 * STRIDE * 4;
+  __device__ __forceinline__ static void put(char* base, int row, int g, const f32x4& x) {
+    float* p = reinterpret_cast<float*>(base);
+#pragma unroll
+    for (int v = 0; v < 4; ++v) p[(4 * g + v) * STRIDE + row] = x[v];
+  }
+  __device__ __forceinline__ static Frag<float> get(char* base, int lane) {
+    return ld8(reinterpret_cast<const float*>(base) + (lane & 15) * STRIDE + 8 * (lane >> 4));
+  }
+};
+
 // ---- scans over the 32 queries of two 16x16 tiles (lane = key l%16, lane group g = l/16 holds t = 4g+v) ----
 struct GroupMasks { float g1, g2, n1, n2; };    // g1 = g&1, g2 = g>>1 as floats, n* their complements
 __device__ __forceinline__ GroupMasks group_masks(int lane) {

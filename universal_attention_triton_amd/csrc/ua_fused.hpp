@@ -164,10 +164,11 @@ __global__ void __launch_bounds__(64 * NW) k_fwd_fused2(const T* __restrict__ Qp
                                                     int R, int L, int Lp, int d) {
   using TN = Tile<T, 32, D>;
   using TT = Tile<T, D, 32>;
-  constexpr int NK = D / 32, ND = D / 16, LS = TN::STRIDE, TS = TT::STRIDE, PS = lds_stride<T>(64);
+  constexpr int NK = D / 32, ND = D / 16, LS = TN::STRIDE, TS = TT::STRIDE;
+  using ST = StageT<T>;
   constexpr int TILES = 2 * TN::BYTES + 2 * TT::BYTES, SB = TILES + NW * 1024;   // + per wave [C row: 64f][lsrc: 64f]
   UA_STAGES(SB);
-  __shared__ __attribute__((aligned(16))) T sPbuf[NW * 16 * PS];
+  __shared__ __attribute__((aligned(256))) char sPbuf[NW * 2 * ST::BYTES];
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
   int bx, zq;
   xcd_map(bx, zq);
@@ -175,7 +176,7 @@ __global__ void __launch_bounds__(64 * NW) k_fwd_fused2(const T* __restrict__ Qp
   const int jt = gridDim.x - 1 - bx;
   const bool live = NW * jt + w < nT16;                      // the last workgroup may hold waves past the end
   const int tq = live ? NW * jt + w : nT16 - 1;             // 16-query tile of this wave
-  T* sPw = sPbuf + w * 16 * PS;
+  char* sPw = sPbuf + w * 2 * ST::BYTES;     // P of the two 32-key halves of a step
   const GroupMasks gm = group_masks(lane);
   Stager<TN, NW> stN;
   Stager<TT, NW> stT;
@@ -271,18 +272,19 @@ __global__ void __launch_bounds__(64 * NW) k_fwd_fused2(const T* __restrict__ Qp
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
+      f32x4 p;
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
-        const float p = __builtin_amdgcn_exp2f(s2[j][v] - m[v]);
-        ls[v] += p;
-        sPw[(4 * g + v) * PS + 16 * j + col] = cvt<T>(p);
+        p[v] = __builtin_amdgcn_exp2f(s2[j][v] - m[v]);
+        ls[v] += p[v];
       }
+      ST::put(sPw + (j >> 1) * ST::BYTES, 16 * (j & 1) + col, g, p);
     }
 #pragma unroll
     for (int kq = 0; kq < 2; ++kq) {                   // 32 keys per k-step
       if (!MASKED || 4 * kt + 2 * kq <= tq) {
         const T* sV = reinterpret_cast<const T*>(base + 2 * TN::BYTES + kq * TT::BYTES);
-        const Frag<T> pa = ld8(sPw + col * PS + 32 * kq + 8 * g);
+        const Frag<T> pa = ST::get(sPw + kq * ST::BYTES, lane);
 #pragma unroll
         for (int n = 0; n < ND; ++n) mma16(o[n], pa, ld8(sV + TT::at(n, col, 0, g)));
       }
@@ -516,16 +518,17 @@ template <class T, int D, int NST>
 __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restrict__ dq, int d) {
   using TN = Tile<T, 32, D>;
   using TT = Tile<T, D, 32>;
-  constexpr int NK = D / 32, ND = D / 16, LS = TN::STRIDE, TS = TT::STRIDE, XS = lds_stride<T>(64);
+  constexpr int NK = D / 32, ND = D / 16, LS = TN::STRIDE, TS = TT::STRIDE;
+  using ST = StageT<T>;
   constexpr int TILES = 4 * TN::BYTES + 2 * TT::BYTES, SB = TILES + 8 * 1024;   // + per wave [C: 64f][lsrc: 64f][Dsuf: 64f]
   UA_STAGES(SB);
-  __shared__ __attribute__((aligned(16))) T sXbuf[8 * 16 * XS];
+  __shared__ __attribute__((aligned(256))) char sXbuf[8 * 2 * ST::BYTES];
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
   int bx, zk;
   xcd_map(bx, zk);
   const int Lp = a.Lp, L = a.L, nT16 = Lp / 16, R = a.R;
   const int jt = gridDim.x - 1 - bx, tq = 8 * jt + w;
-  T* sX = sXbuf + w * 16 * XS;
+  char* sX = sXbuf + w * 2 * ST::BYTES;      // [dS of a 32-key half][dg of that half]
   const GroupMasks gm = group_masks(lane);
   Stager<TN, 8> stN;
   Stager<TT, 8> stT;
@@ -584,7 +587,6 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
       constexpr bool MASKED = decltype(masked_c)::value;
       const float* stats = reinterpret_cast<const float*>(base + TILES + w * 1024);
       // the 64 keys of the step are handled as two halves of 32 (= one contraction step of the column products);
-      // sX holds [16 queries][dS of the half: 32][dg of the half: 32]
 #pragma unroll
       for (int kq = 0; kq < 2; ++kq) {
         if (MASKED && 4 * kti + 2 * kq > tq) continue;     // wave-uniform: the whole half lies after this wave's queries
@@ -639,16 +641,12 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
               dg[v] = decay_grad(dl, aff[v], gk[v]);
             }
           }
-          const int pc = jj ? pc1 : pc0;
-#pragma unroll
-          for (int v = 0; v < 4; ++v) {
-            sX[(4 * g + v) * XS + pc] = cvt<T>(dS[v]);
-            sX[(4 * g + v) * XS + 32 + pc] = cvt<T>(dg[v]);
-          }
+          ST::put(sX, jj ? pc1 : pc0, g, dS);
+          ST::put(sX + ST::BYTES, jj ? pc1 : pc0, g, dg);
         }
         // dQ += dS^T K,  dkcol += dg^T K   (contraction over the 32 keys of the half)
         const T* sKT = reinterpret_cast<const T*>(base + 4 * TN::BYTES + kq * TT::BYTES);
-        const Frag<T> as = ld8(sX + col * XS + 8 * g), ag = ld8(sX + col * XS + 32 + 8 * g);
+        const Frag<T> as = ST::get(sX, lane), ag = ST::get(sX + ST::BYTES, lane);
 #pragma unroll
         for (int n = 0; n < ND; ++n) {
           const Frag<T> kb = ld8(sKT + TT::at(n, col, 0, g));
