@@ -266,7 +266,7 @@ __global__ void __launch_bounds__(64 * NW) k_bwd_keys(BwdArgs<T> a) {
 
 // Combine partial gradients into the caller's contiguous tensors:
 //   dk [Zk][L][d], dv [Zk][L][d], dq [Zq][L][d], dsrc [Zk][L], ddest [Zk][L]
-// grid (ceil(L/4), max(Zk, Zq)); one wave per row.
+// grid (ceil(L/4), max(Zk, Zq)); one wave per row.  The fp32 partial gradients are row-major [Z][Lp][D].
 template <class T>
 __global__ void __launch_bounds__(256) k_bwd_finish(const float* __restrict__ dKrow, const float* __restrict__ dVrow,
                                                     const float* __restrict__ dKdacc, const float* __restrict__ dQacc,
@@ -274,7 +274,7 @@ __global__ void __launch_bounds__(256) k_bwd_finish(const float* __restrict__ dK
                                                     const T* __restrict__ src, const T* __restrict__ dest,
                                                     T* __restrict__ dk, T* __restrict__ dv, T* __restrict__ dq,
                                                     T* __restrict__ dsrc, T* __restrict__ ddest, int Zk, int Zq, int L,
-                                                    int Lp, int D, int d) {
+                                                    int Lp, int D, int d, int tiled) {
   const int z = blockIdx.y, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + wave;
   if (t >= L) return;
@@ -287,7 +287,9 @@ __global__ void __launch_bounds__(256) k_bwd_finish(const float* __restrict__ dK
     for (int c = lane; c < d; c += 64) {
       const long i = ((long)z * Lp + t) * D + c;
       const float kd = dKdacc[i];
-      dot += kd * (float)Kp[i];
+      // the packed keys are row-major in chunked mode and tiled (nat_off) in fused mode
+      const long ik = !tiled ? i : (D == 64 ? nat_off<64>(z, Lp, t, c) : nat_off<128>(z, Lp, t, c));
+      dot += kd * (float)Kp[ik];
       dk[((long)z * L + t) * d + c] = cvt<T>(dKrow[i] + kd);
       dv[((long)z * L + t) * d + c] = cvt<T>(dVrow[i]);
     }

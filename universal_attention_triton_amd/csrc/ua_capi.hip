@@ -108,14 +108,15 @@ ua::RowsView chunked_view(const ua_chunked& c, int nch) {
 }
 ua::RowsView null_view() { ua::RowsView v{}; v.inner = 1; v.H = v.R = v.N = 1; return v; }
 
-template <class T>
-hipError_t pack_t(int D, const ua::RowsView& x, void* nat, void* tr, int d, int L, int Lp, int Z, int tr_mode, hipStream_t s) {
-  if (D == 64) hipLaunchKernelGGL((ua::k_pack<T, 64>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp, tr_mode);
-  else hipLaunchKernelGGL((ua::k_pack<T, 128>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp, tr_mode);
-  return hipGetLastError();
-}
 // tr_mode: column order of the transposed copy inside each group of 32 positions
 enum { TR_PERM16 = 0, TR_PERM32 = 1, TR_NATURAL = 2 };
+template <class T>
+hipError_t pack_t(int D, const ua::RowsView& x, void* nat, void* tr, int d, int L, int Lp, int Z, int tr_mode, hipStream_t s) {
+  const int tiled = tr_mode != TR_PERM16;      // the fused kernels read tiled working tensors, the chunked ones row-major
+  if (D == 64) hipLaunchKernelGGL((ua::k_pack<T, 64>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp, tr_mode, tiled);
+  else hipLaunchKernelGGL((ua::k_pack<T, 128>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp, tr_mode, tiled);
+  return hipGetLastError();
+}
 hipError_t pack(int dtype, int D, const ua::RowsView& x, void* nat, void* tr, int d, int L, int Lp, int Z, int tr_mode, hipStream_t s) {
   return dtype == UA_BF16 ? pack_t<ua::bf16>(D, x, nat, tr, d, L, Lp, Z, tr_mode, s) : pack_t<float>(D, x, nat, tr, d, L, Lp, Z, tr_mode, s);
 }
@@ -209,7 +210,7 @@ int run_fused_fwd_kernels(const ua_desc& d, const Layout& l, char* ws, void* O, 
   {
     UA_PROF("k_carry", s);
     UA_HIP(ua::launch_carry(d.dtype, l.D, ws + l.Kp, (const float*)(ws + l.lsrc), (const float*)(ws + l.ldest),
-                            (float*)(ws + l.C), l.Lp, l.Zk, s));
+                            (float*)(ws + l.C), l.Lp, l.Zk, 1, s));
   }
   UA_PROF("k_fwd_fused", s);
   UA_HIP(ua::launch_fwd_fused(d.dtype, l.D, variant, ws + l.Qp, ws + l.Kp, ws + l.VT, (const float*)(ws + l.lsrc),
@@ -225,7 +226,7 @@ hipError_t finish_t(const Layout& l, const ua_desc& d, char* ws, bool chunked, c
   hipLaunchKernelGGL((ua::k_bwd_finish<T>), dim3((d.L + 3) / 4, Z), dim3(256), 0, s, (const float*)(ws + l.dKrow),
                      (const float*)(ws + l.dVrow), (const float*)(ws + l.dKdacc), chunked ? (const float*)(ws + l.dQacc) : nullptr,
                      (const float*)(ws + l.dsrc_raw), (const T*)(ws + l.Kp), (const T*)src, (const T*)dest, (T*)dk, (T*)dv,
-                     (T*)dq, (T*)dsrc, (T*)ddest, l.Zk, l.Zq, d.L, l.Lp, l.D, d.d);
+                     (T*)dq, (T*)dsrc, (T*)ddest, l.Zk, l.Zq, d.L, l.Lp, l.D, d.d, chunked ? 0 : 1);
   return hipGetLastError();
 }
 
@@ -306,7 +307,7 @@ int ua_fused_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, cons
   if (!ws_has_fwd) {
     if (int e = pack_inputs(d, l, false, kc, vc, xq, static_src, static_dest, w, s)) return e;
     UA_HIP(ua::launch_carry(d.dtype, l.D, w + l.Kp, (const float*)(w + l.lsrc), (const float*)(w + l.ldest),
-                            (float*)(w + l.C), l.Lp, l.Zk, s));
+                            (float*)(w + l.C), l.Lp, l.Zk, 1, s));
   }
   const long rowsz = (long)d.L * d.d;
   const ua::RowsView Ov = contiguous_view(O, rowsz, d.d), dOv = contiguous_view(dO, rowsz, d.d);
@@ -355,7 +356,7 @@ int ua_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
                                   (const float*)(w + l.ldest), nullptr, nullptr, (float*)(w + l.lse2), 0, 0, 0, 0, d.r, d.L, l.Lp, d.d, d.chunk, l.nch, l.Zk, s));
   }
   UA_HIP(ua::launch_carry(d.dtype, l.D, w + l.Kp, (const float*)(w + l.lsrc), (const float*)(w + l.ldest),
-                          (float*)(w + l.C), l.Lp, l.Zk, s));
+                          (float*)(w + l.C), l.Lp, l.Zk, 0, s));
   const ua::RowsView outv = chunked_view(*out, l.nch);
   ua_chunked gmut = *g_out;
   const ua::RowsView gv = chunked_view(gmut, l.nch), none = null_view();

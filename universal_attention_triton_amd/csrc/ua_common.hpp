@@ -132,13 +132,28 @@ __device__ __forceinline__ void stage_tile(T* __restrict__ lds, const T* __restr
 // ---------------------------------------------------------------------------------
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
-// A [ROWS][COLS] operand tile in LDS, filled by asynchronous global->LDS loads in units of 16-byte chunks.
-// ds_read_b128 serves 16 lanes per cycle (256 bytes over 64 banks).  An MFMA operand read (lane = row l%16,
-// chunk l/16 of a 32-wide k-step) from rows padded by one chunk takes 8 cycles instead of 4 on this part; storing
-// payload chunk c of row r at position c ^ swz(r) in UNPADDED rows was measured conflict-free for rows of 16 and
-// 8 chunks with swz = r mod chunks-per-row, and for rows of 4 chunks with swz = (r >> 1) & 3.  bf16 tiles use
-// that; fp32 tiles keep one padding chunk per row.
-template <class T, int ROWS, int COLS> struct Tile {
+// A [ROWS][COLS] operand tile in LDS, filled by asynchronous global->LDS loads in units of 16-byte chunks, and
+// read as MFMA operands: lane l takes the 8 k-values of k-group 4q + l/16 of row 16*blk + l%16.
+//
+// CM = true (the fused kernels): k-group-major order, element (row, k-group kg, e) at ((kg*ROWS + row)*8 + e).
+// The 16 lanes that ds_read_b128 serves together (one k-group, 16 consecutive rows) then read 256 CONTIGUOUS
+// bytes.  Measured on this part: that costs clearly less than 16 chunks scattered over 16 rows, even when the
+// scattered chunks are bank-conflict free.  The working tensors in HBM use the same order tile by tile
+// (nat_off / tr_off below), so a tile is one contiguous block on both sides of the copy.
+//
+// CM = false (carry pre-pass of the chunked mode, which reads row-major working tensors): row-major rows;
+// bf16 rows are unpadded with payload chunk c of row r stored at position c ^ swz(r) (bank-conflict free),
+// fp32 rows keep one padding chunk.
+template <class T, int ROWS, int COLS, bool CM = true> struct Tile;
+template <class T, int ROWS, int COLS> struct Tile<T, ROWS, COLS, true> {
+  static constexpr bool CONTIG = true;
+  static constexpr int BYTES = ROWS * COLS * (int)sizeof(T);
+  static constexpr int NINSTR = BYTES / 1024;
+  static_assert(BYTES % 1024 == 0, "a tile is copied in units of 1 KB");
+  __device__ __forceinline__ static int at(int blk, int col, int q, int g) { return ((4 * q + g) * ROWS + 16 * blk + col) * 8; }
+};
+template <class T, int ROWS, int COLS> struct Tile<T, ROWS, COLS, false> {
+  static constexpr bool CONTIG = false;
   static constexpr bool SWZ = sizeof(T) == 2;
   static constexpr int STRIDE = SWZ ? COLS : COLS + kPad16 / (int)sizeof(T);   // elements per row
   static constexpr int CPR = STRIDE * (int)sizeof(T) / 16;             // 16-byte chunks per row
@@ -147,7 +162,6 @@ template <class T, int ROWS, int COLS> struct Tile {
   static constexpr int BYTES = NINSTR * 1024;                          // LDS footprint
   static_assert(!SWZ || CPP == 4 || CPP == 8 || CPP == 16, "swizzle is defined for rows of 4, 8 or 16 chunks");
   __host__ __device__ static constexpr int swz(int r) { return CPP >= 8 ? (r & (CPP - 1)) : ((r >> 1) & (CPP - 1)); }
-  // element offset of the 8 k-values [32q + 8g, 32q + 8g + 8) of row 16*blk + col  (col = lane & 15, g = lane >> 4)
   __device__ __forceinline__ static int at(int blk, int col, int q, int g) {
     if constexpr (SWZ) {
       if constexpr (CPP >= 8) return (16 * blk + col) * STRIDE + (((4 * q + g) ^ (col & (CPP - 1))) << 3);
@@ -157,20 +171,33 @@ template <class T, int ROWS, int COLS> struct Tile {
     }
   }
 };
+// element offsets inside the tiled working tensors of the fused kernels (Lp is a multiple of 32):
+//   natural    [Z][Lp/32][D/8][32 positions][8 features]     element (position row, feature dd)
+//   transposed [Z][Lp/32][4][D features][8 positions]         element (feature dd, column p of tile `tile`)
+template <int D> __host__ __device__ __forceinline__ constexpr long nat_off(long z, int Lp, int row, int dd) {
+  return ((z * (Lp >> 5) + (row >> 5)) * (D / 8) + (dd >> 3)) * 256 + ((row & 31) << 3) + (dd & 7);
+}
+template <int D> __host__ __device__ __forceinline__ constexpr long tr_off(long z, int Lp, int dd, int tile, int p) {
+  return ((z * (Lp >> 5) + tile) * 4 + (p >> 3)) * (D * 8) + dd * 8 + (p & 7);
+}
 
 template <class TILE, int NWAVES> struct Stager {
   static constexpr int PER = (TILE::NINSTR + NWAVES - 1) / NWAVES;
   int off[PER];
-  // gstride_bytes: distance between consecutive rows of the tile in global memory
+  // gstride_bytes: distance between consecutive rows of the tile in global memory (row-major tiles only)
   __device__ __forceinline__ void init(int w, int lane, long gstride_bytes, int rows) {
 #pragma unroll
     for (int k = 0; k < PER; ++k) {
       const int n = (w + k * NWAVES) * 64 + lane;
-      int row = n / TILE::CPR, c = n - row * TILE::CPR;
-      row = row < rows ? row : rows - 1;
-      if constexpr (TILE::SWZ) c ^= TILE::swz(row);
-      else c = c < TILE::CPP ? c : TILE::CPP - 1;
-      off[k] = (int)(row * gstride_bytes) + c * 16;
+      if constexpr (TILE::CONTIG) {
+        off[k] = n * 16;
+      } else {
+        int row = n / TILE::CPR, c = n - row * TILE::CPR;
+        row = row < rows ? row : rows - 1;
+        if constexpr (TILE::SWZ) c ^= TILE::swz(row);
+        else c = c < TILE::CPP ? c : TILE::CPP - 1;
+        off[k] = (int)(row * gstride_bytes) + c * 16;
+      }
     }
   }
   __device__ __forceinline__ void issue(void* lds_tile, const void* gtile, int w) const {

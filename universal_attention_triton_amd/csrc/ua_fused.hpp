@@ -79,11 +79,12 @@ struct TrueC { static constexpr bool value = true; };
 struct FalseC { static constexpr bool value = false; };
 
 // grid (Lp/128, Zk), 8 waves; wave w owns keys 16*(8*bx+w)..+15 and sweeps the 32-query blocks from its own on.
-template <class T, int D, int NST>
+// CM: the key tensor is stored in tiled k-group-major order (fused mode) rather than row-major (chunked mode).
+template <class T, int D, int NST, bool CM>
 __global__ void __launch_bounds__(512) k_carry2(const T* __restrict__ Kp, const float* __restrict__ lsrc,
                                                 const float* __restrict__ ldest, float* __restrict__ C, int Lp) {
-  using TN = Tile<T, 32, D>;
-  constexpr int NK = D / 32, LS = TN::STRIDE, SB = TN::BYTES + 1024;   // tile + [ldest of the block: 32 floats]
+  using TN = Tile<T, 32, D, CM>;
+  constexpr int NK = D / 32, SB = TN::BYTES + 1024;   // tile + [ldest of the block: 32 floats]
   UA_STAGES(SB);
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
   int bx, z;
@@ -95,9 +96,9 @@ __global__ void __launch_bounds__(512) k_carry2(const T* __restrict__ Kp, const 
   st.init(w, lane, D * (long)sizeof(T), 32);
   Frag<T> ks[NK];
   {
-    const T* krow = Kp + ((long)z * Lp + spos) * D + 8 * g;
 #pragma unroll
-    for (int q = 0; q < NK; ++q) ks[q] = ld8(krow + 32 * q);
+    for (int q = 0; q < NK; ++q)
+      ks[q] = ld8(Kp + (CM ? nat_off<D>(z, Lp, spos, 32 * q + 8 * g) : ((long)z * Lp + spos) * D + 32 * q + 8 * g));
   }
   const float la = lsrc[(long)z * Lp + spos];
   float carry = 0.f;
@@ -164,7 +165,7 @@ __global__ void __launch_bounds__(64 * NW) k_fwd_fused2(const T* __restrict__ Qp
                                                     int R, int L, int Lp, int d) {
   using TN = Tile<T, 32, D>;
   using TT = Tile<T, D, 32>;
-  constexpr int NK = D / 32, ND = D / 16, LS = TN::STRIDE, TS = TT::STRIDE;
+  constexpr int NK = D / 32, ND = D / 16;
   using ST = StageT<T>;
   constexpr int TILES = 2 * TN::BYTES + 2 * TT::BYTES, SB = TILES + NW * 1024;   // + per wave [C row: 64f][lsrc: 64f]
   UA_STAGES(SB);
@@ -185,10 +186,11 @@ __global__ void __launch_bounds__(64 * NW) k_fwd_fused2(const T* __restrict__ Qp
 
   Frag<T> qf[NK], kf[NK];
   {
-    const T* qrow = Qp + ((long)zq * Lp + 16 * tq + col) * D + 8 * g;
-    const T* krow = Kp + ((long)zk * Lp + 16 * tq + col) * D + 8 * g;
 #pragma unroll
-    for (int q = 0; q < NK; ++q) { qf[q] = ld8(qrow + 32 * q); kf[q] = ld8(krow + 32 * q); }
+    for (int q = 0; q < NK; ++q) {
+      qf[q] = ld8(Qp + nat_off<D>(zq, Lp, 16 * tq + col, 32 * q + 8 * g));
+      kf[q] = ld8(Kp + nat_off<D>(zk, Lp, 16 * tq + col, 32 * q + 8 * g));
+    }
   }
   const f32x4 lb = load_t4(ldest + (long)zk * Lp + 16 * tq, g);
   f32x4 o[ND];
@@ -207,8 +209,8 @@ __global__ void __launch_bounds__(64 * NW) k_fwd_fused2(const T* __restrict__ Qp
     const int kt_ = n_kt - 1 - (s);                                                         \
     stN.issue((base), Kz + (long)(64 * kt_) * D, w);                                        \
     stN.issue((base) + TN::BYTES, Kz + (long)(64 * kt_ + 32) * D, w);                       \
-    stT.issue((base) + 2 * TN::BYTES, Vz + 64 * kt_, w);                                    \
-    stT.issue((base) + 2 * TN::BYTES + TT::BYTES, Vz + 64 * kt_ + 32, w);                   \
+    stT.issue((base) + 2 * TN::BYTES, Vz + (long)(2 * kt_) * (32 * D), w);                  \
+    stT.issue((base) + 2 * TN::BYTES + TT::BYTES, Vz + (long)(2 * kt_ + 1) * (32 * D), w);  \
     issue_row((base) + TILES + w * 1024, ((lane & 16) ? lsz : Crow) + 64 * kt_ + 4 * (lane & 15)); \
   }
 #define UA_COMPUTE_FAST(s, base) fwd_tile(n_kt - 1 - (s), (base), FalseC())
@@ -331,7 +333,7 @@ template <class T, int D, int NST, bool MR>
 __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   using TN = Tile<T, 32, D>;
   using TT = Tile<T, D, 32>;
-  constexpr int NK = D / 32, ND = D / 16, LS = TN::STRIDE, TS = TT::STRIDE;
+  constexpr int NK = D / 32, ND = D / 16;
   constexpr int TILES = 3 * TN::BYTES + 3 * TT::BYTES, SB = TILES + 1024;
   // stats row of a stage: [lse2: 32f][delta: 32f][ldest: 32f][unused: 32f][forward carries of the 128 keys: 128f]
   UA_STAGES(SB);
@@ -350,9 +352,12 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
 
   Frag<T> kp[NK], vf[NK];
   {
-    const long ro = ((long)zk * Lp + spos) * D + 8 * g;
 #pragma unroll
-    for (int q = 0; q < NK; ++q) { kp[q] = ld8(a.Kp + ro + 32 * q); vf[q] = ld8(a.Vp + ro + 32 * q); }
+    for (int q = 0; q < NK; ++q) {
+      const long ro = nat_off<D>(zk, Lp, spos, 32 * q + 8 * g);
+      kp[q] = ld8(a.Kp + ro);
+      vf[q] = ld8(a.Vp + ro);
+    }
   }
   const float la = a.lsrc[(long)zk * Lp + spos];
   f32x4 dVt[ND], dKt[ND];
@@ -370,13 +375,13 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   {                                                                                         \
     const int tb_ = nTr - 1 - (s) / R;                                                      \
     const long zq_ = (long)zk * R + (s) % R;                                                \
-    const long qo_ = (zq_ * Lp + 32 * tb_) * D, to_ = zq_ * D * Lp + 32 * tb_;              \
+    const long qo_ = (zq_ * Lp + 32 * tb_) * D;   /* tile base, natural and transposed */      \
     stN.issue((base), Kz + (long)(32 * tb_) * D, w);                                        \
     stN.issue((base) + TN::BYTES, a.Qp + qo_, w);                                           \
     stN.issue((base) + 2 * TN::BYTES, a.dOp + qo_, w);                                      \
-    stT.issue((base) + 3 * TN::BYTES, KTz + 32 * tb_, w);                                   \
-    stT.issue((base) + 3 * TN::BYTES + TT::BYTES, a.QT + to_, w);                           \
-    stT.issue((base) + 3 * TN::BYTES + 2 * TT::BYTES, a.dOT + to_, w);                      \
+    stT.issue((base) + 3 * TN::BYTES, KTz + (long)(32 * tb_) * D, w);                       \
+    stT.issue((base) + 3 * TN::BYTES + TT::BYTES, a.QT + qo_, w);                           \
+    stT.issue((base) + 3 * TN::BYTES + 2 * TT::BYTES, a.dOT + qo_, w);                      \
     if (w == 0) {                                                                           \
       const float* src_;                                                                    \
       if (lane < 8) src_ = a.lse2 + zq_ * Lp + 32 * tb_ + 4 * lane;                         \
@@ -518,7 +523,7 @@ template <class T, int D, int NST>
 __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restrict__ dq, int d) {
   using TN = Tile<T, 32, D>;
   using TT = Tile<T, D, 32>;
-  constexpr int NK = D / 32, ND = D / 16, LS = TN::STRIDE, TS = TT::STRIDE;
+  constexpr int NK = D / 32, ND = D / 16;
   using ST = StageT<T>;
   constexpr int TILES = 4 * TN::BYTES + 2 * TT::BYTES, SB = TILES + 8 * 1024;   // + per wave [C: 64f][lsrc: 64f][Dsuf: 64f]
   UA_STAGES(SB);
@@ -537,9 +542,8 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
 
   Frag<T> kt[NK];
   {
-    const T* krow = a.Kp + ((long)zk * Lp + 16 * tq + col) * D + 8 * g;
 #pragma unroll
-    for (int q = 0; q < NK; ++q) kt[q] = ld8(krow + 32 * q);
+    for (int q = 0; q < NK; ++q) kt[q] = ld8(a.Kp + nat_off<D>(zk, Lp, 16 * tq + col, 32 * q + 8 * g));
   }
   const f32x4 lb = load_t4(a.ldest + (long)zk * Lp + 16 * tq, g);
   f32x4 dKc[ND];
@@ -559,10 +563,12 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
     const long zq = (long)zk * R + r;
     Frag<T> qt[NK], gt[NK];
     {
-      const T* qrow = a.Qp + (zq * Lp + 16 * tq + col) * D + 8 * g;
-      const T* grow = a.dOp + (zq * Lp + 16 * tq + col) * D + 8 * g;
 #pragma unroll
-      for (int q = 0; q < NK; ++q) { qt[q] = ld8(qrow + 32 * q); gt[q] = ld8(grow + 32 * q); }
+      for (int q = 0; q < NK; ++q) {
+        const long ro = nat_off<D>(zq, Lp, 16 * tq + col, 32 * q + 8 * g);
+        qt[q] = ld8(a.Qp + ro);
+        gt[q] = ld8(a.dOp + ro);
+      }
     }
     const f32x4 l2t = load_t4(a.lse2 + zq * Lp + 16 * tq, g), dlt = load_t4(a.delta + zq * Lp + 16 * tq, g);
     f32x4 dQ[ND];
@@ -576,8 +582,8 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
     stN.issue((base) + TN::BYTES, Kz + (long)(k0_ + 32) * D, w);                            \
     stN.issue((base) + 2 * TN::BYTES, Vz + (long)k0_ * D, w);                               \
     stN.issue((base) + 3 * TN::BYTES, Vz + (long)(k0_ + 32) * D, w);                        \
-    stT.issue((base) + 4 * TN::BYTES, KTz + k0_, w);                                        \
-    stT.issue((base) + 4 * TN::BYTES + TT::BYTES, KTz + k0_ + 32, w);                       \
+    stT.issue((base) + 4 * TN::BYTES, KTz + (long)k0_ * D, w);                              \
+    stT.issue((base) + 4 * TN::BYTES + TT::BYTES, KTz + (long)(k0_ + 32) * D, w);           \
     issue_row((base) + TILES + w * 1024,                                                    \
               (lane < 16 ? Crow : (lane < 32 ? lsz : Drow)) + k0_ + 4 * (lane & 15));       \
   }

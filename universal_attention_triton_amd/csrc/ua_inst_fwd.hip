@@ -11,15 +11,16 @@ static void allow_lds(K kernel, size_t bytes) {
 }
 
 template <class T, int D>
-static hipError_t carry_t(const void* Kp, const float* lsrc, const float* ldest, float* C, int Lp, int Zk, hipStream_t s) {
+static hipError_t carry_t(const void* Kp, const float* lsrc, const float* ldest, float* C, int Lp, int Zk, int tiled, hipStream_t s) {
   constexpr int NST = 2;
-  hipLaunchKernelGGL((k_carry2<T, D, NST>), dim3(Lp / 128, Zk), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, C, Lp);
+  if (tiled) hipLaunchKernelGGL((k_carry2<T, D, NST, true>), dim3(Lp / 128, Zk), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, C, Lp);
+  else hipLaunchKernelGGL((k_carry2<T, D, NST, false>), dim3(Lp / 128, Zk), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, C, Lp);
   return hipGetLastError();
 }
 hipError_t launch_carry(int dtype, int D, const void* Kp, const float* lsrc, const float* ldest, float* C, int Lp, int Zk,
-                        hipStream_t s) {
-  if (dtype == 1) return D == 64 ? carry_t<bf16, 64>(Kp, lsrc, ldest, C, Lp, Zk, s) : carry_t<bf16, 128>(Kp, lsrc, ldest, C, Lp, Zk, s);
-  return D == 64 ? carry_t<float, 64>(Kp, lsrc, ldest, C, Lp, Zk, s) : carry_t<float, 128>(Kp, lsrc, ldest, C, Lp, Zk, s);
+                        int tiled, hipStream_t s) {
+  if (dtype == 1) return D == 64 ? carry_t<bf16, 64>(Kp, lsrc, ldest, C, Lp, Zk, tiled, s) : carry_t<bf16, 128>(Kp, lsrc, ldest, C, Lp, Zk, tiled, s);
+  return D == 64 ? carry_t<float, 64>(Kp, lsrc, ldest, C, Lp, Zk, tiled, s) : carry_t<float, 128>(Kp, lsrc, ldest, C, Lp, Zk, tiled, s);
 }
 
 // explicit instantiations (the implicit ones are not emitted on the host side for these kernels)

@@ -15,8 +15,9 @@ struct BwdArgsV {
 };
 
 // Every launcher returns hipGetLastError() after enqueuing.  dtype: 0 fp32, 1 bf16.  D in {64,128}.
+// tiled: Kp is stored in tiles of 32 keys, k-group-major (fused mode) instead of row-major (chunked mode)
 hipError_t launch_carry(int dtype, int D, const void* Kp, const float* lsrc, const float* ldest, float* C, int Lp, int Zk,
-                        hipStream_t s);
+                        int tiled, hipStream_t s);
 int fwd_fused_variants(int dtype, int D);
 hipError_t launch_fwd_fused(int dtype, int D, int variant, const void* Qp, const void* Kp, const void* VT,
                             const float* lsrc, const float* ldest, const float* C, void* O, float* lse, float* lse2, int R,

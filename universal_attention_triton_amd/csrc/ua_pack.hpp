@@ -20,11 +20,13 @@ __device__ __forceinline__ long rows_offset(const RowsView& v, int z, int row) {
          (long)(row % v.inner) * v.si;
 }
 
-// x (dtype T) -> nat [Z][Lp][D] and/or tr [Z][D][Lp], zero padded (rows >= L, cols >= d).
-// tr stores position t at column perm16(t) (tr_mode 0), perm32(t) (1) or t (2).
+// x (dtype T) -> nat and/or tr working tensors, zero padded (rows >= L, cols >= d).
+//   tiled == 0: nat [Z][Lp][D] row-major, tr [Z][D][Lp] row-major       (chunked-mode kernels)
+//   tiled != 0: both in tiles of 32 positions, k-group-major (nat_off / tr_off)   (fused kernels)
+// tr stores position t at column perm16(t) (tr_mode 0), perm32(t) (1) or t (2) of its group of 32.
 template <class T, int D>
 __global__ void __launch_bounds__(256) k_pack(RowsView x, T* __restrict__ nat, T* __restrict__ tr, int d, int L, int Lp,
-                                              int tr_mode) {
+                                              int tr_mode, int tiled) {
   __shared__ float tile[32][D + 1];
   const int z = blockIdx.y, row0 = blockIdx.x * 32, tid = threadIdx.x;
   const T* xp = reinterpret_cast<const T*>(x.p);
@@ -33,15 +35,29 @@ __global__ void __launch_bounds__(256) k_pack(RowsView x, T* __restrict__ nat, T
     float val = 0.f;
     if (row < L && col < d) val = (float)xp[rows_offset(x, z, row) + (long)col * x.sc];
     tile[rr][col] = val;
-    if (nat) nat[((long)z * Lp + row) * D + col] = cvt<T>(val);
+    if (nat && !tiled) nat[((long)z * Lp + row) * D + col] = cvt<T>(val);
+  }
+  if (!tr && !(nat && tiled)) return;
+  __syncthreads();
+  if (nat && tiled) {
+    // consecutive threads write consecutive elements of the tiled order: (k-group, row, e)
+    for (int i = tid; i < 32 * D; i += 256) {
+      const int e = i & 7, rr = (i >> 3) & 31, kg = i >> 8;
+      nat[nat_off<D>(z, Lp, row0 + rr, 8 * kg + e)] = cvt<T>(tile[rr][8 * kg + e]);
+    }
   }
   if (!tr) return;
-  __syncthreads();
   for (int i = tid; i < 32 * D; i += 256) {
-    int dd = i >> 5, rr = i & 31;
-    // perm16 and perm32 are involutions / bijections of 0..31: column rr holds the position that maps onto it
-    const int src = tr_mode == 0 ? perm16(rr) : (tr_mode == 1 ? (((rr >> 3) & 3) << 2 | ((rr >> 2) & 1) << 4 | (rr & 3)) : rr);
-    tr[((long)z * D + dd) * Lp + row0 + rr] = cvt<T>(tile[src][dd]);
+    // perm16 and perm32 are bijections of 0..31: column p holds the position that maps onto it
+    if (tiled) {
+      const int e = i & 7, dd = (i >> 3) % D, kg = i / (8 * D), p = 8 * kg + e;
+      const int src = tr_mode == 0 ? perm16(p) : (tr_mode == 1 ? (((p >> 3) & 3) << 2 | ((p >> 2) & 1) << 4 | (p & 3)) : p);
+      tr[tr_off<D>(z, Lp, dd, blockIdx.x, p)] = cvt<T>(tile[src][dd]);
+    } else {
+      const int dd = i >> 5, rr = i & 31;
+      const int src = tr_mode == 0 ? perm16(rr) : (tr_mode == 1 ? (((rr >> 3) & 3) << 2 | ((rr >> 2) & 1) << 4 | (rr & 3)) : rr);
+      tr[((long)z * D + dd) * Lp + row0 + rr] = cvt<T>(tile[src][dd]);
+    }
   }
 }
 
