@@ -110,11 +110,18 @@ ua::RowsView null_view() { ua::RowsView v{}; v.inner = 1; v.H = v.R = v.N = 1; r
 
 // tr_mode: column order of the transposed copy inside each group of 32 positions
 enum { TR_PERM16 = 0, TR_PERM32 = 1, TR_NATURAL = 2 };
+// rows of the view start 16-byte aligned and the feature stride is 1: 16-byte loads are allowed
+bool vector_ok(const ua::RowsView& v, size_t esz, int d) {
+  const long V = 16 / (long)esz;
+  auto al = [&](long stride) { return stride % V == 0; };
+  return v.sc == 1 && d % V == 0 && (uintptr_t)v.p % 16 == 0 && al(v.sb) && al(v.sh) && al(v.sr) && al(v.sn) && al(v.so) && al(v.si);
+}
 template <class T>
 hipError_t pack_t(int D, const ua::RowsView& x, void* nat, void* tr, int d, int L, int Lp, int Z, int tr_mode, hipStream_t s) {
   const int tiled = tr_mode != TR_PERM16;      // the fused kernels read tiled working tensors, the chunked ones row-major
-  if (D == 64) hipLaunchKernelGGL((ua::k_pack<T, 64>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp, tr_mode, tiled);
-  else hipLaunchKernelGGL((ua::k_pack<T, 128>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp, tr_mode, tiled);
+  const int vec = vector_ok(x, sizeof(T), d) ? 1 : 0;
+  if (D == 64) hipLaunchKernelGGL((ua::k_pack<T, 64>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp, tr_mode, tiled, vec);
+  else hipLaunchKernelGGL((ua::k_pack<T, 128>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp, tr_mode, tiled, vec);
   return hipGetLastError();
 }
 hipError_t pack(int dtype, int D, const ua::RowsView& x, void* nat, void* tr, int d, int L, int Lp, int Z, int tr_mode, hipStream_t s) {
@@ -233,7 +240,8 @@ hipError_t finish_t(const Layout& l, const ua_desc& d, char* ws, bool chunked, c
 template <class T>
 hipError_t delta_t(const ua::RowsView& O, const ua::RowsView& dO, const ua::RowsView& sub, const ua::RowsView& lse_in,
                    float* delta, float* lse2, int d, int L, int Lp, int Z, hipStream_t s) {
-  hipLaunchKernelGGL((ua::k_delta<T>), dim3(Lp / 4, Z), dim3(256), 0, s, O, dO, sub, lse_in, delta, lse2, d, L, Lp);
+  const int vec = vector_ok(O, sizeof(T), d) && vector_ok(dO, sizeof(T), d) ? 1 : 0;
+  hipLaunchKernelGGL((ua::k_delta<T>), dim3(Lp / 16, Z), dim3(256), 0, s, O, dO, sub, lse_in, delta, lse2, d, L, Lp, vec);
   return hipGetLastError();
 }
 
@@ -315,9 +323,9 @@ int ua_fused_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, cons
   {
     UA_PROF("pack_dO+delta", s);
     UA_HIP(pack(d.dtype, l.D, dOv, w + l.dOp, w + l.dOT, d.d, d.L, l.Lp, l.Zq, TR_PERM32, s));
+    if (d.dtype == UA_BF16) UA_HIP(delta_t<ua::bf16>(Ov, dOv, none, lsev, (float*)(w + l.delta), (float*)(w + l.lse2), d.d, d.L, l.Lp, l.Zq, s));
+    else UA_HIP(delta_t<float>(Ov, dOv, none, lsev, (float*)(w + l.delta), (float*)(w + l.lse2), d.d, d.L, l.Lp, l.Zq, s));
   }
-  if (d.dtype == UA_BF16) UA_HIP(delta_t<ua::bf16>(Ov, dOv, none, lsev, (float*)(w + l.delta), (float*)(w + l.lse2), d.d, d.L, l.Lp, l.Zq, s));
-  else UA_HIP(delta_t<float>(Ov, dOv, none, lsev, (float*)(w + l.delta), (float*)(w + l.lse2), d.d, d.L, l.Lp, l.Zq, s));
   return run_bwd_common(d, l, w, false, static_src, static_dest, dkc, dvc, dxq, dsrc, ddest, s);
 }
 

@@ -24,36 +24,70 @@ __device__ __forceinline__ long rows_offset(const RowsView& v, int z, int row) {
 //   tiled == 0: nat [Z][Lp][D] row-major, tr [Z][D][Lp] row-major       (chunked-mode kernels)
 //   tiled != 0: both in tiles of 32 positions, k-group-major (nat_off / tr_off)   (fused kernels)
 // tr stores position t at column perm16(t) (tr_mode 0), perm32(t) (1) or t (2) of its group of 32.
+// vec != 0: every row start of x is 16-byte aligned and d is a multiple of the 16-byte vector (host-checked), so
+// rows are read with 16-byte loads.
 template <class T, int D>
 __global__ void __launch_bounds__(256) k_pack(RowsView x, T* __restrict__ nat, T* __restrict__ tr, int d, int L, int Lp,
-                                              int tr_mode, int tiled) {
+                                              int tr_mode, int tiled, int vec) {
+  constexpr int V = 16 / (int)sizeof(T);
   __shared__ float tile[32][D + 1];
   const int z = blockIdx.y, row0 = blockIdx.x * 32, tid = threadIdx.x;
   const T* xp = reinterpret_cast<const T*>(x.p);
-  for (int i = tid; i < 32 * D; i += 256) {
-    int rr = i / D, col = i - rr * D, row = row0 + rr;
-    float val = 0.f;
-    if (row < L && col < d) val = (float)xp[rows_offset(x, z, row) + (long)col * x.sc];
-    tile[rr][col] = val;
-    if (nat && !tiled) nat[((long)z * Lp + row) * D + col] = cvt<T>(val);
+  if (vec) {
+    for (int i = tid; i < 32 * (D / V); i += 256) {
+      const int rr = i / (D / V), col = (i - rr * (D / V)) * V, row = row0 + rr;
+      T v[V];
+      if (row < L && col < d) {
+        *reinterpret_cast<uint4*>(v) = *reinterpret_cast<const uint4*>(xp + rows_offset(x, z, row) + col);
+      } else {
+#pragma unroll
+        for (int e = 0; e < V; ++e) v[e] = cvt<T>(0.f);
+      }
+#pragma unroll
+      for (int e = 0; e < V; ++e) tile[rr][col + e] = (float)v[e];
+      if (nat && !tiled) *reinterpret_cast<uint4*>(nat + ((long)z * Lp + row) * D + col) = *reinterpret_cast<const uint4*>(v);
+    }
+  } else {
+    for (int i = tid; i < 32 * D; i += 256) {
+      int rr = i / D, col = i - rr * D, row = row0 + rr;
+      float val = 0.f;
+      if (row < L && col < d) val = (float)xp[rows_offset(x, z, row) + (long)col * x.sc];
+      tile[rr][col] = val;
+      if (nat && !tiled) nat[((long)z * Lp + row) * D + col] = cvt<T>(val);
+    }
   }
   if (!tr && !(nat && tiled)) return;
   __syncthreads();
   if (nat && tiled) {
-    // consecutive threads write consecutive elements of the tiled order: (k-group, row, e)
-    for (int i = tid; i < 32 * D; i += 256) {
-      const int e = i & 7, rr = (i >> 3) & 31, kg = i >> 8;
-      nat[nat_off<D>(z, Lp, row0 + rr, 8 * kg + e)] = cvt<T>(tile[rr][8 * kg + e]);
+    // one (k-group, row) cell of 8 elements per thread; consecutive threads write consecutive cells
+    for (int i = tid; i < 4 * D; i += 256) {
+      const int rr = i & 31, kg = i >> 5;
+      T v[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = cvt<T>(tile[rr][8 * kg + e]);
+      T* dst = nat + nat_off<D>(z, Lp, row0 + rr, 8 * kg);
+#pragma unroll
+      for (int u = 0; u < 8 / V; ++u) reinterpret_cast<uint4*>(dst)[u] = reinterpret_cast<const uint4*>(v)[u];
     }
   }
   if (!tr) return;
-  for (int i = tid; i < 32 * D; i += 256) {
-    // perm16 and perm32 are bijections of 0..31: column p holds the position that maps onto it
-    if (tiled) {
-      const int e = i & 7, dd = (i >> 3) % D, kg = i / (8 * D), p = 8 * kg + e;
-      const int src = tr_mode == 0 ? perm16(p) : (tr_mode == 1 ? (((p >> 3) & 3) << 2 | ((p >> 2) & 1) << 4 | (p & 3)) : p);
-      tr[tr_off<D>(z, Lp, dd, blockIdx.x, p)] = cvt<T>(tile[src][dd]);
-    } else {
+  // perm16 and perm32 are bijections of 0..31: column p holds the position that maps onto it
+  if (tiled) {
+    for (int i = tid; i < 4 * D; i += 256) {
+      const int dd = i % D, kg = i / D;
+      T v[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int p = 8 * kg + e;
+        const int src = tr_mode == 0 ? perm16(p) : (tr_mode == 1 ? (((p >> 3) & 3) << 2 | ((p >> 2) & 1) << 4 | (p & 3)) : p);
+        v[e] = cvt<T>(tile[src][dd]);
+      }
+      T* dst = tr + tr_off<D>(z, Lp, dd, blockIdx.x, 8 * kg);
+#pragma unroll
+      for (int u = 0; u < 8 / V; ++u) reinterpret_cast<uint4*>(dst)[u] = reinterpret_cast<const uint4*>(v)[u];
+    }
+  } else {
+    for (int i = tid; i < 32 * D; i += 256) {
       const int dd = i >> 5, rr = i & 31;
       const int src = tr_mode == 0 ? perm16(rr) : (tr_mode == 1 ? (((rr >> 3) & 3) << 2 | ((rr >> 2) & 1) << 4 | (rr & 3)) : rr);
       tr[((long)z * D + dd) * Lp + row0 + rr] = cvt<T>(tile[src][dd]);
@@ -62,23 +96,34 @@ __global__ void __launch_bounds__(256) k_pack(RowsView x, T* __restrict__ nat, T
 }
 
 // delta[z][t] = sum_dd O[z][t][dd] * dO[z][t][dd] - sub[z][t]   (fp32; padded rows -> 0)
-// O, dO, sub are views (sub optional, float); one wave per row.
+// O, dO, sub are views (sub optional, float); 16 lanes per row, 16 rows per block.
 // lse_in (optional, natural log, float view) is rewritten in log2 units into lse2 [Z][Lp].
+// vec != 0: rows of O and dO start 16-byte aligned, have unit feature stride and d is a multiple of the vector.
 template <class T>
 __global__ void __launch_bounds__(256) k_delta(RowsView O, RowsView dO, RowsView sub, RowsView lse_in,
-                                               float* __restrict__ delta, float* __restrict__ lse2, int d, int L, int Lp) {
-  const int z = blockIdx.y, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int t = blockIdx.x * 4 + wave;
-  if (t >= Lp) return;
+                                               float* __restrict__ delta, float* __restrict__ lse2, int d, int L, int Lp, int vec) {
+  constexpr int V = 16 / (int)sizeof(T);
+  const int z = blockIdx.y, sub16 = threadIdx.x & 15;
+  const int t = blockIdx.x * 16 + (threadIdx.x >> 4);
   float s = 0.f;
   if (t < L) {
     const T* o = reinterpret_cast<const T*>(O.p) + rows_offset(O, z, t);
     const T* g = reinterpret_cast<const T*>(dO.p) + rows_offset(dO, z, t);
-    for (int c = lane; c < d; c += 64) s += (float)o[(long)c * O.sc] * (float)g[(long)c * dO.sc];
+    if (vec) {
+      for (int c = sub16 * V; c < d; c += 16 * V) {
+        T a[V], b[V];
+        *reinterpret_cast<uint4*>(a) = *reinterpret_cast<const uint4*>(o + c);
+        *reinterpret_cast<uint4*>(b) = *reinterpret_cast<const uint4*>(g + c);
+#pragma unroll
+        for (int e = 0; e < V; ++e) s += (float)a[e] * (float)b[e];
+      }
+    } else {
+      for (int c = sub16; c < d; c += 16) s += (float)o[(long)c * O.sc] * (float)g[(long)c * dO.sc];
+    }
   }
 #pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) s += __shfl_xor(s, m, 64);
-  if (lane == 0) {
+  for (int m = 8; m >= 1; m >>= 1) s += __shfl_xor(s, m, 64);
+  if (sub16 == 0 && t < Lp) {
     if (sub.p && t < L) s -= reinterpret_cast<const float*>(sub.p)[rows_offset(sub, z, t)];
     delta[(long)z * Lp + t] = s;
     if (lse_in.p) lse2[(long)z * Lp + t] = (t < L) ? reinterpret_cast<const float*>(lse_in.p)[rows_offset(lse_in, z, t)] * kLog2e : 0.f;
