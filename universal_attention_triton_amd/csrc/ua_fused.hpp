@@ -341,7 +341,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   int bx, zk;
   xcd_map(bx, zk);
   const int Lp = a.Lp, L = a.L, nT16 = Lp / 16, R = MR ? a.R : 1;
-  const int kg = gridDim.x - 1 - bx, sb16 = 8 * kg + w, spos = 16 * sb16 + col;
+  const int kg = bx, sb16 = 8 * kg + w, spos = 16 * sb16 + col;      // key group 0 sweeps the most query blocks: first
   const int nTr = (L + 31) / 32, first = 4 * kg;
   if (first >= nTr) return;                      // every key of this workgroup is padding
   const GroupMasks gm = group_masks(lane);
