@@ -38,8 +38,12 @@ enum {
   UA_OP_FUSED_BWD = 3  /* ua_fused_bwd  */
 };
 enum {
-  UA_FLAG_SKIP_MASKED = 1 /* ua_bwd: the upstream gradient is zero for (query, chunk) pairs in which the
-                             query precedes the whole chunk (true when it comes from ua_merge_bwd) */
+  UA_FLAG_SKIP_MASKED = 1, /* ua_bwd: the upstream gradient is zero for (query, chunk) pairs in which the
+                              query precedes the whole chunk (true when it comes from ua_merge_bwd) */
+  UA_FLAG_PRUNE = 2        /* fused ops: skip (key, query) pairs whose softmax weight is provably below 2^-48 because
+                              of the accumulated decay (no counterpart in the reference, which visits every pair).
+                              The bound uses the largest key and query norms of the head; results change by less
+                              than float32 rounding.  ua_fused_bwd with ws_has_fwd follows what the forward recorded. */
 };
 
 /* Problem description.  kc, vc: [b,h,L,d] seen as [b,h,n,c,d]; xq: [b,h,r,L,d]; gates: [b,h,L]. */

@@ -23,6 +23,7 @@ namespace ua {
 
 template <class T>
 struct BwdArgs {
+  const int *reach, *minkey;    // pruning state of the fused mode: [Zk][Lp/16], [Zk][Lp/32]
   const T *Kp, *Vp;             // [Zk][Lp][D]
   const T *KT;                  // [Zk][D][Lp]
   const float *lsrc, *ldest;    // [Zk][Lp]  log2(gate)/3

@@ -34,7 +34,7 @@ struct Layout {
   int D, Lp, nT, nch, Zk, Zq;
   size_t esz;
   // forward state
-  size_t Kp, KT, Vp, VT, Qp, QT, lsrc, ldest, C, lse2, fwd_end;
+  size_t Kp, KT, Vp, VT, Qp, QT, lsrc, ldest, C, lse2, knorm2, qnorm2, reach, minkey, fwd_end;
   // backward scratch
   size_t dOp, dOT, delta, dQacc, dKdacc, Dsuf, dKrow, dVrow, dsrc_raw, total;
 };
@@ -71,6 +71,9 @@ Layout make_layout(const ua_desc& d, bool chunked) {
   l.lsrc = take((size_t)l.Zk * l.Lp * 4); l.ldest = take((size_t)l.Zk * l.Lp * 4);
   l.C = take((size_t)l.Zk * l.nT * l.Lp * 4);
   l.lse2 = take((size_t)l.Zq * l.nch * l.Lp * 4);
+  // pruning state of the fused mode: largest squared row norm of every 32-row block of K and Q, reach of every key
+  // tile, first key tile reaching every query block
+  l.knorm2 = take((size_t)l.Zk * (l.nT / 2) * 4); l.qnorm2 = take((size_t)l.Zq * (l.nT / 2) * 4); l.reach = take((size_t)l.Zk * l.nT * 4); l.minkey = take((size_t)l.Zk * (l.nT / 2) * 4);
   l.fwd_end = off;
   const size_t gbytes = (size_t)l.Zq * l.nch * l.Lp * l.D * l.esz;
   l.dOp = take(gbytes); l.dOT = take(gbytes);
@@ -117,15 +120,19 @@ bool vector_ok(const ua::RowsView& v, size_t esz, int d) {
   return v.sc == 1 && d % V == 0 && (uintptr_t)v.p % 16 == 0 && al(v.sb) && al(v.sh) && al(v.sr) && al(v.sn) && al(v.so) && al(v.si);
 }
 template <class T>
-hipError_t pack_t(int D, const ua::RowsView& x, void* nat, void* tr, int d, int L, int Lp, int Z, int tr_mode, hipStream_t s) {
+hipError_t pack_t(int D, const ua::RowsView& x, void* nat, void* tr, int d, int L, int Lp, int Z, int tr_mode, float* norm2,
+                  hipStream_t s) {
   const int tiled = tr_mode != TR_PERM16;      // the fused kernels read tiled working tensors, the chunked ones row-major
   const int vec = vector_ok(x, sizeof(T), d) ? 1 : 0;
-  if (D == 64) hipLaunchKernelGGL((ua::k_pack<T, 64>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp, tr_mode, tiled, vec);
-  else hipLaunchKernelGGL((ua::k_pack<T, 128>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp, tr_mode, tiled, vec);
+  if (D == 64) hipLaunchKernelGGL((ua::k_pack<T, 64>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp, tr_mode, tiled, vec, norm2);
+  else hipLaunchKernelGGL((ua::k_pack<T, 128>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp, tr_mode, tiled, vec, norm2);
   return hipGetLastError();
 }
-hipError_t pack(int dtype, int D, const ua::RowsView& x, void* nat, void* tr, int d, int L, int Lp, int Z, int tr_mode, hipStream_t s) {
-  return dtype == UA_BF16 ? pack_t<ua::bf16>(D, x, nat, tr, d, L, Lp, Z, tr_mode, s) : pack_t<float>(D, x, nat, tr, d, L, Lp, Z, tr_mode, s);
+// norm2 (optional): [Z][Lp/32] receives the largest squared row norm of every block of 32 rows
+hipError_t pack(int dtype, int D, const ua::RowsView& x, void* nat, void* tr, int d, int L, int Lp, int Z, int tr_mode, hipStream_t s,
+                float* norm2 = nullptr) {
+  return dtype == UA_BF16 ? pack_t<ua::bf16>(D, x, nat, tr, d, L, Lp, Z, tr_mode, norm2, s)
+                          : pack_t<float>(D, x, nat, tr, d, L, Lp, Z, tr_mode, norm2, s);
 }
 
 // ---- optional per-kernel timing (hipEvents on the launch stream) ---------------------------
@@ -179,9 +186,10 @@ int pack_inputs(const ua_desc& d, const Layout& l, bool chunked, const ua_rows* 
   const ua::RowsView K = rows_view(*kc, d.h, 1), V = rows_view(*vc, d.h, 1), Q = rows_view(*xq, d.h, d.r);
   // the chunked kernels work on 32x32 tiles, the fused ones on 16x16 tiles (and read V^T in natural order)
   const int mode = chunked ? TR_PERM16 : TR_PERM32;
-  UA_HIP(pack(d.dtype, l.D, K, ws + l.Kp, ws + l.KT, d.d, d.L, l.Lp, l.Zk, mode, s));
+  const bool prune = !chunked && (d.flags & UA_FLAG_PRUNE);
+  UA_HIP(pack(d.dtype, l.D, K, ws + l.Kp, ws + l.KT, d.d, d.L, l.Lp, l.Zk, mode, s, prune ? (float*)(ws + l.knorm2) : nullptr));
   UA_HIP(pack(d.dtype, l.D, V, ws + l.Vp, ws + l.VT, d.d, d.L, l.Lp, l.Zk, chunked ? TR_PERM16 : TR_NATURAL, s));
-  UA_HIP(pack(d.dtype, l.D, Q, ws + l.Qp, ws + l.QT, d.d, d.L, l.Lp, l.Zq, mode, s));
+  UA_HIP(pack(d.dtype, l.D, Q, ws + l.Qp, ws + l.QT, d.d, d.L, l.Lp, l.Zq, mode, s, prune ? (float*)(ws + l.qnorm2) : nullptr));
   const dim3 grid((l.Lp + 255) / 256, l.Zk);
   if (d.dtype == UA_BF16)
     hipLaunchKernelGGL((ua::k_gates<ua::bf16>), grid, dim3(256), 0, s, (const ua::bf16*)src, (const ua::bf16*)dest,
@@ -217,12 +225,13 @@ int run_fused_fwd_kernels(const ua_desc& d, const Layout& l, char* ws, void* O, 
   {
     UA_PROF("k_carry", s);
     UA_HIP(ua::launch_carry(d.dtype, l.D, ws + l.Kp, (const float*)(ws + l.lsrc), (const float*)(ws + l.ldest),
-                            (float*)(ws + l.C), l.Lp, l.Zk, 1, s));
+                            (float*)(ws + l.C), l.Lp, l.Zk, 1, (d.flags & UA_FLAG_PRUNE) ? (const float*)(ws + l.knorm2) : nullptr,
+                            (const float*)(ws + l.qnorm2), d.r, (int*)(ws + l.reach), (int*)(ws + l.minkey), s));
   }
   UA_PROF("k_fwd_fused", s);
   UA_HIP(ua::launch_fwd_fused(d.dtype, l.D, variant, ws + l.Qp, ws + l.Kp, ws + l.VT, (const float*)(ws + l.lsrc),
-                              (const float*)(ws + l.ldest), (const float*)(ws + l.C), O, lse, (float*)(ws + l.lse2), d.r,
-                              d.L, l.Lp, d.d, l.Zq, s));
+                              (const float*)(ws + l.ldest), (const float*)(ws + l.C), O, lse, (float*)(ws + l.lse2),
+                              (const int*)(ws + l.reach), (const int*)(ws + l.minkey), d.r, d.L, l.Lp, d.d, l.Zq, s));
   return UA_OK;
 }
 
@@ -256,6 +265,7 @@ int run_bwd_common(const ua_desc& d, const Layout& l, char* ws, bool chunked, co
   a.Kp = ws + l.Kp; a.Vp = ws + l.Vp; a.KT = ws + l.KT; a.Qp = ws + l.Qp; a.QT = ws + l.QT; a.dOp = ws + l.dOp;
   a.dOT = ws + l.dOT; a.lsrc = (const float*)(ws + l.lsrc); a.ldest = (const float*)(ws + l.ldest);
   a.lse2 = (const float*)(ws + l.lse2); a.delta = (const float*)(ws + l.delta); a.C = (const float*)(ws + l.C);
+  a.reach = (const int*)(ws + l.reach); a.minkey = (const int*)(ws + l.minkey);
   a.dQacc = (float*)(ws + l.dQacc); a.dKdacc = (float*)(ws + l.dKdacc); a.Dsuf = (float*)(ws + l.Dsuf);
   a.dKrow = (float*)(ws + l.dKrow);
   a.dVrow = (float*)(ws + l.dVrow); a.dsrc_raw = (float*)(ws + l.dsrc_raw);
@@ -315,7 +325,8 @@ int ua_fused_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, cons
   if (!ws_has_fwd) {
     if (int e = pack_inputs(d, l, false, kc, vc, xq, static_src, static_dest, w, s)) return e;
     UA_HIP(ua::launch_carry(d.dtype, l.D, w + l.Kp, (const float*)(w + l.lsrc), (const float*)(w + l.ldest),
-                            (float*)(w + l.C), l.Lp, l.Zk, 1, s));
+                            (float*)(w + l.C), l.Lp, l.Zk, 1, (d.flags & UA_FLAG_PRUNE) ? (const float*)(w + l.knorm2) : nullptr,
+                            (const float*)(w + l.qnorm2), d.r, (int*)(w + l.reach), (int*)(w + l.minkey), s));
   }
   const long rowsz = (long)d.L * d.d;
   const ua::RowsView Ov = contiguous_view(O, rowsz, d.d), dOv = contiguous_view(dO, rowsz, d.d);
@@ -364,7 +375,7 @@ int ua_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
                                   (const float*)(w + l.ldest), nullptr, nullptr, (float*)(w + l.lse2), 0, 0, 0, 0, d.r, d.L, l.Lp, d.d, d.chunk, l.nch, l.Zk, s));
   }
   UA_HIP(ua::launch_carry(d.dtype, l.D, w + l.Kp, (const float*)(w + l.lsrc), (const float*)(w + l.ldest),
-                          (float*)(w + l.C), l.Lp, l.Zk, 0, s));
+                          (float*)(w + l.C), l.Lp, l.Zk, 0, nullptr, nullptr, 1, nullptr, nullptr, s));
   const ua::RowsView outv = chunked_view(*out, l.nch);
   ua_chunked gmut = *g_out;
   const ua::RowsView gv = chunked_view(gmut, l.nch), none = null_view();
@@ -471,8 +482,8 @@ int ua_autotune(const ua_desc* desc, int op, void* ws, size_t ws_bytes, ua_strea
     for (int rep = 0; rep < 2; ++rep) {   // first pass warms up
       UA_HIP(hipEventRecord(e0, s));
       hipError_t e = ua::launch_fwd_fused(desc->dtype, l.D, v, w + l.Qp, w + l.Kp, w + l.VT, (const float*)(w + l.lsrc),
-                                          (const float*)(w + l.ldest), (const float*)(w + l.C), Otmp, lsetmp, (float*)(w + l.lse2), desc->r, desc->L,
-                                          l.Lp, desc->d, l.Zq, s);
+                                          (const float*)(w + l.ldest), (const float*)(w + l.C), Otmp, lsetmp, (float*)(w + l.lse2),
+                                          (const int*)(w + l.reach), (const int*)(w + l.minkey), desc->r, desc->L, l.Lp, desc->d, l.Zq, s);
       if (e != hipSuccess) return fail(UA_ELAUNCH, "autotune launch: %s", hipGetErrorString(e));
       UA_HIP(hipEventRecord(e1, s));
       UA_HIP(hipEventSynchronize(e1));

@@ -29,6 +29,7 @@ typedef __bf16 bf16;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 constexpr float kAMax = (float)(1.0 - 1e-6);      // upper clamp of the affinity (forward and backward)
+constexpr float kPruneLog2 = 48.0f;               // softmax weights provably below 2^-48 are dropped when pruning
 constexpr float kAMinBwd = 1e-6f;                 // lower clamp used only in the backward divisor
 constexpr float kNegFill = -1e12f;                // bias of a (key, query) pair with key > query
 constexpr int kPad16 = 16;                        // bytes of padding per LDS row

@@ -25,10 +25,11 @@ __device__ __forceinline__ void issue_row(void* lds_base, const void* src_lane) 
 // does not wait for them) and provides ISSUE(step, stage) and COMPUTE(step, stage).
 // UA_PIPE_RANGE runs steps [S0, S1) of a pipeline of NSTEPS steps whose step S0 has already been issued
 // (by UA_PIPE_START or by the previous range), so that consecutive ranges may use different COMPUTE bodies.
-#define UA_PIPE_START(NSTEPS, ISSUE)                                                       \
+#define UA_PIPE_START_AT(S0, NSTEPS, ISSUE)                                                \
   do {                                                                                     \
-    if ((NSTEPS) > 0) ISSUE(0, stage0);                                                    \
+    if ((S0) < (NSTEPS)) ISSUE((S0), stage0);                                              \
   } while (0)
+#define UA_PIPE_START(NSTEPS, ISSUE) UA_PIPE_START_AT(0, NSTEPS, ISSUE)
 #define UA_STEP2_(STEP, NSTEPS, CUR, NXT, ISSUE, COMPUTE)                                  \
   {                                                                                        \
     wait_async_loads();                                                                    \
@@ -80,9 +81,16 @@ struct FalseC { static constexpr bool value = false; };
 
 // grid (Lp/128, Zk), 8 waves; wave w owns keys 16*(8*bx+w)..+15 and sweeps the 32-query blocks from its own on.
 // CM: the key tensor is stored in tiled k-group-major order (fused mode) rather than row-major (chunked mode).
+// Pruning (knorm2 != null; knorm2 [Zk][Lp/32] and qnorm2 [Zk*R][Lp/32] hold the largest squared row norm of every
+// block of 32 keys / queries): a key whose accumulated bias has fallen below -(kPruneLog2 + 2 max|k| max|q| log2 e)
+// cannot contribute a softmax weight above 2^-kPruneLog2 to any later query (the bias only decreases, a score
+// is at most max|k| max|q|, and a query's normaliser is at least its own score); a wave stops once all its 16
+// keys are there and records the last 32-query block it reached in reach[z][key tile].
 template <class T, int D, int NST, bool CM>
 __global__ void __launch_bounds__(512) k_carry2(const T* __restrict__ Kp, const float* __restrict__ lsrc,
-                                                const float* __restrict__ ldest, float* __restrict__ C, int Lp) {
+                                                const float* __restrict__ ldest, float* __restrict__ C, int Lp,
+                                                const float* __restrict__ knorm2, const float* __restrict__ qnorm2, int R,
+                                                int* __restrict__ reach) {
   using TN = Tile<T, 32, D, CM>;
   constexpr int NK = D / 32, SB = TN::BYTES + 1024;   // tile + [ldest of the block: 32 floats]
   UA_STAGES(SB);
@@ -104,6 +112,25 @@ __global__ void __launch_bounds__(512) k_carry2(const T* __restrict__ Kp, const 
   float carry = 0.f;
   float* Cz = C + (long)z * nT16 * Lp + spos;
   const T* Kz = Kp + (long)z * Lp * D;
+  bool dead = false;
+  int last = sb16 >> 1;
+  __shared__ int n_dead;
+  __shared__ float red[2][8];
+  float thr = -3.0e38f;
+  if (tid == 0) n_dead = 0;
+  if (knorm2) {
+    float km = 0.f, qm = 0.f;
+    for (int i = tid; i < nT; i += 512) km = fmaxf(km, knorm2[(long)z * nT + i]);
+    for (int i = tid; i < R * nT; i += 512) qm = fmaxf(qm, qnorm2[(long)z * R * nT + i]);
+#pragma unroll
+    for (int m = 1; m <= 32; m <<= 1) { km = fmaxf(km, __shfl_xor(km, m, 64)); qm = fmaxf(qm, __shfl_xor(qm, m, 64)); }
+    if (lane == 0) { red[0][w] = km; red[1][w] = qm; }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { km = fmaxf(km, red[0][i]); qm = fmaxf(qm, red[1][i]); }
+    thr = -(kPruneLog2 + 2.0f * kLog2e * sqrtf(km * qm));
+  }
+  __syncthreads();
 #define UA_ISSUE(s, base)                                                                   \
   {                                                                                         \
     st.issue((base), Kz + (long)32 * (first + (s)) * D, w);                                 \
@@ -117,6 +144,13 @@ __global__ void __launch_bounds__(512) k_carry2(const T* __restrict__ Kp, const 
   auto carry_step = [&] __device__ (int s, const char* base, auto masked_c) {
     constexpr bool MASKED = decltype(masked_c)::value;
     const int tb = first + s;
+    if (dead) return;
+    if (__builtin_amdgcn_ballot_w64(carry > thr) == 0) {        // every key of this wave is out of reach from here on
+      dead = true;
+      if (lane == 0) atomicAdd(&n_dead, 1);
+      return;
+    }
+    last = tb;
     const T* sK = reinterpret_cast<const T*>(base);
     const float* stats = reinterpret_cast<const float*>(base + TN::BYTES);
     f32x4 x[2];
@@ -143,14 +177,36 @@ __global__ void __launch_bounds__(512) k_carry2(const T* __restrict__ Kp, const 
     carry += t0 + t1;
   };
   {
-    const int total = nT - first, nslow = total < 4 ? total : 4;   // the first four blocks hold the diagonals
-    UA_PIPE_START(total, UA_ISSUE);
-    UA_PIPE_RANGE(0, nslow, total, UA_ISSUE, UA_COMPUTE_SLOW);
-    UA_PIPE_RANGE(nslow, total, total, UA_ISSUE, UA_COMPUTE_FAST);
+    // segments of 16 blocks, so that the workgroup can leave once all its waves have stopped
+    const int total = nT - first;
+    for (int s0 = 0; s0 < total; s0 += 16) {
+      const int s1 = min(total, s0 + 16);
+      UA_PIPE_START_AT(s0, s1, UA_ISSUE);
+      if (s0 == 0) {
+        const int nslow = s1 < 4 ? s1 : 4;                         // the first four blocks hold the diagonals
+        UA_PIPE_RANGE(0, nslow, s1, UA_ISSUE, UA_COMPUTE_SLOW);
+        UA_PIPE_RANGE(nslow, s1, s1, UA_ISSUE, UA_COMPUTE_FAST);
+      } else {
+        UA_PIPE_RANGE(s0, s1, s1, UA_ISSUE, UA_COMPUTE_FAST);
+      }
+      __syncthreads();
+      if (n_dead == 8) break;
+    }
   }
 #undef UA_ISSUE
 #undef UA_COMPUTE_FAST
 #undef UA_COMPUTE_SLOW
+  if (reach && lane == 0) reach[z * nT16 + sb16] = last;
+}
+
+// minkey[z][tb] = first key tile (of 16) that reaches query block tb; it never decreases with tb.
+template <class Unused = void>
+__global__ void __launch_bounds__(256) k_minkey(const int* __restrict__ reach, int* __restrict__ minkey, int nT16) {
+  const int z = blockIdx.y, tb = blockIdx.x * 256 + threadIdx.x, nT32 = nT16 / 2;
+  if (tb >= nT32) return;
+  int sb = 0;
+  while (sb < 2 * tb && reach[z * nT16 + sb] < tb) ++sb;          // tiles 2 tb and 2 tb + 1 hold the block's own keys
+  minkey[z * nT32 + tb] = sb;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -162,6 +218,7 @@ __global__ void __launch_bounds__(64 * NW) k_fwd_fused2(const T* __restrict__ Qp
                                                     const T* __restrict__ VT, const float* __restrict__ lsrc,
                                                     const float* __restrict__ ldest, const float* __restrict__ C,
                                                     T* __restrict__ O, float* __restrict__ lse, float* __restrict__ lse2,
+                                                    const int* __restrict__ reach, const int* __restrict__ minkey,
                                                     int R, int L, int Lp, int d) {
   using TN = Tile<T, 32, D>;
   using TT = Tile<T, D, 32>;
@@ -197,12 +254,22 @@ __global__ void __launch_bounds__(64 * NW) k_fwd_fused2(const T* __restrict__ Qp
 #pragma unroll
   for (int n = 0; n < ND; ++n) o[n] = (f32x4){0, 0, 0, 0};
   f32x4 m = {-1.0e30f, -1.0e30f, -1.0e30f, -1.0e30f}, ls = {0, 0, 0, 0};
-  const float* Crow = C + ((long)zk * nT16 + tq) * Lp;
-  const float* lsz = lsrc + (long)zk * Lp;
   const T* Kz = Kp + (long)zk * Lp * D;
   const T* Vz = VT + (long)zk * D * Lp;
   const int tq_end = min(NW * (jt + 1), nT16);
   const int n_kt = (tq_end + 3) / 4;   // key tiles of 64 covering s <= last query of the workgroup
+  // key tiles that cannot reach this workgroup's first query block (see k_carry2) are not visited at all; inside
+  // the visited range a tile that does not reach this wave's block gets a carry of -1e30 (its weights become 0)
+  const int tbq = tq >> 1;
+  const int kt_min = minkey[zk * (nT16 >> 1) + ((NW * jt) >> 1)] >> 2;
+  const int n_steps = n_kt - kt_min;
+  // per-wave stats row of a step: [C row: 64f][lsrc: 64f][reach of the 4 key tiles: 4 ints]; source of each lane's
+  // 16 bytes as base + step * stride (in 4-byte units)
+  const float* row_base;
+  int row_step = 64;
+  if (lane < 16) row_base = C + ((long)zk * nT16 + tq) * Lp + 4 * lane;
+  else if (lane < 32) row_base = lsrc + (long)zk * Lp + 4 * (lane - 16);
+  else { row_base = reinterpret_cast<const float*>(reach + zk * nT16); row_step = 4; }
 
 #define UA_ISSUE(s, base)                                                                   \
   {                                                                                         \
@@ -211,7 +278,7 @@ __global__ void __launch_bounds__(64 * NW) k_fwd_fused2(const T* __restrict__ Qp
     stN.issue((base) + TN::BYTES, Kz + (long)(64 * kt_ + 32) * D, w);                       \
     stT.issue((base) + 2 * TN::BYTES, Vz + (long)(2 * kt_) * (32 * D), w);                  \
     stT.issue((base) + 2 * TN::BYTES + TT::BYTES, Vz + (long)(2 * kt_ + 1) * (32 * D), w);  \
-    issue_row((base) + TILES + w * 1024, ((lane & 16) ? lsz : Crow) + 64 * kt_ + 4 * (lane & 15)); \
+    issue_row((base) + TILES + w * 1024, row_base + (long)kt_ * row_step);                  \
   }
 #define UA_COMPUTE_FAST(s, base) fwd_tile(n_kt - 1 - (s), (base), FalseC())
 #define UA_COMPUTE_SLOW(s, base) fwd_tile(n_kt - 1 - (s), (base), TrueC())
@@ -224,7 +291,7 @@ __global__ void __launch_bounds__(64 * NW) k_fwd_fused2(const T* __restrict__ Qp
       const int sbk = 4 * kt + j;                      // 16-key tile
       const T* sK = reinterpret_cast<const T*>(base + (j >> 1) * TN::BYTES);
       if (!MASKED || sbk <= tq) {
-        const float c = stats[16 * j + col];
+        const float c = reinterpret_cast<const int*>(stats)[128 + j] >= tbq ? stats[16 * j + col] : -1.0e30f;
         const float la = stats[64 + 16 * j + col];
         f32x4 gt = {0, 0, 0, 0}, sc = {0, 0, 0, 0};
 #pragma unroll
@@ -294,10 +361,10 @@ __global__ void __launch_bounds__(64 * NW) k_fwd_fused2(const T* __restrict__ Qp
   };
   {
     // the key tiles visited first hold the diagonal blocks of the waves
-    const int nslow = min(n_kt, (n_kt - (NW * jt) / 4 + 1) & ~1);
-    UA_PIPE_START(n_kt, UA_ISSUE);
-    UA_PIPE_RANGE(0, nslow, n_kt, UA_ISSUE, UA_COMPUTE_SLOW);
-    UA_PIPE_RANGE(nslow, n_kt, n_kt, UA_ISSUE, UA_COMPUTE_FAST);
+    const int nslow = min(n_steps, (n_kt - (NW * jt) / 4 + 1) & ~1);
+    UA_PIPE_START(n_steps, UA_ISSUE);
+    UA_PIPE_RANGE(0, nslow, n_steps, UA_ISSUE, UA_COMPUTE_SLOW);
+    UA_PIPE_RANGE(nslow, n_steps, n_steps, UA_ISSUE, UA_COMPUTE_FAST);
   }
 #undef UA_ISSUE
 #undef UA_COMPUTE_FAST
@@ -344,6 +411,14 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   const int kg = bx, sb16 = 8 * kg + w, spos = 16 * sb16 + col;      // key group 0 sweeps the most query blocks: first
   const int nTr = (L + 31) / 32, first = 4 * kg;
   if (first >= nTr) return;                      // every key of this workgroup is padding
+  // query blocks beyond the reach of a key tile (see k_carry2) are not visited: the sweep starts at the farthest
+  // block any of the 8 waves reaches, and a wave joins in at its own
+  const int* reach_z = a.reach + zk * nT16 + 8 * kg;
+  int top = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) top = max(top, reach_z[i]);
+  top = min(top, nTr - 1);
+  const int myreach = reach_z[w];
   const GroupMasks gm = group_masks(lane);
   Stager<TN, 8> stN;
   Stager<TT, 8> stT;
@@ -373,7 +448,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
 
 #define UA_ISSUE(s, base)                                                                   \
   {                                                                                         \
-    const int tb_ = nTr - 1 - (s) / R;                                                      \
+    const int tb_ = top - (s) / R;                                                          \
     const long zq_ = (long)zk * R + (s) % R;                                                \
     const long qo_ = (zq_ * Lp + 32 * tb_) * D;   /* tile base, natural and transposed */      \
     stN.issue((base), Kz + (long)(32 * tb_) * D, w);                                        \
@@ -391,16 +466,19 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
       issue_row((base) + TILES, src_);                                                      \
     }                                                                                       \
   }
-#define UA_COMPUTE_FAST(s, base) bwd_step((s), (base), FalseC(), false)
+#define UA_COMPUTE_FAST(s, base)                                                            \
+  {                                                                                         \
+    if (top - (s) / R <= myreach) bwd_step((s), (base), FalseC(), false);                   \
+  }
 #define UA_COMPUTE_SLOW(s, base)                                                            \
   {                                                                                         \
-    const int tb_ = nTr - 1 - (s) / R;                                                      \
-    if (tb_ >= (sb16 >> 1)) bwd_step((s), (base), TrueC(), tb_ == (sb16 >> 1));             \
+    const int tb_ = top - (s) / R;                                                          \
+    if (tb_ >= (sb16 >> 1) && tb_ <= myreach) bwd_step((s), (base), TrueC(), tb_ == (sb16 >> 1)); \
   }
   // MASKED: the step may be the query block that holds this wave's own keys (run-time flag diag)
   auto bwd_step = [&] __device__ (int s, const char* base, auto masked_c, const bool diag) {
     constexpr bool MASKED = decltype(masked_c)::value;
-    const int tb = nTr - 1 - s / R, r = s % R;
+    const int tb = top - s / R, r = s % R;
     const T* sKt = reinterpret_cast<const T*>(base);
     const T* sQ = reinterpret_cast<const T*>(base + TN::BYTES);
     const T* sdO = reinterpret_cast<const T*>(base + 2 * TN::BYTES);
@@ -489,7 +567,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   };
   {
     // the last four query blocks of the sweep hold the diagonal blocks of the eight waves
-    const int nblk = nTr - first, total = nblk * R, nfast = ((nblk > 4 ? nblk - 4 : 0) * R) & ~1;
+    const int nblk = top + 1 - first, total = nblk * R, nfast = ((nblk > 4 ? nblk - 4 : 0) * R) & ~1;
     UA_PIPE_START(total, UA_ISSUE);
     UA_PIPE_RANGE(0, nfast, total, UA_ISSUE, UA_COMPUTE_FAST);
     UA_PIPE_RANGE(nfast, total, total, UA_ISSUE, UA_COMPUTE_SLOW);
@@ -549,13 +627,22 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
   f32x4 dKc[ND];
 #pragma unroll
   for (int n = 0; n < ND; ++n) dKc[n] = (f32x4){0, 0, 0, 0};
-  const float* Crow = a.C + ((long)zk * nT16 + tq) * Lp;
-  const float* Drow = a.Dsuf + ((long)zk * nT16 + tq) * Lp;
-  const float* lsz = a.lsrc + (long)zk * Lp;
   const T* Kz = a.Kp + (long)zk * Lp * D;
   const T* Vz = a.Vp + (long)zk * Lp * D;
   const T* KTz = a.KT + (long)zk * D * Lp;
   const int n_kt = 2 * jt + 2;
+  // key tiles out of reach of this workgroup's first query block are not visited (see k_carry2); inside the range
+  // a tile that does not reach this wave's block gets a carry of -1e30, which zeroes its dS and dG
+  const int tbq = tq >> 1;
+  const int kt_min = (a.minkey[zk * (nT16 >> 1) + 4 * jt] >> 2) & ~1;
+  // per-wave stats row of a step: [C row: 64f][lsrc: 64f][Dsuf row: 64f][reach of the 4 key tiles: 4 ints]; source of
+  // each lane's 16 bytes as base + step * stride (in 4-byte units)
+  const float* row_base;
+  int row_step = 64;
+  if (lane < 16) row_base = a.C + ((long)zk * nT16 + tq) * Lp + 4 * lane;
+  else if (lane < 32) row_base = a.lsrc + (long)zk * Lp + 4 * (lane - 16);
+  else if (lane < 48) row_base = a.Dsuf + ((long)zk * nT16 + tq) * Lp + 4 * (lane - 32);
+  else { row_base = reinterpret_cast<const float*>(a.reach + zk * nT16); row_step = 4; }
   // column of key (16*(j&1) + col) inside its 32-key group of the transposed key tile
   const int pc0 = perm32(col), pc1 = perm32(16 + col);
 
@@ -584,8 +671,7 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
     stN.issue((base) + 3 * TN::BYTES, Vz + (long)(k0_ + 32) * D, w);                        \
     stT.issue((base) + 4 * TN::BYTES, KTz + (long)k0_ * D, w);                              \
     stT.issue((base) + 4 * TN::BYTES + TT::BYTES, KTz + (long)(k0_ + 32) * D, w);           \
-    issue_row((base) + TILES + w * 1024,                                                    \
-              (lane < 16 ? Crow : (lane < 32 ? lsz : Drow)) + k0_ + 4 * (lane & 15));       \
+    issue_row((base) + TILES + w * 1024, row_base + (long)(s) * row_step);                  \
   }
 #define UA_COMPUTE_FAST(s, base) bq_step((s), (base), FalseC())
 #define UA_COMPUTE_SLOW(s, base) bq_step((s), (base), TrueC())
@@ -605,9 +691,10 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
           if (live) {
             const T* sK = reinterpret_cast<const T*>(base + kq * TN::BYTES);
             const T* sV = reinterpret_cast<const T*>(base + (2 + kq) * TN::BYTES);
-            const float cin = stats[16 * j + col];
+            const bool in_reach = reinterpret_cast<const int*>(stats)[192 + j] >= tbq;
+            const float cin = in_reach ? stats[16 * j + col] : -1.0e30f;
             const float la = stats[64 + 16 * j + col];
-            const float din = (r == 0) ? stats[128 + 16 * j + col] : 0.f;
+            const float din = (r == 0 && in_reach) ? stats[128 + 16 * j + col] : 0.f;
             f32x4 acc = {0, 0, 0, 0}, sc = {0, 0, 0, 0}, dP = {0, 0, 0, 0};
 #pragma unroll
             for (int q = 0; q < NK; ++q) {
@@ -663,9 +750,9 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
     };
     {
       // the last two key tiles hold the diagonal blocks of the eight waves
-      const int nfast = n_kt - 2;
-      UA_PIPE_START(n_kt, UA_ISSUE);
-      UA_PIPE_RANGE(0, nfast, n_kt, UA_ISSUE, UA_COMPUTE_FAST);
+      const int nfast = max(n_kt - 2, kt_min);
+      UA_PIPE_START_AT(kt_min, n_kt, UA_ISSUE);
+      UA_PIPE_RANGE(kt_min, nfast, n_kt, UA_ISSUE, UA_COMPUTE_FAST);
       UA_PIPE_RANGE(nfast, n_kt, n_kt, UA_ISSUE, UA_COMPUTE_SLOW);
     }
 #undef UA_ISSUE
@@ -695,6 +782,7 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
 #undef UA_PIPELINE
 #undef UA_PIPE_RANGE
 #undef UA_PIPE_START
+#undef UA_PIPE_START_AT
 #undef UA_STEP2_
 #undef UA_STAGES
 

@@ -8,6 +8,7 @@ namespace ua {
 template <class T>
 static BwdArgs<T> typed(const BwdArgsV& v) {
   BwdArgs<T> a;
+  a.reach = v.reach; a.minkey = v.minkey;
   a.Kp = (const T*)v.Kp; a.Vp = (const T*)v.Vp; a.KT = (const T*)v.KT; a.Qp = (const T*)v.Qp; a.QT = (const T*)v.QT;
   a.dOp = (const T*)v.dOp; a.dOT = (const T*)v.dOT; a.lsrc = v.lsrc; a.ldest = v.ldest; a.lse2 = v.lse2; a.delta = v.delta;
   a.C = v.C;

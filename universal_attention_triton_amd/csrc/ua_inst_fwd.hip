@@ -11,22 +11,30 @@ static void allow_lds(K kernel, size_t bytes) {
 }
 
 template <class T, int D>
-static hipError_t carry_t(const void* Kp, const float* lsrc, const float* ldest, float* C, int Lp, int Zk, int tiled, hipStream_t s) {
+static hipError_t carry_t(const void* Kp, const float* lsrc, const float* ldest, float* C, int Lp, int Zk, int tiled,
+                          const float* knorm2, const float* qnorm2, int R, int* reach, int* minkey, hipStream_t s) {
   constexpr int NST = 2;
-  if (tiled) hipLaunchKernelGGL((k_carry2<T, D, NST, true>), dim3(Lp / 128, Zk), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, C, Lp);
-  else hipLaunchKernelGGL((k_carry2<T, D, NST, false>), dim3(Lp / 128, Zk), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, C, Lp);
-  return hipGetLastError();
+  if (tiled) hipLaunchKernelGGL((k_carry2<T, D, NST, true>), dim3(Lp / 128, Zk), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, C, Lp, knorm2, qnorm2, R, reach);
+  else hipLaunchKernelGGL((k_carry2<T, D, NST, false>), dim3(Lp / 128, Zk), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, C, Lp, knorm2, qnorm2, R, reach);
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess && reach && minkey) {
+    hipLaunchKernelGGL((k_minkey<>), dim3((Lp / 32 + 255) / 256, Zk), dim3(256), 0, s, (const int*)reach, minkey, Lp / 16);
+    e = hipGetLastError();
+  }
+  return e;
 }
 hipError_t launch_carry(int dtype, int D, const void* Kp, const float* lsrc, const float* ldest, float* C, int Lp, int Zk,
-                        int tiled, hipStream_t s) {
-  if (dtype == 1) return D == 64 ? carry_t<bf16, 64>(Kp, lsrc, ldest, C, Lp, Zk, tiled, s) : carry_t<bf16, 128>(Kp, lsrc, ldest, C, Lp, Zk, tiled, s);
-  return D == 64 ? carry_t<float, 64>(Kp, lsrc, ldest, C, Lp, Zk, tiled, s) : carry_t<float, 128>(Kp, lsrc, ldest, C, Lp, Zk, tiled, s);
+                        int tiled, const float* knorm2, const float* qnorm2, int R, int* reach, int* minkey, hipStream_t s) {
+#define UA_ARGS Kp, lsrc, ldest, C, Lp, Zk, tiled, knorm2, qnorm2, R, reach, minkey, s
+  if (dtype == 1) return D == 64 ? carry_t<bf16, 64>(UA_ARGS) : carry_t<bf16, 128>(UA_ARGS);
+  return D == 64 ? carry_t<float, 64>(UA_ARGS) : carry_t<float, 128>(UA_ARGS);
+#undef UA_ARGS
 }
 
 // explicit instantiations (the implicit ones are not emitted on the host side for these kernels)
 #define UA_INST(T, D, NST, NW)                                                                                        \
   template __global__ void k_fwd_fused2<T, D, NST, NW>(const T*, const T*, const T*, const float*, const float*,      \
-                                                       const float*, T*, float*, float*, int, int, int, int);
+                                                       const float*, T*, float*, float*, const int*, const int*, int, int, int, int);
 UA_INST(bf16, 64, 1, 8) UA_INST(bf16, 64, 2, 8) UA_INST(bf16, 64, 2, 12) UA_INST(bf16, 64, 2, 16)
 UA_INST(bf16, 128, 1, 8) UA_INST(bf16, 128, 2, 8) UA_INST(bf16, 128, 2, 12) UA_INST(bf16, 128, 2, 16)
 UA_INST(float, 64, 1, 8) UA_INST(float, 128, 1, 8)
@@ -34,9 +42,10 @@ UA_INST(float, 64, 1, 8) UA_INST(float, 128, 1, 8)
 
 template <class T, int D, int NST, int NW>
 static hipError_t fused_t(const void* Qp, const void* Kp, const void* VT, const float* lsrc, const float* ldest,
-                          const float* C, void* O, float* lse, float* lse2, int R, int L, int Lp, int d, int Zq, hipStream_t s) {
+                          const float* C, void* O, float* lse, float* lse2, const int* reach, const int* minkey, int R, int L,
+                          int Lp, int d, int Zq, hipStream_t s) {
   hipLaunchKernelGGL((k_fwd_fused2<T, D, NST, NW>), dim3((Lp / 16 + NW - 1) / NW, Zq), dim3(64 * NW), 0, s, (const T*)Qp,
-                     (const T*)Kp, (const T*)VT, lsrc, ldest, C, (T*)O, lse, lse2, R, L, Lp, d);
+                     (const T*)Kp, (const T*)VT, lsrc, ldest, C, (T*)O, lse, lse2, reach, minkey, R, L, Lp, d);
   return hipGetLastError();
 }
 // variants (bf16): 0 = 8 waves, double-buffered stages; 1 = 8 waves, single stage; 2 = 12 waves; 3 = 16 waves
@@ -44,8 +53,9 @@ static hipError_t fused_t(const void* Qp, const void* Kp, const void* VT, const 
 int fwd_fused_variants(int dtype, int D) { (void)D; return dtype == 1 ? 4 : 1; }
 template <class T, int D>
 static hipError_t fused_v(int variant, const void* Qp, const void* Kp, const void* VT, const float* lsrc, const float* ldest,
-                          const float* C, void* O, float* lse, float* lse2, int R, int L, int Lp, int d, int Zq, hipStream_t s) {
-#define UA_ARGS Qp, Kp, VT, lsrc, ldest, C, O, lse, lse2, R, L, Lp, d, Zq, s
+                          const float* C, void* O, float* lse, float* lse2, const int* reach, const int* minkey, int R, int L,
+                          int Lp, int d, int Zq, hipStream_t s) {
+#define UA_ARGS Qp, Kp, VT, lsrc, ldest, C, O, lse, lse2, reach, minkey, R, L, Lp, d, Zq, s
   switch (variant) {
     case 1: return fused_t<T, D, 1, 8>(UA_ARGS);
     case 2: return fused_t<T, D, 2, 12>(UA_ARGS);
@@ -55,9 +65,9 @@ static hipError_t fused_v(int variant, const void* Qp, const void* Kp, const voi
 #undef UA_ARGS
 }
 hipError_t launch_fwd_fused(int dtype, int D, int variant, const void* Qp, const void* Kp, const void* VT,
-                            const float* lsrc, const float* ldest, const float* C, void* O, float* lse, float* lse2, int R,
-                            int L, int Lp, int d, int Zq, hipStream_t s) {
-#define UA_ARGS Qp, Kp, VT, lsrc, ldest, C, O, lse, lse2, R, L, Lp, d, Zq, s
+                            const float* lsrc, const float* ldest, const float* C, void* O, float* lse, float* lse2,
+                            const int* reach, const int* minkey, int R, int L, int Lp, int d, int Zq, hipStream_t s) {
+#define UA_ARGS Qp, Kp, VT, lsrc, ldest, C, O, lse, lse2, reach, minkey, R, L, Lp, d, Zq, s
   if (dtype == 1) return D == 64 ? fused_v<bf16, 64>(variant, UA_ARGS) : fused_v<bf16, 128>(variant, UA_ARGS);
   return D == 64 ? fused_t<float, 64, 1, 8>(UA_ARGS) : fused_t<float, 128, 1, 8>(UA_ARGS);
 #undef UA_ARGS

@@ -28,7 +28,7 @@ __device__ __forceinline__ long rows_offset(const RowsView& v, int z, int row) {
 // rows are read with 16-byte loads.
 template <class T, int D>
 __global__ void __launch_bounds__(256) k_pack(RowsView x, T* __restrict__ nat, T* __restrict__ tr, int d, int L, int Lp,
-                                              int tr_mode, int tiled, int vec) {
+                                              int tr_mode, int tiled, int vec, float* __restrict__ norm2) {
   constexpr int V = 16 / (int)sizeof(T);
   __shared__ float tile[32][D + 1];
   const int z = blockIdx.y, row0 = blockIdx.x * 32, tid = threadIdx.x;
@@ -56,8 +56,23 @@ __global__ void __launch_bounds__(256) k_pack(RowsView x, T* __restrict__ nat, T
       if (nat && !tiled) nat[((long)z * Lp + row) * D + col] = cvt<T>(val);
     }
   }
-  if (!tr && !(nat && tiled)) return;
+  if (!tr && !(nat && tiled) && !norm2) return;
   __syncthreads();
+  if (norm2) {
+    // largest squared row norm of the block's (dtype-rounded) rows -> norm2[z][block]: 8 threads per row, then the
+    // maximum over the block
+    __shared__ float wmax[4];
+    const int rr = tid >> 3;
+    float s2 = 0.f;
+    for (int c = tid & 7; c < D; c += 8) s2 += tile[rr][c] * tile[rr][c];
+#pragma unroll
+    for (int m = 1; m <= 4; m <<= 1) s2 += __shfl_xor(s2, m, 64);             // the 8 threads of a row
+#pragma unroll
+    for (int m = 8; m <= 32; m <<= 1) s2 = fmaxf(s2, __shfl_xor(s2, m, 64));   // the 8 rows of a wave
+    if ((tid & 63) == 0) wmax[tid >> 6] = s2;
+    __syncthreads();
+    if (tid == 0) norm2[(long)z * gridDim.x + blockIdx.x] = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
+  }
   if (nat && tiled) {
     // one (k-group, row) cell of 8 elements per thread; consecutive threads write consecutive cells
     for (int i = tid; i < 4 * D; i += 256) {

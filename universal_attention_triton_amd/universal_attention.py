@@ -40,9 +40,10 @@ class UniversalAttention(_ChunkedBase):
 
 class _FusedUniversalAttention(Function):
     @staticmethod
-    def forward(ctx, kc, vc, xq, static_src, static_dest):
+    def forward(ctx, kc, vc, xq, static_src, static_dest, prune=False):
         need_grad = any(ctx.needs_input_grad)
-        O, lse, ws = ops.fused_forward(kc, vc, xq, static_src, static_dest, for_backward=need_grad)
+        O, lse, ws = ops.fused_forward(kc, vc, xq, static_src, static_dest, for_backward=need_grad, prune=prune)
+        ctx.prune = prune
         ctx.save_for_backward(kc, vc, xq, static_src, static_dest, O, lse)
         ctx.ws = ws if need_grad else None
         ctx.mark_non_differentiable(lse)
@@ -53,15 +54,16 @@ class _FusedUniversalAttention(Function):
         kc, vc, xq, static_src, static_dest, O, lse = ctx.saved_tensors
         b, h, n, c, d = kc.shape
         dO = dO.reshape(b, h, xq.shape[2], n * c, d)
-        dk, dv, dq, dsrc, ddest = ops.fused_backward(kc, vc, xq, static_src, static_dest, O, lse, dO, ws=ctx.ws)
+        dk, dv, dq, dsrc, ddest = ops.fused_backward(kc, vc, xq, static_src, static_dest, O, lse, dO, ws=ctx.ws, prune=ctx.prune)
         ctx.ws = None
-        return dk, dv, dq.view(xq.shape), dsrc.view(static_src.shape), ddest.view(static_dest.shape)
+        return dk, dv, dq.view(xq.shape), dsrc.view(static_src.shape), ddest.view(static_dest.shape), None
 
 
-def universal_attention(kc, vc, xq, static_src, static_dest, return_lse=False):
+def universal_attention(kc, vc, xq, static_src, static_dest, return_lse=False, prune=False):
     """Fused forward/backward.  Accepts the 1-D (xq [b,h,r,l,d]) and the 2-D (xq [b,h,r,_n,_c,d]) layouts;
-    the result has xq's shape."""
-    O, lse = _FusedUniversalAttention.apply(kc, vc, xq, static_src, static_dest)
+    the result has xq's shape.  prune=True skips (key, query) pairs whose softmax weight is provably below 2^-48
+    because of the accumulated decay: same results to float32 rounding, less work on long sequences."""
+    O, lse = _FusedUniversalAttention.apply(kc, vc, xq, static_src, static_dest, prune)
     return (O, lse) if return_lse else O
 
 
