@@ -8,6 +8,7 @@ upstream gradient dO shaped like the output).  Prints ONE JSON line:
   roofline  the dominant kernel (k_bwd_keys: the six causal products it evaluates, G, S, dP, dV, dK(score side),
             dK(decay side) = (2+4r) d L^2 b h flops per launch) against the bf16 dense MFMA peak, its duration
             measured with hipEvents on the launch stream during the timed steps
+  config.pruned_mode  the same step with the optional pruning of provably negligible pairs (never part of `value`)
   cpu_baseline  the oracle (a port of the reference's torch operator) timed on the host cores on a bounded sample:
             whole kv heads of the same workload, one after the other, until about 10 s have passed
 """
@@ -102,13 +103,13 @@ def main():
     dO = inp["dO"].cuda()
 
     if cfg["bwd"]:
-        def step():
-            O = universal_attention(*leaves)
+        def step(prune=False):
+            O = universal_attention(*leaves, prune=prune)
             return torch.autograd.grad(O, leaves, dO)
     else:
-        def step():
+        def step(prune=False):
             with torch.no_grad():
-                return universal_attention(*leaves)
+                return universal_attention(*leaves, prune=prune)
 
     if args.calibrate_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").fill_(1.0)
@@ -150,6 +151,18 @@ def main():
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
                      "frac": round(achieved / peak, 4), "traffic": None},
     }
+    # the same step with UA_FLAG_PRUNE (pairs whose softmax weight is provably below 2^-48 are skipped): reported
+    # beside the headline, never as `value`, because it executes fewer pairs than the flop count assumes
+    for _ in range(2):
+        step(prune=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(prune=True)
+    torch.cuda.synchronize()
+    ms_p = (time.perf_counter() - t0) * 1e3 / args.steps
+    out["config"]["pruned_mode"] = {"ms_per_step": round(ms_p, 4), "speedup": round(ms / ms_p, 2),
+                                    "note": "optional exact pruning of negligible pairs; not counted in value"}
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(cfg, args.config)
     print(json.dumps(out))
