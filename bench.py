@@ -83,6 +83,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", type=int, default=2)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--api", choices=["fused", "chunked"], default="fused",
+                    help="fused (default): universal_attention(); chunked: the reference's call sequence "
+                         "UniversalAttention.apply + SMVecMatMul.apply, which materialises out[b,h,r,L,d,n]")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device-to-device copy, the known-size kernel that HBM counters of a "
                          "profiler run are scaled against")
@@ -102,7 +105,14 @@ def main():
     leaves = [inp[k].cuda().requires_grad_() for k in names]
     dO = inp["dO"].cuda()
 
-    if cfg["bwd"]:
+    if args.api == "chunked":
+        import universal_attention_autograd as ref_api
+
+        def step(prune=False):
+            out_c, denom_c = ref_api.UniversalAttention.apply(*leaves)
+            O = ref_api.SMVecMatMul.apply(out_c, denom_c)
+            return torch.autograd.grad(O, leaves, dO) if cfg["bwd"] else O
+    elif cfg["bwd"]:
         def step(prune=False):
             O = universal_attention(*leaves, prune=prune)
             return torch.autograd.grad(O, leaves, dO)
@@ -135,10 +145,20 @@ def main():
     if not cfg["bwd"]:
         f_bwd = 0
     dom = "k_bwd_keys" if cfg["bwd"] else "k_fwd_fused"
+    if args.api == "chunked":
+        dom = "k_fwd_chunked"
     kern = {k: round(v[1] / v[0], 4) for k, v in prof.items()}
     dom_ms = prof[dom][1] / prof[dom][0]
     peak = PEAK_TFLOPS[cfg["dtype"]]
-    achieved = kernel_flops(cfg, dom) / (dom_ms * 1e-3) / 1e12
+    if args.api == "chunked":
+        # the chunked forward is bound by writing out[b,h,r,L,d,n] and denom[b,h,r,L,n]
+        n_chunks = cfg["L"] // cfg["c"]
+        esz = 2 if cfg["dtype"] == "bf16" else 4
+        out_bytes = cfg["b"] * cfg["h"] * cfg["r"] * cfg["L"] * n_chunks * (cfg["d"] + 1) * esz
+        gbs = out_bytes / (dom_ms * 1e-3) / 1e9
+        roof = {"bound": "hbm", "kernel": dom, "achieved": round(gbs, 1), "peak": 8000.0, "unit": "GB/s",
+                "frac": round(gbs / 8000.0, 4), "traffic": None}
+    achieved = kernel_flops(cfg, dom if args.api == "fused" else "k_fwd_fused") / (dom_ms * 1e-3) / 1e12
     out = {
         "metric": "fwd+bwd ms and TFLOP/s (bf16, L=8192, d=128) on 1 MI355X; % MFMA peak", "value": round((f_fwd + f_bwd) / (ms * 1e-3) / 1e12, 2),
         "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
@@ -151,6 +171,14 @@ def main():
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
                      "frac": round(achieved / peak, 4), "traffic": None},
     }
+    if args.api == "chunked":
+        out["roofline"] = roof
+        out["config"]["workload"] += "; chunked API (reference call sequence, chunk %d)" % cfg["c"]
+        out["config"].pop("pct_of_mfma_peak", None)
+        if not args.no_cpu:
+            out["cpu_baseline"] = cpu_baseline(cfg, args.config)
+        print(json.dumps(out))
+        return
     # the same step with UA_FLAG_PRUNE (pairs whose softmax weight is provably below 2^-48 are skipped): reported
     # beside the headline, never as `value`, because it executes fewer pairs than the flop count assumes
     for _ in range(2):

@@ -180,8 +180,13 @@ hipError_t zero_fill(void* p, size_t bytes, hipStream_t s) {   // bytes is a mul
 }
 
 // packs K, V and Q in both orientations and the log-gates
-int pack_inputs(const ua_desc& d, const Layout& l, bool chunked, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq,
+// chunk sizes the query-stationary kernels handle (the others go through the key-chunk-stationary ones)
+bool fast_chunk(const ua_desc& d) { return d.chunk % 64 == 0; }
+
+// rowmajor: working tensors for the key-chunk-stationary (32x32 tile) kernels; otherwise the tiled layout
+int pack_inputs(const ua_desc& d, const Layout& l, bool rowmajor, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq,
                 const void* src, const void* dest, char* ws, hipStream_t s) {
+  const bool chunked = rowmajor;
   UA_PROF("pack_inputs", s);
   const ua::RowsView K = rows_view(*kc, d.h, 1), V = rows_view(*vc, d.h, 1), Q = rows_view(*xq, d.h, d.r);
   // the chunked kernels work on 32x32 tiles, the fused ones on 16x16 tiles (and read V^T in natural order)
@@ -349,6 +354,20 @@ int ua_fwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
   char* w = (char*)ws;
   hipStream_t s = (hipStream_t)stream;
   const ua_desc& d = *desc;
+  if (fast_chunk(d)) {
+    if (int e = pack_inputs(d, l, false, kc, vc, xq, static_src, static_dest, w, s)) return e;
+    {
+      UA_PROF("k_carry", s);
+      UA_HIP(ua::launch_carry(d.dtype, l.D, w + l.Kp, (const float*)(w + l.lsrc), (const float*)(w + l.ldest), (float*)(w + l.C), l.Lp,
+                              l.Zk, 1, nullptr, nullptr, d.r, (int*)(w + l.reach), (int*)(w + l.minkey), s));
+    }
+    UA_PROF("k_fwd_chunked", s);
+    UA_HIP(ua::launch_fwd_chunked2(d.dtype, l.D, w + l.Qp, w + l.Kp, w + l.Vp, w + l.VT, (const float*)(w + l.lsrc),
+                                   (const float*)(w + l.ldest), (const float*)(w + l.C), (const int*)(w + l.reach),
+                                   (const int*)(w + l.minkey), out->ptr, denom, (float*)(w + l.lse2), out->stride_z, out->stride_t,
+                                   out->stride_d, out->stride_i, d.r, d.L, l.Lp, d.d, d.chunk, l.nch, l.Zq, s));
+    return UA_OK;
+  }
   if (int e = pack_inputs(d, l, true, kc, vc, xq, static_src, static_dest, w, s)) return e;
   UA_PROF("k_fwd_chunked", s);
   UA_HIP(ua::launch_fwd_chunked(d.dtype, l.D, w + l.Qp, w + l.Kp, w + l.VT, (const float*)(w + l.lsrc),
@@ -368,6 +387,10 @@ int ua_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
   char* w = (char*)ws;
   hipStream_t s = (hipStream_t)stream;
   const ua_desc& d = *desc;
+  if (ws_has_fwd && fast_chunk(d)) {
+    // the forward left tiled working tensors; the key-chunk-stationary backward reads row-major ones
+    if (int e = pack_inputs(d, l, true, kc, vc, xq, static_src, static_dest, w, s)) return e;
+  }
   if (!ws_has_fwd) {
     // recompute the per-chunk normalisers (the partial outputs themselves are passed in)
     if (int e = pack_inputs(d, l, true, kc, vc, xq, static_src, static_dest, w, s)) return e;

@@ -31,6 +31,8 @@ constexpr float kLn2 = 0.6931471805599453f;
 constexpr float kAMax = (float)(1.0 - 1e-6);      // upper clamp of the affinity (forward and backward)
 constexpr float kPruneLog2 = 48.0f;               // softmax weights provably below 2^-48 are dropped when pruning
 constexpr float kAMinBwd = 1e-6f;                 // lower clamp used only in the backward divisor
+// marker stored in the log2-unit normaliser buffer for a (query, chunk) pair with no visible key
+constexpr float kNoKeyLse = 3.0e38f;
 constexpr float kNegFill = -1e12f;                // bias of a (key, query) pair with key > query
 constexpr int kPad16 = 16;                        // bytes of padding per LDS row
 

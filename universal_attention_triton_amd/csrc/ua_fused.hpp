@@ -209,17 +209,76 @@ __global__ void __launch_bounds__(256) k_minkey(const int* __restrict__ reach, i
   minkey[z * nT32 + tb] = sb;
 }
 
+// Destination of the per-chunk results of the chunked operator (reference universal_attention_autograd.py:9-38):
+// out element (zq, t, dd, i) at zq*sz + t*st + dd*sd + i*si, denom [Zq][L][nch]; either may be null.
+template <class T> struct ChunkOut {
+  T* out;
+  T* denom;
+  long sz, st, sd, si;
+  int c, nch;
+  int vec;      // rows of out[.., i] are contiguous in dd (sd == 1), 16-byte aligned, and d is a multiple of the vector
+};
+
+// Queries that precede a whole chunk see none of its keys; the reference's softmax over a row of equal fill values
+// is uniform there: out = mean of the chunk's values (through a dtype-rounded 1/c), denom = float32(-1e12).
+// grid (ceil(max rows / 256), nch, Zq), 256 threads: slab x of chunk i writes rows [256 x, 256 x + 256) ∩ [0, i*c) of
+// out[.., i].  vec: rows of out[.., i] are contiguous in dd, 16-byte aligned and d is a multiple of the vector.
+template <class T, int D>
+__global__ void __launch_bounds__(256) k_chunk_masked_out(const T* __restrict__ Vp, ChunkOut<T> co, int R, int L, int Lp, int d,
+                                                          int vec) {
+  constexpr int V = 16 / (int)sizeof(T);
+  __shared__ __attribute__((aligned(16))) T mean[D];
+  const int i = blockIdx.y, zq = blockIdx.z, zk = zq / R, tid = threadIdx.x;
+  const int rows = min(i * co.c, L), r0 = blockIdx.x * 256, r1 = min(rows, r0 + 256);
+  if (r0 >= rows) return;
+  const float pu = (float)cvt<T>(1.0f / (float)co.c);
+  for (int dd = tid; dd < D; dd += 256) {
+    float acc = 0.f;
+    for (int s = 0; s < co.c; ++s) acc += pu * (float)Vp[nat_off<D>(zk, Lp, i * co.c + s, dd)];
+    mean[dd] = cvt<T>(acc);
+  }
+  __syncthreads();
+  T* base = co.out + (long)zq * co.sz + (long)i * co.si;
+  if (vec) {
+    const int vpr = d / V;                                      // vectors per row
+    for (int idx = tid; idx < (r1 - r0) * vpr; idx += 256) {
+      const int t = r0 + idx / vpr, cv = idx % vpr;
+      *reinterpret_cast<uint4*>(base + (long)t * co.st + cv * V) = *reinterpret_cast<const uint4*>(mean + cv * V);
+    }
+  } else {
+    for (int idx = tid; idx < (r1 - r0) * d; idx += 256) {
+      const int t = r0 + idx / d, dd = idx % d;
+      base[(long)t * co.st + (long)dd * co.sd] = mean[dd];
+    }
+  }
+}
+// denom[zq][t][i] = -1e12 and lse2[zq*nch + i][t] = "no visible key" for the chunks i after the one holding query t.
+// grid (ceil(Lp/256), Zq); denom may be null.
+template <class T>
+__global__ void __launch_bounds__(256) k_chunk_masked_denom(T* __restrict__ denom, float* __restrict__ lse2, int L, int Lp,
+                                                            int c, int nch) {
+  const int t = blockIdx.x * 256 + threadIdx.x, zq = blockIdx.y;
+  if (t >= Lp) return;
+  const T fill = cvt<T>(kNegFill);
+  for (int i = t / c + 1; i < nch; ++i) {
+    if (denom && t < L) denom[((long)zq * L + t) * nch + i] = fill;
+    lse2[((long)zq * nch + i) * Lp + t] = kNoKeyLse;
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // Fused forward.  grid (ceil(Lp/16/NW), Zq); NW waves; wave w owns queries 16*(NW*jt+w)..+15; 64 keys per step,
 // key tiles visited from the diagonal backwards.
 // ---------------------------------------------------------------------------------------------
-template <class T, int D, int NST, int NW>
-__global__ void __launch_bounds__(64 * NW) k_fwd_fused2(const T* __restrict__ Qp, const T* __restrict__ Kp,
+// CHUNKED: the reference's chunked operator instead of the merged one: the softmax restarts at every chunk of
+// co.c keys (a multiple of 64) and each chunk's result goes to out[.., i] / denom[.., i] / lse2[zq*nch + i][t].
+template <class T, int D, int NST, int NW, bool CHUNKED>
+__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4, NW / 4))) k_fwd_fused2(const T* __restrict__ Qp, const T* __restrict__ Kp,
                                                     const T* __restrict__ VT, const float* __restrict__ lsrc,
                                                     const float* __restrict__ ldest, const float* __restrict__ C,
                                                     T* __restrict__ O, float* __restrict__ lse, float* __restrict__ lse2,
                                                     const int* __restrict__ reach, const int* __restrict__ minkey,
-                                                    int R, int L, int Lp, int d) {
+                                                    int R, int L, int Lp, int d, ChunkOut<T> co) {
   using TN = Tile<T, 32, D>;
   using TT = Tile<T, D, 32>;
   constexpr int NK = D / 32, ND = D / 16;
@@ -235,6 +294,9 @@ __global__ void __launch_bounds__(64 * NW) k_fwd_fused2(const T* __restrict__ Qp
   const bool live = NW * jt + w < nT16;                      // the last workgroup may hold waves past the end
   const int tq = live ? NW * jt + w : nT16 - 1;             // 16-query tile of this wave
   char* sPw = sPbuf + w * 2 * ST::BYTES;     // P of the two 32-key halves of a step
+  // chunked operator, 16-bit outputs: per-wave [16 queries][D + 8] tile through which a chunk's result is transposed
+  __shared__ __attribute__((aligned(16))) T sObuf[(CHUNKED && sizeof(T) == 2) ? NW * 16 * (D + 8) : 8];
+  T* sOw = sObuf + ((CHUNKED && sizeof(T) == 2) ? w * 16 * (D + 8) : 0);
   const GroupMasks gm = group_masks(lane);
   Stager<TN, NW> stN;
   Stager<TT, NW> stT;
@@ -282,6 +344,48 @@ __global__ void __launch_bounds__(64 * NW) k_fwd_fused2(const T* __restrict__ Qp
   }
 #define UA_COMPUTE_FAST(s, base) fwd_tile(n_kt - 1 - (s), (base), FalseC())
 #define UA_COMPUTE_SLOW(s, base) fwd_tile(n_kt - 1 - (s), (base), TrueC())
+  // chunked operator: chunk i is complete, write its normalised result and restart the softmax
+  auto flush_chunk = [&] __device__ (int i) __attribute__((always_inline)) {
+    if (live && i <= (16 * tq) / co.c) {     // chunks after this wave's queries are written by k_chunk_masked_*
+      const bool via_lds = sizeof(T) == 2 && co.vec && co.out;
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const float tot = allsum16(ls[v]);
+        const float inv = 1.0f / tot;
+        const int t = 16 * tq + 4 * g + v;
+        if (via_lds) {
+          // transpose through the wave's LDS tile [16 queries][D] so that rows leave as 16-byte vectors
+#pragma unroll
+          for (int n = 0; n < ND; ++n) sOw[(4 * g + v) * (D + 8) + 16 * n + col] = cvt<T>(o[n][v] * inv);
+        } else if (t < L && co.out) {
+#pragma unroll
+          for (int n = 0; n < ND; ++n) {
+            const int dd = 16 * n + col;
+            if (dd < d) co.out[(long)zq * co.sz + (long)t * co.st + (long)dd * co.sd + (long)i * co.si] = cvt<T>(o[n][v] * inv);
+          }
+        }
+        if (col == 0) {
+          const float l2v = m[v] + __builtin_amdgcn_logf(tot);
+          lse2[((long)zq * co.nch + i) * Lp + t] = (t < L) ? l2v : 0.f;
+          if (t < L && co.denom) co.denom[((long)zq * L + t) * co.nch + i] = cvt<T>(l2v * kLn2);
+        }
+      }
+      if (via_lds) {
+        constexpr int VPR = D / 8;                               // 16-byte vectors per row
+        T* dst = co.out + (long)zq * co.sz + (long)i * co.si;
+#pragma unroll
+        for (int k = 0; k < 16 * VPR / 64; ++k) {
+          const int idx = 64 * k + lane, row = idx / VPR, cv = idx % VPR, t = 16 * tq + row;
+          if (t < L && 8 * cv < d)
+            *reinterpret_cast<uint4*>(dst + (long)t * co.st + 8 * cv) = *reinterpret_cast<const uint4*>(sOw + row * (D + 8) + 8 * cv);
+        }
+      }
+    }
+#pragma unroll
+    for (int v = 0; v < 4; ++v) { m[v] = -1.0e30f; ls[v] = 0.f; }
+#pragma unroll
+    for (int n = 0; n < ND; ++n) o[n] = (f32x4){0, 0, 0, 0};
+  };
   auto fwd_tile = [&] __device__ (int kt, const char* base, auto masked_c) {
     constexpr bool MASKED = decltype(masked_c)::value;
     const float* stats = reinterpret_cast<const float*>(base + TILES + w * 1024);
@@ -358,6 +462,9 @@ __global__ void __launch_bounds__(64 * NW) k_fwd_fused2(const T* __restrict__ Qp
         for (int n = 0; n < ND; ++n) mma16(o[n], pa, ld8(sV + TT::at(n, col, 0, g)));
       }
     }
+    if constexpr (CHUNKED) {
+      if ((64 * kt) % co.c == 0) flush_chunk(64 * kt / co.c);
+    }
   };
   {
     // the key tiles visited first hold the diagonal blocks of the waves
@@ -370,7 +477,7 @@ __global__ void __launch_bounds__(64 * NW) k_fwd_fused2(const T* __restrict__ Qp
 #undef UA_COMPUTE_FAST
 #undef UA_COMPUTE_SLOW
   // epilogue
-  if (!live) return;
+  if (CHUNKED || !live) return;
 #pragma unroll
   for (int v = 0; v < 4; ++v) {
     const float tot = allsum16(ls[v]);

@@ -6,8 +6,7 @@
 
 namespace ua {
 
-// marker stored in the log2-unit normaliser buffer for a (query, chunk) pair with no visible key
-constexpr float kLseMasked = 3.0e38f;
+constexpr float kLseMasked = kNoKeyLse;
 constexpr float kNegBig = -1.0e30f;
 
 // ---------------------------------------------------------------------------------------------

@@ -1,4 +1,6 @@
 // Instantiations and launchers of the forward kernels.
+#include <algorithm>
+#include <cstdint>
 #include "ua_fused.hpp"
 #include "ua_fwd.hpp"
 #include "ua_internal.hpp"
@@ -32,20 +34,22 @@ hipError_t launch_carry(int dtype, int D, const void* Kp, const float* lsrc, con
 }
 
 // explicit instantiations (the implicit ones are not emitted on the host side for these kernels)
-#define UA_INST(T, D, NST, NW)                                                                                        \
-  template __global__ void k_fwd_fused2<T, D, NST, NW>(const T*, const T*, const T*, const float*, const float*,      \
-                                                       const float*, T*, float*, float*, const int*, const int*, int, int, int, int);
-UA_INST(bf16, 64, 1, 8) UA_INST(bf16, 64, 2, 8) UA_INST(bf16, 64, 2, 12) UA_INST(bf16, 64, 2, 16)
-UA_INST(bf16, 128, 1, 8) UA_INST(bf16, 128, 2, 8) UA_INST(bf16, 128, 2, 12) UA_INST(bf16, 128, 2, 16)
-UA_INST(float, 64, 1, 8) UA_INST(float, 128, 1, 8)
+#define UA_INST(T, D, NST, NW, CH)                                                                                    \
+  template __global__ void k_fwd_fused2<T, D, NST, NW, CH>(const T*, const T*, const T*, const float*, const float*,  \
+                                                           const float*, T*, float*, float*, const int*, const int*, \
+                                                           int, int, int, int, ChunkOut<T>);
+UA_INST(bf16, 64, 1, 8, false) UA_INST(bf16, 64, 2, 8, false) UA_INST(bf16, 64, 2, 12, false) UA_INST(bf16, 64, 2, 16, false)
+UA_INST(bf16, 128, 1, 8, false) UA_INST(bf16, 128, 2, 8, false) UA_INST(bf16, 128, 2, 12, false) UA_INST(bf16, 128, 2, 16, false)
+UA_INST(float, 64, 1, 8, false) UA_INST(float, 128, 1, 8, false)
+UA_INST(bf16, 64, 2, 8, true) UA_INST(bf16, 128, 2, 8, true) UA_INST(float, 64, 1, 8, true) UA_INST(float, 128, 1, 8, true)
 #undef UA_INST
 
 template <class T, int D, int NST, int NW>
 static hipError_t fused_t(const void* Qp, const void* Kp, const void* VT, const float* lsrc, const float* ldest,
                           const float* C, void* O, float* lse, float* lse2, const int* reach, const int* minkey, int R, int L,
                           int Lp, int d, int Zq, hipStream_t s) {
-  hipLaunchKernelGGL((k_fwd_fused2<T, D, NST, NW>), dim3((Lp / 16 + NW - 1) / NW, Zq), dim3(64 * NW), 0, s, (const T*)Qp,
-                     (const T*)Kp, (const T*)VT, lsrc, ldest, C, (T*)O, lse, lse2, reach, minkey, R, L, Lp, d);
+  hipLaunchKernelGGL((k_fwd_fused2<T, D, NST, NW, false>), dim3((Lp / 16 + NW - 1) / NW, Zq), dim3(64 * NW), 0, s, (const T*)Qp,
+                     (const T*)Kp, (const T*)VT, lsrc, ldest, C, (T*)O, lse, lse2, reach, minkey, R, L, Lp, d, ChunkOut<T>{});
   return hipGetLastError();
 }
 // variants (bf16): 0 = 8 waves, double-buffered stages; 1 = 8 waves, single stage; 2 = 12 waves; 3 = 16 waves
@@ -70,6 +74,41 @@ hipError_t launch_fwd_fused(int dtype, int D, int variant, const void* Qp, const
 #define UA_ARGS Qp, Kp, VT, lsrc, ldest, C, O, lse, lse2, reach, minkey, R, L, Lp, d, Zq, s
   if (dtype == 1) return D == 64 ? fused_v<bf16, 64>(variant, UA_ARGS) : fused_v<bf16, 128>(variant, UA_ARGS);
   return D == 64 ? fused_t<float, 64, 1, 8>(UA_ARGS) : fused_t<float, 128, 1, 8>(UA_ARGS);
+#undef UA_ARGS
+}
+
+// chunked operator through the query-stationary kernel (chunk a multiple of 64; tiled working tensors)
+template <class T, int D>
+static hipError_t chunked2_t(const void* Qp, const void* Kp, const void* Vp, const void* VT, const float* lsrc, const float* ldest,
+                             const float* C, const int* reach, const int* minkey, void* out, void* denom, float* lse2, long o_sz,
+                             long o_st, long o_sd, long o_si, int R, int L, int Lp, int d, int c, int nch, int Zq, hipStream_t s) {
+  constexpr int NST = sizeof(T) == 2 ? 2 : 1, NW = 8;
+  constexpr long VV = 16 / (long)sizeof(T);
+  const int ovec = out && o_sd == 1 && d % VV == 0 && (uintptr_t)out % 16 == 0 && o_sz % VV == 0 && o_st % VV == 0 && o_si % VV == 0;
+  ChunkOut<T> co{(T*)out, (T*)denom, o_sz, o_st, o_sd, o_si, c, nch, ovec};
+  hipLaunchKernelGGL((k_fwd_fused2<T, D, NST, NW, true>), dim3((Lp / 16 + NW - 1) / NW, Zq), dim3(64 * NW), 0, s, (const T*)Qp,
+                     (const T*)Kp, (const T*)VT, lsrc, ldest, C, (T*)nullptr, (float*)nullptr, lse2, reach, minkey, R, L, Lp, d, co);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  if (out && nch > 1) {
+    const int vec = ovec;
+    const int slabs = (std::min((nch - 1) * c, L) + 255) / 256;
+    hipLaunchKernelGGL((k_chunk_masked_out<T, D>), dim3(slabs, nch, Zq), dim3(256), 0, s, (const T*)Vp, co, R, L, Lp, d, vec);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+  }
+  if (nch > 1) {
+    hipLaunchKernelGGL((k_chunk_masked_denom<T>), dim3((Lp + 255) / 256, Zq), dim3(256), 0, s, (T*)denom, lse2, L, Lp, c, nch);
+    e = hipGetLastError();
+  }
+  return e;
+}
+hipError_t launch_fwd_chunked2(int dtype, int D, const void* Qp, const void* Kp, const void* Vp, const void* VT, const float* lsrc,
+                               const float* ldest, const float* C, const int* reach, const int* minkey, void* out, void* denom,
+                               float* lse2, long o_sz, long o_st, long o_sd, long o_si, int R, int L, int Lp, int d, int c, int nch,
+                               int Zq, hipStream_t s) {
+#define UA_ARGS Qp, Kp, Vp, VT, lsrc, ldest, C, reach, minkey, out, denom, lse2, o_sz, o_st, o_sd, o_si, R, L, Lp, d, c, nch, Zq, s
+  if (dtype == 1) return D == 64 ? chunked2_t<bf16, 64>(UA_ARGS) : chunked2_t<bf16, 128>(UA_ARGS);
+  return D == 64 ? chunked2_t<float, 64>(UA_ARGS) : chunked2_t<float, 128>(UA_ARGS);
 #undef UA_ARGS
 }
 

@@ -28,6 +28,12 @@ hipError_t launch_fwd_fused(int dtype, int D, int variant, const void* Qp, const
 hipError_t launch_fwd_chunked(int dtype, int D, const void* Qp, const void* Kp, const void* VT, const float* lsrc,
                               const float* ldest, void* out, void* denom, float* lse2, long o_sz, long o_st, long o_sd,
                               long o_si, int R, int L, int Lp, int d, int c, int nch, int Zk, hipStream_t s);
+// chunk a multiple of 64: the chunked operator through the query-stationary kernel (tiled working tensors, carries
+// C and reach / minkey from launch_carry); also fills the results of the queries that precede a chunk
+hipError_t launch_fwd_chunked2(int dtype, int D, const void* Qp, const void* Kp, const void* Vp, const void* VT, const float* lsrc,
+                               const float* ldest, const float* C, const int* reach, const int* minkey, void* out, void* denom,
+                               float* lse2, long o_sz, long o_st, long o_sd, long o_si, int R, int L, int Lp, int d, int c, int nch,
+                               int Zq, hipStream_t s);
 // cols != 0: the kernel also produces dQ / dkcol through atomics (chunked mode); cols == 0: it records the
 // suffix carries and launch_bwd_queries finishes the query side.
 hipError_t launch_bwd_keys(int dtype, int D, const BwdArgsV& a, int Zk, int cols, hipStream_t s);

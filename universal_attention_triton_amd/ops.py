@@ -42,11 +42,15 @@ def _rows_q(t):
 
 
 def _chunked(t):
-    """[b,h,r,l,d,n] tensor whose leading three dims are mergeable into one index"""
-    b, h, r = t.shape[:3]
-    if not (t.stride(0) == h * t.stride(1) and t.stride(1) == r * t.stride(2)):
+    """[b,h,r,l,d,n] tensor -> (tensor kept alive, descriptor); the three leading dims must merge into one index,
+    which `view` decides (it ignores the strides of size-1 dims); otherwise the tensor is copied."""
+    L, d, n = t.shape[-3:]
+    try:
+        v = t.view(-1, L, d, n)
+    except RuntimeError:
         t = t.contiguous()
-    return t, UaChunked(t.data_ptr(), t.stride(2), t.stride(3), t.stride(4), t.stride(5))
+        v = t.view(-1, L, d, n)
+    return t, UaChunked(v.data_ptr(), v.stride(0), v.stride(1), v.stride(2), v.stride(3))
 
 
 def _desc(kc, xq, chunked, flags=0):
@@ -171,7 +175,13 @@ def fused_backward(kc, vc, xq, static_src, static_dest, O, lse, dO, ws=None, pru
 def _merge_views(mat):
     """mat [..., L, d, n] -> 4-D view [Z, L, d, n] whose Z stride is uniform"""
     L, d, n = mat.shape[-3:]
-    m4 = mat.reshape(-1, L, d, n) if mat.dim() != 4 else mat
+    if mat.dim() == 4:
+        m4 = mat
+    else:
+        try:
+            m4 = mat.view(-1, L, d, n)
+        except RuntimeError:
+            m4 = mat.reshape(-1, L, d, n)
     return m4, UaChunked(m4.data_ptr(), m4.stride(0), m4.stride(1), m4.stride(2), m4.stride(3))
 
 
