@@ -24,6 +24,7 @@ namespace ua {
 template <class T>
 struct BwdArgs {
   const int *reach, *minkey;    // pruning state of the fused mode: [Zk][Lp/16], [Zk][Lp/32]
+  const int* masked_nz;         // chunked mode: non-zero when an upstream gradient of a (query, later chunk) pair is non-zero
   const T *Kp, *Vp;             // [Zk][Lp][D]
   const T *KT;                  // [Zk][D][Lp]
   const float *lsrc, *ldest;    // [Zk][Lp]  log2(gate)/3

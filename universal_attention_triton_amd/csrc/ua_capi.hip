@@ -36,7 +36,7 @@ struct Layout {
   // forward state
   size_t Kp, KT, Vp, VT, Qp, QT, lsrc, ldest, C, lse2, knorm2, qnorm2, reach, minkey, fwd_end;
   // backward scratch
-  size_t dOp, dOT, delta, dQacc, dKdacc, Dsuf, dKrow, dVrow, dsrc_raw, total;
+  size_t dOp, dOT, delta, dQacc, dKdacc, Dsuf, dKrow, dVrow, dsrc_raw, masked_nz, total;
 };
 
 int check_desc(const ua_desc* d, bool chunked) {
@@ -78,9 +78,13 @@ Layout make_layout(const ua_desc& d, bool chunked) {
   const size_t gbytes = (size_t)l.Zq * l.nch * l.Lp * l.D * l.esz;
   l.dOp = take(gbytes); l.dOT = take(gbytes);
   l.delta = take((size_t)l.Zq * l.nch * l.Lp * 4);
-  l.dQacc = chunked ? take((size_t)l.Zq * l.Lp * l.D * 4) : 0;     // atomics target of the chunked mode only
+  // the key-chunk-stationary backward (chunk not a multiple of 64) adds up dQ through atomics; the other paths keep
+  // suffix carries instead
+  const bool atomics = chunked && d.chunk % 64 != 0;
+  l.dQacc = atomics ? take((size_t)l.Zq * l.Lp * l.D * 4) : 0;
   l.dKdacc = take((size_t)l.Zk * l.Lp * l.D * 4);
-  l.Dsuf = chunked ? 0 : take((size_t)l.Zk * l.nT * l.Lp * 4);
+  l.Dsuf = atomics ? 0 : take((size_t)l.Zk * l.nT * l.Lp * 4);
+  l.masked_nz = take(256);
   l.dKrow = take((size_t)l.Zk * l.Lp * l.D * 4);
   l.dVrow = take((size_t)l.Zk * l.Lp * l.D * 4);
   l.dsrc_raw = take((size_t)l.Zk * l.Lp * 4);
@@ -121,18 +125,19 @@ bool vector_ok(const ua::RowsView& v, size_t esz, int d) {
 }
 template <class T>
 hipError_t pack_t(int D, const ua::RowsView& x, void* nat, void* tr, int d, int L, int Lp, int Z, int tr_mode, float* norm2,
-                  hipStream_t s) {
+                  hipStream_t s, const int* masked_nz, int c) {
   const int tiled = tr_mode != TR_PERM16;      // the fused kernels read tiled working tensors, the chunked ones row-major
   const int vec = vector_ok(x, sizeof(T), d) ? 1 : 0;
-  if (D == 64) hipLaunchKernelGGL((ua::k_pack<T, 64>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp, tr_mode, tiled, vec, norm2);
-  else hipLaunchKernelGGL((ua::k_pack<T, 128>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp, tr_mode, tiled, vec, norm2);
+  if (D == 64) hipLaunchKernelGGL((ua::k_pack<T, 64>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp, tr_mode, tiled, vec, norm2, masked_nz, c);
+  else hipLaunchKernelGGL((ua::k_pack<T, 128>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp, tr_mode, tiled, vec, norm2, masked_nz, c);
   return hipGetLastError();
 }
 // norm2 (optional): [Z][Lp/32] receives the largest squared row norm of every block of 32 rows
+// masked_nz, c (optional, chunked upstream gradient): see k_pack
 hipError_t pack(int dtype, int D, const ua::RowsView& x, void* nat, void* tr, int d, int L, int Lp, int Z, int tr_mode, hipStream_t s,
-                float* norm2 = nullptr) {
-  return dtype == UA_BF16 ? pack_t<ua::bf16>(D, x, nat, tr, d, L, Lp, Z, tr_mode, norm2, s)
-                          : pack_t<float>(D, x, nat, tr, d, L, Lp, Z, tr_mode, norm2, s);
+                float* norm2 = nullptr, const int* masked_nz = nullptr, int c = 0) {
+  return dtype == UA_BF16 ? pack_t<ua::bf16>(D, x, nat, tr, d, L, Lp, Z, tr_mode, norm2, s, masked_nz, c)
+                          : pack_t<float>(D, x, nat, tr, d, L, Lp, Z, tr_mode, norm2, s, masked_nz, c);
 }
 
 // ---- optional per-kernel timing (hipEvents on the launch stream) ---------------------------
@@ -253,14 +258,18 @@ hipError_t finish_t(const Layout& l, const ua_desc& d, char* ws, bool chunked, c
 
 template <class T>
 hipError_t delta_t(const ua::RowsView& O, const ua::RowsView& dO, const ua::RowsView& sub, const ua::RowsView& lse_in,
-                   float* delta, float* lse2, int d, int L, int Lp, int Z, hipStream_t s) {
+                   float* delta, float* lse2, int d, int L, int Lp, int Z, hipStream_t s, int* masked_nz = nullptr, int c = 0) {
   const int vec = vector_ok(O, sizeof(T), d) && vector_ok(dO, sizeof(T), d) ? 1 : 0;
-  hipLaunchKernelGGL((ua::k_delta<T>), dim3(Lp / 16, Z), dim3(256), 0, s, O, dO, sub, lse_in, delta, lse2, d, L, Lp, vec);
+  hipLaunchKernelGGL((ua::k_delta<T>), dim3(Lp / 128, Z), dim3(256), 0, s, O, dO, sub, lse_in, delta, lse2, d, L, Lp, vec, masked_nz, c);
   return hipGetLastError();
 }
 
+// chunked with a chunk that is not a multiple of 64: key-chunk-stationary kernel over row-major working tensors (atomics);
+// otherwise the key-stationary and query-stationary kernels over tiled working tensors
 int run_bwd_common(const ua_desc& d, const Layout& l, char* ws, bool chunked, const void* src, const void* dest, void* dkc,
                    void* dvc, void* dxq, void* dsrc, void* ddest, hipStream_t s) {
+  const bool is_chunked = chunked;
+  chunked = is_chunked && !fast_chunk(d);      // from here on: the atomics path
   if (chunked) {
     UA_PROF("k_zero", s);
     UA_HIP(zero_fill(ws + l.dQacc, (size_t)l.Zq * l.Lp * l.D * 4, s));
@@ -274,7 +283,8 @@ int run_bwd_common(const ua_desc& d, const Layout& l, char* ws, bool chunked, co
   a.dQacc = (float*)(ws + l.dQacc); a.dKdacc = (float*)(ws + l.dKdacc); a.Dsuf = (float*)(ws + l.Dsuf);
   a.dKrow = (float*)(ws + l.dKrow);
   a.dVrow = (float*)(ws + l.dVrow); a.dsrc_raw = (float*)(ws + l.dsrc_raw);
-  a.R = d.r; a.L = d.L; a.Lp = l.Lp; a.c = chunked ? d.chunk : 128; a.nch = l.nch; a.chunked = chunked ? 1 : 0;
+  a.masked_nz = (const int*)(ws + l.masked_nz);
+  a.R = d.r; a.L = d.L; a.Lp = l.Lp; a.c = is_chunked ? d.chunk : 128; a.nch = l.nch; a.chunked = is_chunked ? 1 : 0;
   a.skip_masked = (d.flags & UA_FLAG_SKIP_MASKED) ? 1 : 0;
   {
     UA_PROF("k_bwd_keys", s);
@@ -387,9 +397,35 @@ int ua_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
   char* w = (char*)ws;
   hipStream_t s = (hipStream_t)stream;
   const ua_desc& d = *desc;
-  if (ws_has_fwd && fast_chunk(d)) {
-    // the forward left tiled working tensors; the key-chunk-stationary backward reads row-major ones
-    if (int e = pack_inputs(d, l, true, kc, vc, xq, static_src, static_dest, w, s)) return e;
+  const ua::RowsView outv = chunked_view(*out, l.nch);
+  ua_chunked gmut = *g_out;
+  const ua::RowsView gv = chunked_view(gmut, l.nch), none = null_view();
+  // g_denom [zq][t][i] seen per z = zq*nch + i
+  ua::RowsView gdv;
+  gdv.p = g_denom; gdv.sb = (long)d.L * l.nch; gdv.sh = 0; gdv.sr = 0; gdv.sn = 1; gdv.so = 0; gdv.si = l.nch; gdv.sc = 1;
+  gdv.inner = 1 << 30; gdv.H = 1; gdv.R = 1; gdv.N = l.nch;
+  if (fast_chunk(d)) {
+    if (!ws_has_fwd) {
+      // recompute the carries and the per-chunk normalisers (the partial outputs themselves are passed in)
+      if (int e = pack_inputs(d, l, false, kc, vc, xq, static_src, static_dest, w, s)) return e;
+      UA_HIP(ua::launch_carry(d.dtype, l.D, w + l.Kp, (const float*)(w + l.lsrc), (const float*)(w + l.ldest), (float*)(w + l.C), l.Lp,
+                              l.Zk, 1, nullptr, nullptr, d.r, (int*)(w + l.reach), (int*)(w + l.minkey), s));
+      UA_HIP(ua::launch_fwd_chunked2(d.dtype, l.D, w + l.Qp, w + l.Kp, w + l.Vp, w + l.VT, (const float*)(w + l.lsrc),
+                                     (const float*)(w + l.ldest), (const float*)(w + l.C), (const int*)(w + l.reach),
+                                     (const int*)(w + l.minkey), nullptr, nullptr, (float*)(w + l.lse2), 0, 0, 0, 0, d.r, d.L, l.Lp,
+                                     d.d, d.chunk, l.nch, l.Zq, s));
+    }
+    {
+      UA_PROF("pack_dO+delta", s);
+      UA_HIP(zero_fill(w + l.masked_nz, 256, s));
+      // with UA_FLAG_SKIP_MASKED the flag stays 0: rows before their chunk are neither checked nor packed
+      int* nz = (int*)(w + l.masked_nz);
+      int* detect = (d.flags & UA_FLAG_SKIP_MASKED) ? nullptr : nz;
+      if (d.dtype == UA_BF16) UA_HIP(delta_t<ua::bf16>(outv, gv, gdv, none, (float*)(w + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s, detect, d.chunk));
+      else UA_HIP(delta_t<float>(outv, gv, gdv, none, (float*)(w + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s, detect, d.chunk));
+      UA_HIP(pack(d.dtype, l.D, gv, w + l.dOp, w + l.dOT, d.d, d.L, l.Lp, l.Zq * l.nch, TR_PERM32, s, nullptr, nz, d.chunk));
+    }
+    return run_bwd_common(d, l, w, true, static_src, static_dest, dkc, dvc, dxq, dsrc, ddest, s);
   }
   if (!ws_has_fwd) {
     // recompute the per-chunk normalisers (the partial outputs themselves are passed in)
@@ -399,17 +435,19 @@ int ua_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
   }
   UA_HIP(ua::launch_carry(d.dtype, l.D, w + l.Kp, (const float*)(w + l.lsrc), (const float*)(w + l.ldest),
                           (float*)(w + l.C), l.Lp, l.Zk, 0, nullptr, nullptr, 1, nullptr, nullptr, s));
-  const ua::RowsView outv = chunked_view(*out, l.nch);
-  ua_chunked gmut = *g_out;
-  const ua::RowsView gv = chunked_view(gmut, l.nch), none = null_view();
-  // g_denom [zq][t][i] seen per z = zq*nch + i
-  ua::RowsView gdv;
-  gdv.p = g_denom; gdv.sb = (long)d.L * l.nch; gdv.sh = 0; gdv.sr = 0; gdv.sn = 1; gdv.so = 0; gdv.si = l.nch; gdv.sc = 1;
-  gdv.inner = 1 << 30; gdv.H = 1; gdv.R = 1; gdv.N = l.nch;
   UA_HIP(pack(d.dtype, l.D, gv, w + l.dOp, w + l.dOT, d.d, d.L, l.Lp, l.Zq * l.nch, TR_PERM16, s));
   if (d.dtype == UA_BF16) UA_HIP(delta_t<ua::bf16>(outv, gv, gdv, none, (float*)(w + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s));
   else UA_HIP(delta_t<float>(outv, gv, gdv, none, (float*)(w + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s));
   return run_bwd_common(d, l, w, true, static_src, static_dest, dkc, dvc, dxq, dsrc, ddest, s);
+}
+
+// 16-byte accesses to every (row, chunk) slice of a chunked tensor, with d / V lanes per slice (a power of two <= 64)
+static bool merge_vector_ok(const ua_chunked& c, int dtype, int d) {
+  const long V = dtype == UA_BF16 ? 8 : 4;
+  if (c.stride_d != 1 || d % V != 0) return false;
+  const long lpr = d / V;
+  if (lpr > 64 || (lpr & (lpr - 1)) != 0) return false;
+  return (uintptr_t)c.ptr % 16 == 0 && c.stride_z % V == 0 && c.stride_t % V == 0 && c.stride_i % V == 0;
 }
 
 int ua_merge_fwd(int dtype, int64_t rows, int32_t L, int32_t d, int32_t n, const ua_chunked* mat, const void* vec,
@@ -421,8 +459,11 @@ int ua_merge_fwd(int dtype, int64_t rows, int32_t L, int32_t d, int32_t n, const
   const dim3 grid((unsigned)((rows + 3) / 4));
   const size_t lds = 4 * (size_t)n * sizeof(float);
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == UA_BF16) hipLaunchKernelGGL((ua::k_merge_fwd<ua::bf16>), grid, dim3(256), lds, s, m, (const ua::bf16*)vec, (ua::bf16*)result, (long)rows, L, d, n);
-  else hipLaunchKernelGGL((ua::k_merge_fwd<float>), grid, dim3(256), lds, s, m, (const float*)vec, (float*)result, (long)rows, L, d, n);
+  const bool vecp = merge_vector_ok(*mat, dtype, d) && (uintptr_t)result % 16 == 0;
+#define UA_MERGE_FWD(T, VEC) hipLaunchKernelGGL((ua::k_merge_fwd<T, VEC>), grid, dim3(256), lds, s, m, (const T*)vec, (T*)result, (long)rows, L, d, n)
+  if (dtype == UA_BF16) { if (vecp) UA_MERGE_FWD(ua::bf16, true); else UA_MERGE_FWD(ua::bf16, false); }
+  else { if (vecp) UA_MERGE_FWD(float, true); else UA_MERGE_FWD(float, false); }
+#undef UA_MERGE_FWD
   UA_HIP(hipGetLastError());
   return UA_OK;
 }
@@ -437,8 +478,11 @@ int ua_merge_bwd(int dtype, int64_t rows, int32_t L, int32_t d, int32_t n, const
   const dim3 grid((unsigned)((rows + 3) / 4));
   const size_t lds = 8 * (size_t)n * sizeof(float);
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == UA_BF16) hipLaunchKernelGGL((ua::k_merge_bwd<ua::bf16>), grid, dim3(256), lds, s, m, (const ua::bf16*)vec, (const ua::bf16*)g, dm, (ua::bf16*)d_vec, (long)rows, L, d, n);
-  else hipLaunchKernelGGL((ua::k_merge_bwd<float>), grid, dim3(256), lds, s, m, (const float*)vec, (const float*)g, dm, (float*)d_vec, (long)rows, L, d, n);
+  const bool vecp = merge_vector_ok(*mat, dtype, d) && merge_vector_ok(*d_mat, dtype, d) && (uintptr_t)g % 16 == 0;
+#define UA_MERGE_BWD(T, VEC) hipLaunchKernelGGL((ua::k_merge_bwd<T, VEC>), grid, dim3(256), lds, s, m, (const T*)vec, (const T*)g, dm, (T*)d_vec, (long)rows, L, d, n)
+  if (dtype == UA_BF16) { if (vecp) UA_MERGE_BWD(ua::bf16, true); else UA_MERGE_BWD(ua::bf16, false); }
+  else { if (vecp) UA_MERGE_BWD(float, true); else UA_MERGE_BWD(float, false); }
+#undef UA_MERGE_BWD
   UA_HIP(hipGetLastError());
   return UA_OK;
 }

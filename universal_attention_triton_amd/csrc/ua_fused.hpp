@@ -221,20 +221,38 @@ template <class T> struct ChunkOut {
 
 // Queries that precede a whole chunk see none of its keys; the reference's softmax over a row of equal fill values
 // is uniform there: out = mean of the chunk's values (through a dtype-rounded 1/c), denom = float32(-1e12).
-// grid (ceil(max rows / 256), nch, Zq), 256 threads: slab x of chunk i writes rows [256 x, 256 x + 256) ∩ [0, i*c) of
-// out[.., i].  vec: rows of out[.., i] are contiguous in dd, 16-byte aligned and d is a multiple of the vector.
+// grid (ceil(max rows / kMaskedSlab), nch, Zq), 256 threads: slab x of chunk i writes rows [x kMaskedSlab, (x + 1) kMaskedSlab)
+// ∩ [0, i*c) of out[.., i].  vec: rows of out[.., i] are contiguous in dd, 16-byte aligned and d is a multiple of the vector.
+constexpr int kMaskedSlab = 1024;
 template <class T, int D>
 __global__ void __launch_bounds__(256) k_chunk_masked_out(const T* __restrict__ Vp, ChunkOut<T> co, int R, int L, int Lp, int d,
                                                           int vec) {
-  constexpr int V = 16 / (int)sizeof(T);
+  constexpr int V = 16 / (int)sizeof(T), NKG = D / 8, NRG = 256 / NKG;
   __shared__ __attribute__((aligned(16))) T mean[D];
+  __shared__ float part[NRG][D];
   const int i = blockIdx.y, zq = blockIdx.z, zk = zq / R, tid = threadIdx.x;
-  const int rows = min(i * co.c, L), r0 = blockIdx.x * 256, r1 = min(rows, r0 + 256);
+  const int rows = min(i * co.c, L), r0 = blockIdx.x * kMaskedSlab, r1 = min(rows, r0 + kMaskedSlab);
   if (r0 >= rows) return;
   const float pu = (float)cvt<T>(1.0f / (float)co.c);
+  {
+    // thread (k-group kg, row group rg) adds up the 8-element cells of rows rg, rg + NRG, ... of the chunk
+    const int kg = tid % NKG, rg = tid / NKG;
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+    for (int s = rg; s < co.c; s += NRG) {
+      const Frag<T> x = ld8(Vp + nat_off<D>(zk, Lp, i * co.c + s, 8 * kg));
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += pu * (float)x.v[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) part[rg][8 * kg + e] = acc[e];
+  }
+  __syncthreads();
   for (int dd = tid; dd < D; dd += 256) {
     float acc = 0.f;
-    for (int s = 0; s < co.c; ++s) acc += pu * (float)Vp[nat_off<D>(zk, Lp, i * co.c + s, dd)];
+#pragma unroll
+    for (int rg = 0; rg < NRG; ++rg) acc += part[rg][dd];
     mean[dd] = cvt<T>(acc);
   }
   __syncthreads();
@@ -503,13 +521,17 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW
 // sweeps the 32-query blocks from the last one down to its own; one (query block, query group) per step.
 // MR = more than one query group per kv head (the decay state of a query block then lives across steps).
 // ---------------------------------------------------------------------------------------------
-template <class T, int D, int NST, bool MR>
+// CH: chunked operator (a.c a multiple of 64): the upstream gradient, delta and the normaliser depend on the key's chunk
+// (z index zq*nch + chunk); the 128 keys of a workgroup lie in at most two chunks, whose dO tiles are both staged.
+template <class T, int D, int NST, bool MR, bool CH>
 __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   using TN = Tile<T, 32, D>;
   using TT = Tile<T, D, 32>;
   constexpr int NK = D / 32, ND = D / 16;
-  constexpr int TILES = 3 * TN::BYTES + 3 * TT::BYTES, SB = TILES + 1024;
+  constexpr int TILES = (CH ? 4 : 3) * (TN::BYTES + TT::BYTES), SB = TILES + (CH ? 2048 : 1024);
+  // tiles of a stage: Kt, Q, dO | KT, QT, dOT | (CH) dO, dOT of the workgroup's second chunk
   // stats row of a stage: [lse2: 32f][delta: 32f][ldest: 32f][unused: 32f][forward carries of the 128 keys: 128f]
+  // (CH) followed by [lse2: 32f][delta: 32f] of the second chunk
   UA_STAGES(SB);
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
   int bx, zk;
@@ -518,6 +540,16 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   const int kg = bx, sb16 = 8 * kg + w, spos = 16 * sb16 + col;      // key group 0 sweeps the most query blocks: first
   const int nTr = (L + 31) / 32, first = 4 * kg;
   if (first >= nTr) return;                      // every key of this workgroup is padding
+  // chunked operator: chunk of the workgroup's first key, whether the workgroup reaches into the next one, and which
+  // of the two this wave's keys belong to
+  const int nch = CH ? a.nch : 1;
+  const int ch0 = CH ? min((128 * kg) / a.c, nch - 1) : 0;
+  const bool two = CH && min((128 * kg + 127) / a.c, nch - 1) != ch0;
+  const int csel = CH ? min((16 * sb16) / a.c, nch - 1) - ch0 : 0;
+  const int cstart32 = CH ? ((ch0 + csel) * a.c) >> 5 : 0;      // first query block of this wave's chunk
+  const float inv_c = CH ? 1.0f / (float)a.c : 0.f;
+  // the blocks before the chunk are swept only when some upstream gradient there is non-zero (flag set by k_delta)
+  const bool uniform_part = CH && !a.skip_masked && *a.masked_nz != 0;
   // query blocks beyond the reach of a key tile (see k_carry2) are not visited: the sweep starts at the farthest
   // block any of the 8 waves reaches, and a wave joins in at its own
   const int* reach_z = a.reach + zk * nT16 + 8 * kg;
@@ -558,19 +590,29 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
     const int tb_ = top - (s) / R;                                                          \
     const long zq_ = (long)zk * R + (s) % R;                                                \
     const long qo_ = (zq_ * Lp + 32 * tb_) * D;   /* tile base, natural and transposed */      \
+    const long zg_ = zq_ * nch + ch0;             /* z index of dO, delta, lse2 */             \
+    const long go_ = (zg_ * Lp + 32 * tb_) * D;                                             \
     stN.issue((base), Kz + (long)(32 * tb_) * D, w);                                        \
     stN.issue((base) + TN::BYTES, a.Qp + qo_, w);                                           \
-    stN.issue((base) + 2 * TN::BYTES, a.dOp + qo_, w);                                      \
+    stN.issue((base) + 2 * TN::BYTES, a.dOp + go_, w);                                      \
     stT.issue((base) + 3 * TN::BYTES, KTz + (long)(32 * tb_) * D, w);                       \
     stT.issue((base) + 3 * TN::BYTES + TT::BYTES, a.QT + qo_, w);                           \
-    stT.issue((base) + 3 * TN::BYTES + 2 * TT::BYTES, a.dOT + qo_, w);                      \
+    stT.issue((base) + 3 * TN::BYTES + 2 * TT::BYTES, a.dOT + go_, w);                      \
     if (w == 0) {                                                                           \
       const float* src_;                                                                    \
-      if (lane < 8) src_ = a.lse2 + zq_ * Lp + 32 * tb_ + 4 * lane;                         \
-      else if (lane < 16) src_ = a.delta + zq_ * Lp + 32 * tb_ + 4 * (lane - 8);            \
+      if (lane < 8) src_ = a.lse2 + zg_ * Lp + 32 * tb_ + 4 * lane;                         \
+      else if (lane < 16) src_ = a.delta + zg_ * Lp + 32 * tb_ + 4 * (lane - 8);            \
       else if (lane < 32) src_ = ldz + 32 * tb_ + 4 * (lane & 7);                           \
       else src_ = Cz + (long)(2 * tb_) * Lp + 4 * (lane - 32);                              \
       issue_row((base) + TILES, src_);                                                      \
+    }                                                                                       \
+    if (CH && two) {                                                                        \
+      stN.issue((base) + 3 * TN::BYTES + 3 * TT::BYTES, a.dOp + go_ + (long)Lp * D, w);     \
+      stT.issue((base) + 4 * TN::BYTES + 3 * TT::BYTES, a.dOT + go_ + (long)Lp * D, w);     \
+      if (w == 1) {                                                                         \
+        const float* src_ = ((lane & 8) ? a.delta : a.lse2) + (zg_ + 1) * Lp + 32 * tb_ + 4 * (lane & 7); \
+        issue_row((base) + TILES + 1024, src_);                                             \
+      }                                                                                     \
     }                                                                                       \
   }
 #define UA_COMPUTE_FAST(s, base)                                                            \
@@ -580,19 +622,49 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
 #define UA_COMPUTE_SLOW(s, base)                                                            \
   {                                                                                         \
     const int tb_ = top - (s) / R;                                                          \
-    if (tb_ >= (sb16 >> 1) && tb_ <= myreach) bwd_step((s), (base), TrueC(), tb_ == (sb16 >> 1)); \
+    if (tb_ >= (sb16 >> 1)) {                                                               \
+      if (tb_ <= myreach) bwd_step((s), (base), TrueC(), tb_ == (sb16 >> 1));               \
+    } else if (CH && tb_ < cstart32) {                                                      \
+      uniform_step((s), (base));                                                            \
+    }                                                                                       \
   }
+  // Chunked operator, query block entirely before this wave's chunk: the reference fills the bias of such a
+  // (key, query) pair with -1e12, which swamps the score, so the softmax over the chunk's keys is uniform
+  // (universal_attention_autograd.py:27-33) while the gradient still flows through the score:
+  //   P = 1/c,  dS = (dP - delta) / c,  no decay part.
+  auto uniform_step = [&] __device__ (int s, const char* base) __attribute__((always_inline)) {
+    const T* sdO = reinterpret_cast<const T*>(base + (csel ? 3 * TN::BYTES + 3 * TT::BYTES : 2 * TN::BYTES));
+    const T* sQT = reinterpret_cast<const T*>(base + 3 * TN::BYTES + TT::BYTES);
+    const T* sdOT = reinterpret_cast<const T*>(base + (csel ? 4 * TN::BYTES + 3 * TT::BYTES : 3 * TN::BYTES + 2 * TT::BYTES));
+    const float* qstats = reinterpret_cast<const float*>(base + TILES) + (csel ? 256 : 0);
+    f32x4 P[2], dS[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      f32x4 dP = {0, 0, 0, 0};
+#pragma unroll
+      for (int q = 0; q < NK; ++q) mma16(dP, ld8(sdO + TN::at(i, col, q, g)), vf[q]);
+      const f32x4 dlt = load_t4(qstats + 32 + 16 * i, g);
+#pragma unroll
+      for (int v = 0; v < 4; ++v) { P[i][v] = inv_c; dS[i][v] = inv_c * (dP[v] - dlt[v]); }
+    }
+    const Frag<T> bp = as_operand16<T>(P[0], P[1]), bs = as_operand16<T>(dS[0], dS[1]);
+#pragma unroll
+    for (int n = 0; n < ND; ++n) mma16(dVt[n], ld8(sdOT + TT::at(n, col, 0, g)), bp);
+#pragma unroll
+    for (int n = 0; n < ND; ++n) mma16(dKt[n], ld8(sQT + TT::at(n, col, 0, g)), bs);
+  };
   // MASKED: the step may be the query block that holds this wave's own keys (run-time flag diag)
   auto bwd_step = [&] __device__ (int s, const char* base, auto masked_c, const bool diag) {
     constexpr bool MASKED = decltype(masked_c)::value;
     const int tb = top - s / R, r = s % R;
     const T* sKt = reinterpret_cast<const T*>(base);
     const T* sQ = reinterpret_cast<const T*>(base + TN::BYTES);
-    const T* sdO = reinterpret_cast<const T*>(base + 2 * TN::BYTES);
+    const T* sdO = reinterpret_cast<const T*>(base + (csel ? 3 * TN::BYTES + 3 * TT::BYTES : 2 * TN::BYTES));
     const T* sKT = reinterpret_cast<const T*>(base + 3 * TN::BYTES);
     const T* sQT = reinterpret_cast<const T*>(base + 3 * TN::BYTES + TT::BYTES);
-    const T* sdOT = reinterpret_cast<const T*>(base + 3 * TN::BYTES + 2 * TT::BYTES);
+    const T* sdOT = reinterpret_cast<const T*>(base + (csel ? 4 * TN::BYTES + 3 * TT::BYTES : 3 * TN::BYTES + 2 * TT::BYTES));
     const float* stats = reinterpret_cast<const float*>(base + TILES);
+    const float* qstats = stats + (csel ? 256 : 0);       // lse2 / delta of this wave's chunk
     f32x4 aff_l[2], bias_l[2], gk_l[2], dB_l[2];
     f32x4 (&aff)[2] = MR ? aff_s : aff_l;
     f32x4 (&bias)[2] = MR ? bias_s : bias_l;
@@ -630,7 +702,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
         for (int q = 0; q < NK; ++q) mma16(sc, ld8(sQ + TN::at(i, col, q, g)), kp[q]);
 #pragma unroll
         for (int q = 0; q < NK; ++q) mma16(dP, ld8(sdO + TN::at(i, col, q, g)), vf[q]);
-        const f32x4 l2t = load_t4(stats + 16 * i, g), dlt = load_t4(stats + 32 + 16 * i, g);
+        const f32x4 l2t = load_t4(qstats + 16 * i, g), dlt = load_t4(qstats + 32 + 16 * i, g);
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
           float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[v], kLog2e, bias[i][v]) - l2t[v]);
@@ -674,7 +746,8 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   };
   {
     // the last four query blocks of the sweep hold the diagonal blocks of the eight waves
-    const int nblk = top + 1 - first, total = nblk * R, nfast = ((nblk > 4 ? nblk - 4 : 0) * R) & ~1;
+    const int nblk = top + 1 - first, nfast = ((nblk > 4 ? nblk - 4 : 0) * R) & ~1;
+    const int total = (uniform_part ? top + 1 : nblk) * R;
     UA_PIPE_START(total, UA_ISSUE);
     UA_PIPE_RANGE(0, nfast, total, UA_ISSUE, UA_COMPUTE_FAST);
     UA_PIPE_RANGE(nfast, total, total, UA_ISSUE, UA_COMPUTE_SLOW);
@@ -704,7 +777,9 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
 // repeated per group; dg is linear in dBias, so the groups' contributions to dkcol add up (the cross-tile
 // suffix carry is added in the first group only).
 // ---------------------------------------------------------------------------------------------
-template <class T, int D, int NST>
+// CH: chunked operator (a.c a multiple of 64): the upstream gradient, delta and the normaliser are those of the chunk
+// the step's 64 keys belong to (z index zq*nch + chunk) and are reloaded when the chunk changes.
+template <class T, int D, int NST, bool CH>
 __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restrict__ dq, int d) {
   using TN = Tile<T, 32, D>;
   using TT = Tile<T, D, 32>;
@@ -752,39 +827,84 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
   else { row_base = reinterpret_cast<const float*>(a.reach + zk * nT16); row_step = 4; }
   // column of key (16*(j&1) + col) inside its 32-key group of the transposed key tile
   const int pc0 = perm32(col), pc1 = perm32(16 + col);
+  // chunked operator: key tiles [uk0, uk1) belong to chunks after the workgroup's first query (uk0_w: after this
+  // wave's queries); they are swept only when some upstream gradient there is non-zero (flag set by k_delta)
+  const float inv_c = CH ? 1.0f / (float)a.c : 0.f;
+  const bool uniform_part = CH && !a.skip_masked && *a.masked_nz != 0;
+  const int uk0 = CH ? ((min((128 * jt) / a.c, a.nch - 1) + 1) * a.c) >> 6 : 0;
+  const int uk0_w = CH ? ((min((16 * tq) / a.c, a.nch - 1) + 1) * a.c) >> 6 : 0;
+  const int uk1 = uniform_part ? max(uk0, L >> 6) : uk0;
 
   for (int r = 0; r < R; ++r) {
     const long zq = (long)zk * R + r;
     Frag<T> qt[NK], gt[NK];
+    f32x4 l2t, dlt;
+    int cur_chunk = -1;
+    // upstream operands of chunk ch (chunked operator) or of the merged operator (ch = 0, nch = 1)
+    auto load_upstream = [&] __device__ (int ch) __attribute__((always_inline)) {
+      const long zg = CH ? zq * a.nch + ch : zq;
+#pragma unroll
+      for (int q = 0; q < NK; ++q) gt[q] = ld8(a.dOp + nat_off<D>(zg, Lp, 16 * tq + col, 32 * q + 8 * g));
+      l2t = load_t4(a.lse2 + zg * Lp + 16 * tq, g);
+      dlt = load_t4(a.delta + zg * Lp + 16 * tq, g);
+      cur_chunk = ch;
+    };
     {
 #pragma unroll
-      for (int q = 0; q < NK; ++q) {
-        const long ro = nat_off<D>(zq, Lp, 16 * tq + col, 32 * q + 8 * g);
-        qt[q] = ld8(a.Qp + ro);
-        gt[q] = ld8(a.dOp + ro);
-      }
+      for (int q = 0; q < NK; ++q) qt[q] = ld8(a.Qp + nat_off<D>(zq, Lp, 16 * tq + col, 32 * q + 8 * g));
     }
-    const f32x4 l2t = load_t4(a.lse2 + zq * Lp + 16 * tq, g), dlt = load_t4(a.delta + zq * Lp + 16 * tq, g);
+    if (!CH) load_upstream(0);
     f32x4 dQ[ND];
 #pragma unroll
     for (int n = 0; n < ND; ++n) dQ[n] = (f32x4){0, 0, 0, 0};
 
 #define UA_ISSUE(s, base)                                                                   \
   {                                                                                         \
-    const int k0_ = 64 * (s);                                                               \
+    const int k0_ = 64 * ((s) < n_kt ? (s) : (s) - n_kt + uk0);                             \
     stN.issue((base), Kz + (long)k0_ * D, w);                                               \
     stN.issue((base) + TN::BYTES, Kz + (long)(k0_ + 32) * D, w);                            \
     stN.issue((base) + 2 * TN::BYTES, Vz + (long)k0_ * D, w);                               \
     stN.issue((base) + 3 * TN::BYTES, Vz + (long)(k0_ + 32) * D, w);                        \
     stT.issue((base) + 4 * TN::BYTES, KTz + (long)k0_ * D, w);                              \
     stT.issue((base) + 4 * TN::BYTES + TT::BYTES, KTz + (long)(k0_ + 32) * D, w);           \
-    issue_row((base) + TILES + w * 1024, row_base + (long)(s) * row_step);                  \
+    issue_row((base) + TILES + w * 1024, row_base + (long)(k0_ >> 6) * row_step);           \
   }
 #define UA_COMPUTE_FAST(s, base) bq_step((s), (base), FalseC())
-#define UA_COMPUTE_SLOW(s, base) bq_step((s), (base), TrueC())
+#define UA_COMPUTE_SLOW(s, base)                                                            \
+  {                                                                                         \
+    if ((s) < n_kt) bq_step((s), (base), TrueC());                                          \
+    else if (CH && (s) - n_kt + uk0 >= uk0_w) uniform_step((s) - n_kt + uk0, (base));       \
+  }
+    // Chunked operator, key tile of a chunk after this wave's queries: uniform softmax over the chunk's keys,
+    // dS = (dP - delta) / c (see k_bwd_keys2), no decay part.
+    auto uniform_step = [&] __device__ (int kti, const char* base) __attribute__((always_inline)) {
+      const int ch = min((64 * kti) / a.c, a.nch - 1);
+      if (ch != cur_chunk) load_upstream(ch);
+#pragma unroll
+      for (int kq = 0; kq < 2; ++kq) {
+        const T* sV = reinterpret_cast<const T*>(base + (2 + kq) * TN::BYTES);
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj) {
+          f32x4 dP = {0, 0, 0, 0}, dS;
+#pragma unroll
+          for (int q = 0; q < NK; ++q) mma16(dP, gt[q], ld8(sV + TN::at(jj, col, q, g)));
+#pragma unroll
+          for (int v = 0; v < 4; ++v) dS[v] = inv_c * (dP[v] - dlt[v]);
+          ST::put(sX, jj ? pc1 : pc0, g, dS);
+        }
+        const T* sKT = reinterpret_cast<const T*>(base + 4 * TN::BYTES + kq * TT::BYTES);
+        const Frag<T> as = ST::get(sX, lane);
+#pragma unroll
+        for (int n = 0; n < ND; ++n) mma16(dQ[n], as, ld8(sKT + TT::at(n, col, 0, g)));
+      }
+    };
     auto bq_step = [&] __device__ (int kti, const char* base, auto masked_c) {
       constexpr bool MASKED = decltype(masked_c)::value;
       const float* stats = reinterpret_cast<const float*>(base + TILES + w * 1024);
+      if constexpr (CH) {
+        const int ch = min((64 * kti) / a.c, a.nch - 1);
+        if (ch != cur_chunk) load_upstream(ch);
+      }
       // the 64 keys of the step are handled as two halves of 32 (= one contraction step of the column products);
 #pragma unroll
       for (int kq = 0; kq < 2; ++kq) {
@@ -857,10 +977,10 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
     };
     {
       // the last two key tiles hold the diagonal blocks of the eight waves
-      const int nfast = max(n_kt - 2, kt_min);
-      UA_PIPE_START_AT(kt_min, n_kt, UA_ISSUE);
-      UA_PIPE_RANGE(kt_min, nfast, n_kt, UA_ISSUE, UA_COMPUTE_FAST);
-      UA_PIPE_RANGE(nfast, n_kt, n_kt, UA_ISSUE, UA_COMPUTE_SLOW);
+      const int nfast = max(n_kt - 2, kt_min), n_all = n_kt + uk1 - uk0;
+      UA_PIPE_START_AT(kt_min, n_all, UA_ISSUE);
+      UA_PIPE_RANGE(kt_min, nfast, n_all, UA_ISSUE, UA_COMPUTE_FAST);
+      UA_PIPE_RANGE(nfast, n_all, n_all, UA_ISSUE, UA_COMPUTE_SLOW);
     }
 #undef UA_ISSUE
 #undef UA_COMPUTE_FAST

@@ -8,7 +8,7 @@ namespace ua {
 template <class T>
 static BwdArgs<T> typed(const BwdArgsV& v) {
   BwdArgs<T> a;
-  a.reach = v.reach; a.minkey = v.minkey;
+  a.reach = v.reach; a.minkey = v.minkey; a.masked_nz = v.masked_nz;
   a.Kp = (const T*)v.Kp; a.Vp = (const T*)v.Vp; a.KT = (const T*)v.KT; a.Qp = (const T*)v.Qp; a.QT = (const T*)v.QT;
   a.dOp = (const T*)v.dOp; a.dOT = (const T*)v.dOT; a.lsrc = v.lsrc; a.ldest = v.ldest; a.lse2 = v.lse2; a.delta = v.delta;
   a.C = v.C;
@@ -28,20 +28,24 @@ static hipError_t bwd_t(const BwdArgsV& v, int Zk, hipStream_t s) {
   return hipGetLastError();
 }
 // explicit instantiations (the implicit ones are not emitted on the host side for kernels holding lambdas)
-#define UA_INST(T, D, NST) \
-  template __global__ void k_bwd_keys2<T, D, NST, false>(BwdArgs<T>); template __global__ void k_bwd_keys2<T, D, NST, true>(BwdArgs<T>);
+#define UA_INST(T, D, NST)                                                   \
+  template __global__ void k_bwd_keys2<T, D, NST, false, false>(BwdArgs<T>); \
+  template __global__ void k_bwd_keys2<T, D, NST, true, false>(BwdArgs<T>);  \
+  template __global__ void k_bwd_keys2<T, D, NST, false, true>(BwdArgs<T>);  \
+  template __global__ void k_bwd_keys2<T, D, NST, true, true>(BwdArgs<T>);
 UA_INST(bf16, 64, 2) UA_INST(bf16, 128, 2) UA_INST(float, 64, 1) UA_INST(float, 128, 1)
 #undef UA_INST
 
-template <class T, int D, int NST, bool MR>
+template <class T, int D, int NST, bool MR, bool CH>
 static hipError_t bwd2_mr(const BwdArgs<T>& a, int Lp, int Zk, hipStream_t s) {
-  hipLaunchKernelGGL((k_bwd_keys2<T, D, NST, MR>), dim3(Lp / 128, Zk), dim3(512), 0, s, a);
+  hipLaunchKernelGGL((k_bwd_keys2<T, D, NST, MR, CH>), dim3(Lp / 128, Zk), dim3(512), 0, s, a);
   return hipGetLastError();
 }
 template <class T, int D, int NST>
 static hipError_t bwd2_t(const BwdArgsV& v, int Zk, hipStream_t s) {
   const BwdArgs<T> a = typed<T>(v);
-  return v.R > 1 ? bwd2_mr<T, D, NST, true>(a, v.Lp, Zk, s) : bwd2_mr<T, D, NST, false>(a, v.Lp, Zk, s);
+  if (v.chunked) return v.R > 1 ? bwd2_mr<T, D, NST, true, true>(a, v.Lp, Zk, s) : bwd2_mr<T, D, NST, false, true>(a, v.Lp, Zk, s);
+  return v.R > 1 ? bwd2_mr<T, D, NST, true, false>(a, v.Lp, Zk, s) : bwd2_mr<T, D, NST, false, false>(a, v.Lp, Zk, s);
 }
 template <class T, int D>
 static hipError_t bwd_nw(const BwdArgsV& v, int Zk, int cols, hipStream_t s) {
@@ -56,14 +60,17 @@ hipError_t launch_bwd_keys(int dtype, int D, const BwdArgsV& a, int Zk, int cols
 }
 
 // explicit instantiations (the implicit ones are not emitted on the host side for this kernel)
-#define UA_INST(T, D, NST) template __global__ void k_bwd_queries2<T, D, NST>(BwdArgs<T>, T*, int);
+#define UA_INST(T, D, NST)                                                      \
+  template __global__ void k_bwd_queries2<T, D, NST, false>(BwdArgs<T>, T*, int); \
+  template __global__ void k_bwd_queries2<T, D, NST, true>(BwdArgs<T>, T*, int);
 UA_INST(bf16, 64, 2) UA_INST(bf16, 128, 2) UA_INST(float, 64, 1) UA_INST(float, 128, 1)
 #undef UA_INST
 
 template <class T, int D, int NST>
 static hipError_t bwdq_t(const BwdArgsV& v, void* dq, int d, int Zk, hipStream_t s) {
   const BwdArgs<T> a = typed<T>(v);
-  hipLaunchKernelGGL((k_bwd_queries2<T, D, NST>), dim3(v.Lp / 128, Zk), dim3(512), 0, s, a, (T*)dq, d);
+  if (v.chunked) hipLaunchKernelGGL((k_bwd_queries2<T, D, NST, true>), dim3(v.Lp / 128, Zk), dim3(512), 0, s, a, (T*)dq, d);
+  else hipLaunchKernelGGL((k_bwd_queries2<T, D, NST, false>), dim3(v.Lp / 128, Zk), dim3(512), 0, s, a, (T*)dq, d);
   return hipGetLastError();
 }
 hipError_t launch_bwd_queries(int dtype, int D, const BwdArgsV& a, void* dq, int d, int Zk, hipStream_t s) {

@@ -92,7 +92,7 @@ static hipError_t chunked2_t(const void* Qp, const void* Kp, const void* Vp, con
   if (e != hipSuccess) return e;
   if (out && nch > 1) {
     const int vec = ovec;
-    const int slabs = (std::min((nch - 1) * c, L) + 255) / 256;
+    const int slabs = (std::min((nch - 1) * c, L) + kMaskedSlab - 1) / kMaskedSlab;
     hipLaunchKernelGGL((k_chunk_masked_out<T, D>), dim3(slabs, nch, Zq), dim3(256), 0, s, (const T*)Vp, co, R, L, Lp, d, vec);
     if ((e = hipGetLastError()) != hipSuccess) return e;
   }

@@ -8,7 +8,7 @@ namespace ua {
 
 // type-erased argument block of k_bwd_keys (same field order as BwdArgs<T>)
 struct BwdArgsV {
-  const int *reach, *minkey;
+  const int *reach, *minkey, *masked_nz;
   const void *Kp, *Vp, *KT, *Qp, *QT, *dOp, *dOT;
   const float *lsrc, *ldest, *lse2, *delta, *C;
   float *dQacc, *dKdacc, *Dsuf, *dKrow, *dVrow, *dsrc_raw;
@@ -34,8 +34,9 @@ hipError_t launch_fwd_chunked2(int dtype, int D, const void* Qp, const void* Kp,
                                const float* ldest, const float* C, const int* reach, const int* minkey, void* out, void* denom,
                                float* lse2, long o_sz, long o_st, long o_sd, long o_si, int R, int L, int Lp, int d, int c, int nch,
                                int Zq, hipStream_t s);
-// cols != 0: the kernel also produces dQ / dkcol through atomics (chunked mode); cols == 0: it records the
-// suffix carries and launch_bwd_queries finishes the query side.
+// cols != 0: the kernel also produces dQ / dkcol through atomics (chunked mode, row-major working tensors);
+// cols == 0: it records the suffix carries and launch_bwd_queries finishes the query side (tiled working tensors;
+// with a.chunked set: the chunked operator for a chunk that is a multiple of 64).
 hipError_t launch_bwd_keys(int dtype, int D, const BwdArgsV& a, int Zk, int cols, hipStream_t s);
 hipError_t launch_bwd_queries(int dtype, int D, const BwdArgsV& a, void* dq, int d, int Zk, hipStream_t s);
 

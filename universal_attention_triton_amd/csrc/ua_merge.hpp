@@ -24,7 +24,10 @@ __device__ __forceinline__ void row_softmax(const T* __restrict__ vec, int n, fl
   for (int i = lane; i < n; i += 64) wts[i] *= inv;
 }
 
-template <class T>
+// VEC: unit feature stride, every (row, chunk) slice 16-byte aligned and d / V (V = elements per 16 bytes) a power of
+// two of at most 64 (host-checked): lpr = d / V lanes read one slice with 16-byte loads and the 64 / lpr lane groups
+// of a wave take chunks i = group, group + 64 / lpr, ...
+template <class T, bool VEC>
 __global__ void __launch_bounds__(256) k_merge_fwd(ChunkedView mat, const T* __restrict__ vec, T* __restrict__ res,
                                                    long rows, int L, int d, int n) {
   extern __shared__ __align__(16) char smem[];
@@ -35,6 +38,31 @@ __global__ void __launch_bounds__(256) k_merge_fwd(ChunkedView mat, const T* __r
   row_softmax(vec + row * n, n, wts, lane);
   __builtin_amdgcn_wave_barrier();
   const T* m = reinterpret_cast<const T*>(mat.p) + (row / L) * mat.sz + (row % L) * mat.st;
+  if constexpr (VEC) {
+    constexpr int V = 16 / (int)sizeof(T);
+    const int lpr = d / V, sub = lane & (lpr - 1), grp = lane / lpr, ng = 64 / lpr;
+    float acc[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) acc[e] = 0.f;
+    for (int i = grp; i < n; i += ng) {
+      T x[V];
+      *reinterpret_cast<uint4*>(x) = *reinterpret_cast<const uint4*>(m + sub * V + i * mat.si);
+      const float wi = wts[i];
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc[e] += wi * (float)x[e];
+    }
+    for (int k = lpr; k < 64; k <<= 1) {
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc[e] += __shfl_xor(acc[e], k, 64);
+    }
+    if (grp == 0) {
+      T y[V];
+#pragma unroll
+      for (int e = 0; e < V; ++e) y[e] = cvt<T>(acc[e]);
+      *reinterpret_cast<uint4*>(res + row * d + sub * V) = *reinterpret_cast<const uint4*>(y);
+    }
+    return;
+  }
   for (int dd = lane; dd < d; dd += 64) {
     float acc = 0.f;
     for (int i = 0; i < n; ++i) acc += wts[i] * (float)m[dd * mat.sd + i * mat.si];
@@ -42,7 +70,7 @@ __global__ void __launch_bounds__(256) k_merge_fwd(ChunkedView mat, const T* __r
   }
 }
 
-template <class T>
+template <class T, bool VEC>
 __global__ void __launch_bounds__(256) k_merge_bwd(ChunkedView mat, const T* __restrict__ vec, const T* __restrict__ g,
                                                    ChunkedView dmat, T* __restrict__ dvec, long rows, int L, int d, int n) {
   extern __shared__ __align__(16) char smem[];
@@ -56,6 +84,29 @@ __global__ void __launch_bounds__(256) k_merge_bwd(ChunkedView mat, const T* __r
   const T* m = reinterpret_cast<const T*>(mat.p) + (row / L) * mat.sz + (row % L) * mat.st;
   T* dm = reinterpret_cast<T*>(dmat.p) + (row / L) * dmat.sz + (row % L) * dmat.st;
   const T* gr = g + row * d;
+  if constexpr (VEC) {
+    constexpr int V = 16 / (int)sizeof(T);
+    const int lpr = d / V, sub = lane & (lpr - 1), grp = lane / lpr, ng = 64 / lpr;
+    T gx[V];
+    *reinterpret_cast<uint4*>(gx) = *reinterpret_cast<const uint4*>(gr + sub * V);
+    float gf[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) gf[e] = (float)gx[e];
+    for (int i0 = 0; i0 < n; i0 += ng) {          // uniform trip count: the shuffles below involve every lane
+      const int i = i0 + grp;
+      float acc = 0.f;
+      if (i < n) {
+        T x[V], y[V];
+        *reinterpret_cast<uint4*>(x) = *reinterpret_cast<const uint4*>(m + sub * V + i * mat.si);
+        const float wi = wts[i];
+#pragma unroll
+        for (int e = 0; e < V; ++e) { acc += gf[e] * (float)x[e]; y[e] = cvt<T>(gf[e] * wi); }
+        *reinterpret_cast<uint4*>(dm + sub * V + i * dmat.si) = *reinterpret_cast<const uint4*>(y);
+      }
+      for (int k = 1; k < lpr; k <<= 1) acc += __shfl_xor(acc, k, 64);
+      if (sub == 0 && i < n) dw[i] = acc;
+    }
+  } else {
   // d_mat[dd, i] = g[dd] * w[i]
   for (int dd = lane; dd < d; dd += 64) {
     const float gv = (float)gr[dd];
@@ -68,6 +119,7 @@ __global__ void __launch_bounds__(256) k_merge_bwd(ChunkedView mat, const T* __r
 #pragma unroll
     for (int k = 32; k >= 1; k >>= 1) acc += __shfl_xor(acc, k, 64);
     if (lane == 0) dw[i] = acc;
+  }
   }
   __builtin_amdgcn_wave_barrier();
   float dot = 0.f;

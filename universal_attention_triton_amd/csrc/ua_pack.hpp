@@ -20,18 +20,34 @@ __device__ __forceinline__ long rows_offset(const RowsView& v, int z, int row) {
          (long)(row % v.inner) * v.si;
 }
 
+// the same offset split into its z part and its row part (the row part without divisions when row < inner)
+__device__ __forceinline__ long rows_base(const RowsView& v, int z) {
+  int i = z % v.N; z /= v.N;
+  int r = z % v.R; z /= v.R;
+  int h = z % v.H, b = z / v.H;
+  return (long)b * v.sb + (long)h * v.sh + (long)r * v.sr + (long)i * v.sn;
+}
+__device__ __forceinline__ long rows_row(const RowsView& v, int row) {
+  if (row < v.inner) return (long)row * v.si;
+  return (long)(row / v.inner) * v.so + (long)(row % v.inner) * v.si;
+}
+
 // x (dtype T) -> nat and/or tr working tensors, zero padded (rows >= L, cols >= d).
 //   tiled == 0: nat [Z][Lp][D] row-major, tr [Z][D][Lp] row-major       (chunked-mode kernels)
 //   tiled != 0: both in tiles of 32 positions, k-group-major (nat_off / tr_off)   (fused kernels)
 // tr stores position t at column perm16(t) (tr_mode 0), perm32(t) (1) or t (2) of its group of 32.
 // vec != 0: every row start of x is 16-byte aligned and d is a multiple of the 16-byte vector (host-checked), so
 // rows are read with 16-byte loads.
+// masked_nz (optional; chunked operator, z = zq*N + chunk, chunk size c): blocks of rows before their chunk are left
+// untouched while *masked_nz is 0 (k_delta has found every such row of x to be zero, and no kernel reads them then).
 template <class T, int D>
 __global__ void __launch_bounds__(256) k_pack(RowsView x, T* __restrict__ nat, T* __restrict__ tr, int d, int L, int Lp,
-                                              int tr_mode, int tiled, int vec, float* __restrict__ norm2) {
+                                              int tr_mode, int tiled, int vec, float* __restrict__ norm2,
+                                              const int* __restrict__ masked_nz, int c) {
   constexpr int V = 16 / (int)sizeof(T);
   __shared__ float tile[32][D + 1];
   const int z = blockIdx.y, row0 = blockIdx.x * 32, tid = threadIdx.x;
+  if (masked_nz && row0 + 32 <= (z % x.N) * c && *masked_nz == 0) return;
   const T* xp = reinterpret_cast<const T*>(x.p);
   if (vec) {
     for (int i = tid; i < 32 * (D / V); i += 256) {
@@ -111,37 +127,71 @@ __global__ void __launch_bounds__(256) k_pack(RowsView x, T* __restrict__ nat, T
 }
 
 // delta[z][t] = sum_dd O[z][t][dd] * dO[z][t][dd] - sub[z][t]   (fp32; padded rows -> 0)
-// O, dO, sub are views (sub optional, float); 16 lanes per row, 16 rows per block.
+// O, dO, sub are views (sub optional, float); 16 lanes per row, 128 rows per block (grid (Lp/128, Z)).
 // lse_in (optional, natural log, float view) is rewritten in log2 units into lse2 [Z][Lp].
 // vec != 0: rows of O and dO start 16-byte aligned, have unit feature stride and d is a multiple of the vector.
+// masked_nz (optional; chunked operator, z = zq*N + chunk, chunk size c): set to 1 when a row of dO or sub that lies
+// before its chunk (t < chunk*c, a query that sees no key of the chunk) holds a non-zero.
 template <class T>
 __global__ void __launch_bounds__(256) k_delta(RowsView O, RowsView dO, RowsView sub, RowsView lse_in,
-                                               float* __restrict__ delta, float* __restrict__ lse2, int d, int L, int Lp, int vec) {
-  constexpr int V = 16 / (int)sizeof(T);
+                                               float* __restrict__ delta, float* __restrict__ lse2, int d, int L, int Lp, int vec,
+                                               int* __restrict__ masked_nz, int c) {
+  constexpr int V = 16 / (int)sizeof(T), IT = 8;
   const int z = blockIdx.y, sub16 = threadIdx.x & 15;
-  const int t = blockIdx.x * 16 + (threadIdx.x >> 4);
-  float s = 0.f;
-  if (t < L) {
-    const T* o = reinterpret_cast<const T*>(O.p) + rows_offset(O, z, t);
-    const T* g = reinterpret_cast<const T*>(dO.p) + rows_offset(dO, z, t);
-    if (vec) {
-      for (int c = sub16 * V; c < d; c += 16 * V) {
-        T a[V], b[V];
-        *reinterpret_cast<uint4*>(a) = *reinterpret_cast<const uint4*>(o + c);
-        *reinterpret_cast<uint4*>(b) = *reinterpret_cast<const uint4*>(g + c);
+  const int t0 = blockIdx.x * (16 * IT) + (threadIdx.x >> 4);
+  const int chunk_start = masked_nz ? (z % dO.N) * c : 0;
+  const T* Oz = reinterpret_cast<const T*>(O.p) + rows_base(O, z);
+  const T* Gz = reinterpret_cast<const T*>(dO.p) + rows_base(dO, z);
+  const float* Sz = sub.p ? reinterpret_cast<const float*>(sub.p) + rows_base(sub, z) : nullptr;
+  const float* Lz = lse_in.p ? reinterpret_cast<const float*>(lse_in.p) + rows_base(lse_in, z) : nullptr;
+  bool flag = false;
 #pragma unroll
-        for (int e = 0; e < V; ++e) s += (float)a[e] * (float)b[e];
+  for (int it = 0; it < IT; ++it) {
+    const int t = t0 + 16 * it;
+    float s = 0.f;
+    bool nz = false;
+    if (t < L) {
+      const T* o = Oz + rows_row(O, t);
+      const T* g = Gz + rows_row(dO, t);
+      if (vec) {
+        // a row before its chunk normally holds zeros: its product with O is then not needed
+        const bool before_chunk = t < chunk_start;
+        for (int cc = sub16 * V; cc < d; cc += 16 * V) {
+          T a[V], b[V];
+          *reinterpret_cast<uint4*>(b) = *reinterpret_cast<const uint4*>(g + cc);
+          if (before_chunk) {
+            bool any = false;
+#pragma unroll
+            for (int e = 0; e < V; ++e) any |= ((float)b[e] != 0.f);
+            if (!any) continue;
+          }
+          *reinterpret_cast<uint4*>(a) = *reinterpret_cast<const uint4*>(o + cc);
+#pragma unroll
+          for (int e = 0; e < V; ++e) { s += (float)a[e] * (float)b[e]; nz |= ((float)b[e] != 0.f); }
+        }
+      } else {
+        for (int cc = sub16; cc < d; cc += 16) {
+          const float b = (float)g[(long)cc * dO.sc];
+          s += (float)o[(long)cc * O.sc] * b;
+          nz |= (b != 0.f);
+        }
       }
-    } else {
-      for (int c = sub16; c < d; c += 16) s += (float)o[(long)c * O.sc] * (float)g[(long)c * dO.sc];
     }
-  }
 #pragma unroll
-  for (int m = 8; m >= 1; m >>= 1) s += __shfl_xor(s, m, 64);
-  if (sub16 == 0 && t < Lp) {
-    if (sub.p && t < L) s -= reinterpret_cast<const float*>(sub.p)[rows_offset(sub, z, t)];
-    delta[(long)z * Lp + t] = s;
-    if (lse_in.p) lse2[(long)z * Lp + t] = (t < L) ? reinterpret_cast<const float*>(lse_in.p)[rows_offset(lse_in, z, t)] * kLog2e : 0.f;
+    for (int m = 8; m >= 1; m >>= 1) s += __shfl_xor(s, m, 64);
+    if (sub16 == 0 && t < Lp) {
+      if (Sz && t < L) {
+        const float sv = Sz[rows_row(sub, t)];
+        s -= sv;
+        nz |= (sv != 0.f);
+      }
+      delta[(long)z * Lp + t] = s;
+      if (Lz) lse2[(long)z * Lp + t] = (t < L) ? Lz[rows_row(lse_in, t)] * kLog2e : 0.f;
+    }
+    flag |= nz && t < chunk_start;
+  }
+  if (masked_nz && __any(flag)) {
+    if ((threadIdx.x & 63) == 0 && *reinterpret_cast<volatile int*>(masked_nz) == 0) atomicOr(masked_nz, 1);
   }
 }
 
