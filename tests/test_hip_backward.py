@@ -18,7 +18,7 @@ GRADS = ("dkc", "dvc", "dxq", "dsrc", "ddest")
 
 
 def _report(tag, got, want, tol, tol_dkc=None):
-    errs = {n: rel_err(g, w) for n, g, w in zip(GRADS, got, want)}
+    errs = {n: rel_err(g.reshape(w.shape), w) for n, g, w in zip(GRADS, got, want)}
     print(tag, {k: "%.2e" % v for k, v in errs.items()}, flush=True)
     bad = {k: v for k, v in errs.items() if not v <= (tol_dkc if (k == "dkc" and tol_dkc) else tol)}
     assert not bad, bad
@@ -111,3 +111,64 @@ def test_merge_kernels_match_oracle():
         dm, dv = torch.autograd.grad(res, [m, v], g.cuda())
         assert rel_err(res, want) <= TOL[dtype]
         assert rel_err(dm, wd[0]) <= TOL[dtype] and rel_err(dv, wd[1]) <= TOL[dtype]
+
+
+def _summation_order_sensitivity(inp, g_out, g_denom, dkc):
+    """How far the float32 oracle's own dkc moves when the head dimension is summed in another order (features of k, v,
+    q and of the upstream gradient permuted, result permuted back; largest move over the reversed order and four
+    random ones): mathematically the same gradient, but the key-key products round differently and
+    (2/3)(k_s.k_u)^(-1/3) amplifies that for tiny positive products (one pair with k_s.k_u = 5.6e-6 carries half of
+    the whole tensor's error in the 512x64 case)."""
+    d = inp["kc"].shape[-1]
+    gen = torch.Generator().manual_seed(1)
+    worst = 0.0
+    for trial in range(5):
+        perm = torch.arange(d).flip(0) if trial == 0 else torch.randperm(d, generator=gen)
+        inv = torch.argsort(perm)
+        args = [inp[k].float()[..., perm] for k in ("kc", "vc", "xq")] + [inp[k].float() for k in ("static_src", "static_dest")]
+        g = orc.chunked_backward(*args, g_out.float()[..., perm, :], g_denom)
+        worst = max(worst, rel_err(g[0][..., inv], dkc))
+    return worst
+
+
+FAST_CHUNK_SHAPES = [  # chunk a multiple of 64: key-/query-stationary kernels; b, h, r, L, d, c
+    (1, 2, 2, 512, 64, 64),      # query groups, two chunks per 128-key workgroup
+    (1, 1, 1, 768, 128, 192),    # chunk boundaries that are not multiples of 128
+    (1, 1, 2, 512, 32, 256),     # one chunk spans two workgroups
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", FAST_CHUNK_SHAPES)
+def test_chunked_backward_chunk_multiple_of_64(shape, dtype):
+    """Arbitrary upstream gradients (the uniform-softmax region is live), with the forward's workspace and without
+    it (recompute), then an upstream that is zero before each chunk (the region is skipped, with and without
+    UA_FLAG_SKIP_MASKED)."""
+    from universal_attention_triton_amd import ops
+    print("case chunked_bwd_fast", shape, dtype, flush=True)
+    b, h, r, L, d, c = shape
+    n = L // c
+    inp = orc.make_inputs(b, h, r, L, d, c, dtype=dtype, seed=33)
+    g = torch.Generator().manual_seed(6)
+    g_out = torch.randn(b, h, r, L, d, n, generator=g).to(dtype)
+    g_denom = torch.randn(b, h, r, L, n, generator=g).to(dtype).float()
+    ins = [inp[k].cuda() for k in NAMES]
+    out, denom, ws = ops.chunked_forward(*ins, for_backward=True)
+    want = orc.chunked_backward(*[inp[k].float() for k in NAMES], g_out.float(), g_denom)
+    tol_dkc = max(TOL[dtype], 2 * _summation_order_sensitivity(inp, g_out, g_denom, want[0]))
+    got = ops.chunked_backward(*ins, out, g_out.cuda(), g_denom.cuda(), ws=ws)
+    torch.cuda.synchronize()
+    _report("with workspace", got, want, TOL[dtype], tol_dkc)
+    got = ops.chunked_backward(*ins, out, g_out.cuda(), g_denom.cuda(), ws=None)
+    torch.cuda.synchronize()
+    _report("recompute", got, want, TOL[dtype], tol_dkc)
+    # upstream that vanishes wherever a query precedes the chunk
+    t = torch.arange(L).view(L, 1, 1)
+    live = (t >= torch.arange(n).view(1, 1, n) * c)
+    g_out0 = g_out * live.to(dtype)
+    g_denom0 = g_denom * live.view(L, n).float()
+    want0 = orc.chunked_backward(*[inp[k].float() for k in NAMES], g_out0.float(), g_denom0)
+    for skip in (False, True):
+        got0 = ops.chunked_backward(*ins, out, g_out0.cuda(), g_denom0.cuda(), ws=ws, skip_masked=skip)
+        torch.cuda.synchronize()
+        _report("zero before chunk, skip=%s" % skip, got0, want0, TOL[dtype], tol_dkc)

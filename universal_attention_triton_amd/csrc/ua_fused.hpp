@@ -624,7 +624,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
     const int tb_ = top - (s) / R;                                                          \
     if (tb_ >= (sb16 >> 1)) {                                                               \
       if (tb_ <= myreach) bwd_step((s), (base), TrueC(), tb_ == (sb16 >> 1));               \
-    } else if (CH && tb_ < cstart32) {                                                      \
+    } else if (CH && uniform_part && tb_ < cstart32) {                                      \
       uniform_step((s), (base));                                                            \
     }                                                                                       \
   }
