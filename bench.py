@@ -76,6 +76,13 @@ def cpu_baseline(cfg, index, budget_s=10.0):
                       % (heads, cfg["b"] * cfg["h"], cfg["r"], cfg["L"], cfg["d"], cfg["c"], " + backward" if cfg["bwd"] else "")}
 
 
+# HBM bytes per launch of the roofline kernel, from the TCC counters FETCH_SIZE and WRITE_SIZE of two `rocprofv3 --pmc`
+# runs of this script, each scaled by what the same counter reads for the plain 1 GiB copy of --calibrate-copy
+# (profiles/bench_cfg2_fused_fwd_bwd.md: 1.50 GB read + 0.54 GB written by k_bwd_keys2).  A measured constant, not
+# collected by a default run; configurations without such a measurement report null.
+MEASURED_TRAFFIC = {(2, "k_bwd_keys"): 2.04e9}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -86,6 +93,9 @@ def main():
     ap.add_argument("--api", choices=["fused", "chunked"], default="fused",
                     help="fused (default): universal_attention(); chunked: the reference's call sequence "
                          "UniversalAttention.apply + SMVecMatMul.apply, which materialises out[b,h,r,L,d,n]")
+    ap.add_argument("--no-pruned", action="store_true",
+                    help="skip the extra timing of the optional pruned mode (keeps a profiler's per-kernel statistics "
+                         "to the launches `value` is made of)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device-to-device copy, the known-size kernel that HBM counters of a "
                          "profiler run are scaled against")
@@ -169,7 +179,7 @@ def main():
                    "pct_of_mfma_peak": round(100 * (f_fwd + f_bwd) / (ms * 1e-3) / 1e12 / peak, 2),
                    "kernel_ms": kern},
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
-                     "frac": round(achieved / peak, 4), "traffic": None},
+                     "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get((args.config, dom))},
     }
     if args.api == "chunked":
         out["roofline"] = roof
@@ -181,16 +191,17 @@ def main():
         return
     # the same step with UA_FLAG_PRUNE (pairs whose softmax weight is provably below 2^-48 are skipped): reported
     # beside the headline, never as `value`, because it executes fewer pairs than the flop count assumes
-    for _ in range(2):
-        step(prune=True)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step(prune=True)
-    torch.cuda.synchronize()
-    ms_p = (time.perf_counter() - t0) * 1e3 / args.steps
-    out["config"]["pruned_mode"] = {"ms_per_step": round(ms_p, 4), "speedup": round(ms / ms_p, 2),
-                                    "note": "optional exact pruning of negligible pairs; not counted in value"}
+    if not args.no_pruned:
+        for _ in range(2):
+            step(prune=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step(prune=True)
+        torch.cuda.synchronize()
+        ms_p = (time.perf_counter() - t0) * 1e3 / args.steps
+        out["config"]["pruned_mode"] = {"ms_per_step": round(ms_p, 4), "speedup": round(ms / ms_p, 2),
+                                        "note": "optional exact pruning of negligible pairs; not counted in value"}
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(cfg, args.config)
     print(json.dumps(out))
