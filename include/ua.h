@@ -39,7 +39,10 @@ enum {
 };
 enum {
   UA_FLAG_SKIP_MASKED = 1, /* ua_bwd: the upstream gradient is zero for (query, chunk) pairs in which the
-                              query precedes the whole chunk (true when it comes from ua_merge_bwd) */
+                              query precedes the whole chunk (true when it comes from ua_merge_bwd).  Without the
+                              flag ua_bwd finds this out by itself for chunks that are multiples of 64 (one pass
+                              over g_out and g_denom that it makes anyway); the flag saves that check and, for the
+                              other chunk sizes, the sweep over those pairs. */
   UA_FLAG_PRUNE = 2        /* fused ops: skip (key, query) pairs whose softmax weight is provably below 2^-48 because
                               of the accumulated decay (no counterpart in the reference, which visits every pair).
                               The bound uses the largest key and query norms of the head; results change by less

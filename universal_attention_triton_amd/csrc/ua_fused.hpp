@@ -291,7 +291,7 @@ __global__ void __launch_bounds__(256) k_chunk_masked_denom(T* __restrict__ deno
 // CHUNKED: the reference's chunked operator instead of the merged one: the softmax restarts at every chunk of
 // co.c keys (a multiple of 64) and each chunk's result goes to out[.., i] / denom[.., i] / lse2[zq*nch + i][t].
 template <class T, int D, int NST, int NW, bool CHUNKED>
-__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4, NW / 4))) k_fwd_fused2(const T* __restrict__ Qp, const T* __restrict__ Kp,
+__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW >= 8 ? NW / 4 : 2, NW >= 8 ? NW / 4 : 2))) k_fwd_fused2(const T* __restrict__ Qp, const T* __restrict__ Kp,
                                                     const T* __restrict__ VT, const float* __restrict__ lsrc,
                                                     const float* __restrict__ ldest, const float* __restrict__ C,
                                                     T* __restrict__ O, float* __restrict__ lse, float* __restrict__ lse2,

@@ -39,7 +39,7 @@ hipError_t launch_carry(int dtype, int D, const void* Kp, const float* lsrc, con
                                                            const float*, T*, float*, float*, const int*, const int*, \
                                                            int, int, int, int, ChunkOut<T>);
 UA_INST(bf16, 64, 1, 8, false) UA_INST(bf16, 64, 2, 8, false) UA_INST(bf16, 64, 2, 12, false) UA_INST(bf16, 64, 2, 16, false)
-UA_INST(bf16, 128, 1, 8, false) UA_INST(bf16, 128, 2, 8, false) UA_INST(bf16, 128, 2, 12, false) UA_INST(bf16, 128, 2, 16, false)
+UA_INST(bf16, 128, 2, 4, false) UA_INST(bf16, 64, 2, 4, false) UA_INST(bf16, 128, 1, 8, false) UA_INST(bf16, 128, 2, 8, false) UA_INST(bf16, 128, 2, 12, false) UA_INST(bf16, 128, 2, 16, false)
 UA_INST(float, 64, 1, 8, false) UA_INST(float, 128, 1, 8, false)
 UA_INST(bf16, 64, 2, 8, true) UA_INST(bf16, 128, 2, 8, true) UA_INST(float, 64, 1, 8, true) UA_INST(float, 128, 1, 8, true)
 #undef UA_INST
@@ -54,7 +54,7 @@ static hipError_t fused_t(const void* Qp, const void* Kp, const void* VT, const 
 }
 // variants (bf16): 0 = 8 waves, double-buffered stages; 1 = 8 waves, single stage; 2 = 12 waves; 3 = 16 waves
 // (both double-buffered).  fp32 always runs 8 waves with a single stage.
-int fwd_fused_variants(int dtype, int D) { (void)D; return dtype == 1 ? 4 : 1; }
+int fwd_fused_variants(int dtype, int D) { (void)D; return dtype == 1 ? 5 : 1; }
 template <class T, int D>
 static hipError_t fused_v(int variant, const void* Qp, const void* Kp, const void* VT, const float* lsrc, const float* ldest,
                           const float* C, void* O, float* lse, float* lse2, const int* reach, const int* minkey, int R, int L,
@@ -64,6 +64,7 @@ static hipError_t fused_v(int variant, const void* Qp, const void* Kp, const voi
     case 1: return fused_t<T, D, 1, 8>(UA_ARGS);
     case 2: return fused_t<T, D, 2, 12>(UA_ARGS);
     case 3: return fused_t<T, D, 2, 16>(UA_ARGS);
+    case 4: return fused_t<T, D, 2, 4>(UA_ARGS);
     default: return fused_t<T, D, 2, 8>(UA_ARGS);
   }
 #undef UA_ARGS
