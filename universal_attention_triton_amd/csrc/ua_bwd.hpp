@@ -38,6 +38,7 @@ struct BwdArgs {
   float *dKrow, *dVrow;         // [Zk][Lp][D]
   float* dsrc_raw;              // [Zk][Lp]
   int R, L, Lp, c, nch, chunked, skip_masked;
+  int split_r;                  // k_bwd_queries2: one workgroup per (kv head, query group); dKdacc is then [Zq][Lp][D]
 };
 
 // grid (key groups, Zk).  chunked == 0: key group = 128 consecutive keys, 4 waves.
@@ -276,7 +277,7 @@ __global__ void __launch_bounds__(256) k_bwd_finish(const float* __restrict__ dK
                                                     const T* __restrict__ src, const T* __restrict__ dest,
                                                     T* __restrict__ dk, T* __restrict__ dv, T* __restrict__ dq,
                                                     T* __restrict__ dsrc, T* __restrict__ ddest, int Zk, int Zq, int L,
-                                                    int Lp, int D, int d, int tiled) {
+                                                    int Lp, int D, int d, int tiled, int RS) {
   const int z = blockIdx.y, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + wave;
   if (t >= L) return;
@@ -288,7 +289,9 @@ __global__ void __launch_bounds__(256) k_bwd_finish(const float* __restrict__ dK
     float dot = 0.f;
     for (int c = lane; c < d; c += 64) {
       const long i = ((long)z * Lp + t) * D + c;
-      const float kd = dKdacc[i];
+      // RS > 1: the column side comes in one slice per query group of the head
+      float kd = 0.f;
+      for (int r = 0; r < RS; ++r) kd += dKdacc[(((long)z * RS + r) * Lp + t) * D + c];
       // the packed keys are row-major in chunked mode and tiled (nat_off) in fused mode
       const long ik = !tiled ? i : (D == 64 ? nat_off<64>(z, Lp, t, c) : nat_off<128>(z, Lp, t, c));
       dot += kd * (float)Kp[ik];

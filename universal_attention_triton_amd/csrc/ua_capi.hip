@@ -82,7 +82,7 @@ Layout make_layout(const ua_desc& d, bool chunked) {
   // suffix carries instead
   const bool atomics = chunked && d.chunk % 64 != 0;
   l.dQacc = atomics ? take((size_t)l.Zq * l.Lp * l.D * 4) : 0;
-  l.dKdacc = take((size_t)l.Zk * l.Lp * l.D * 4);
+  l.dKdacc = take((size_t)(atomics ? l.Zk : l.Zq) * l.Lp * l.D * 4);   // one slice per query group without atomics
   l.Dsuf = atomics ? 0 : take((size_t)l.Zk * l.nT * l.Lp * 4);
   l.masked_nz = take(256);
   l.dKrow = take((size_t)l.Zk * l.Lp * l.D * 4);
@@ -252,7 +252,7 @@ hipError_t finish_t(const Layout& l, const ua_desc& d, char* ws, bool chunked, c
   hipLaunchKernelGGL((ua::k_bwd_finish<T>), dim3((d.L + 3) / 4, Z), dim3(256), 0, s, (const float*)(ws + l.dKrow),
                      (const float*)(ws + l.dVrow), (const float*)(ws + l.dKdacc), chunked ? (const float*)(ws + l.dQacc) : nullptr,
                      (const float*)(ws + l.dsrc_raw), (const T*)(ws + l.Kp), (const T*)src, (const T*)dest, (T*)dk, (T*)dv,
-                     (T*)dq, (T*)dsrc, (T*)ddest, l.Zk, l.Zq, d.L, l.Lp, l.D, d.d, chunked ? 0 : 1);
+                     (T*)dq, (T*)dsrc, (T*)ddest, l.Zk, l.Zq, d.L, l.Lp, l.D, d.d, chunked ? 0 : 1, chunked ? 1 : d.r);
   return hipGetLastError();
 }
 
@@ -286,6 +286,7 @@ int run_bwd_common(const ua_desc& d, const Layout& l, char* ws, bool chunked, co
   a.masked_nz = (const int*)(ws + l.masked_nz);
   a.R = d.r; a.L = d.L; a.Lp = l.Lp; a.c = is_chunked ? d.chunk : 128; a.nch = l.nch; a.chunked = is_chunked ? 1 : 0;
   a.skip_masked = (d.flags & UA_FLAG_SKIP_MASKED) ? 1 : 0;
+  a.split_r = (!chunked && d.r > 1) ? 1 : 0;
   {
     UA_PROF("k_bwd_keys", s);
     UA_HIP(ua::launch_bwd_keys(d.dtype, l.D, a, l.Zk, chunked ? 1 : 0, s));

@@ -789,9 +789,14 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
   UA_STAGES(SB);
   __shared__ __attribute__((aligned(256))) char sXbuf[8 * 2 * ST::BYTES];
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
-  int bx, zk;
-  xcd_map(bx, zk);
+  // grid y: kv heads (the query groups of a head are then swept one after the other), or, when gridDim.y is the number
+  // of query heads, one (kv head, query group) per workgroup: more, smaller workgroups; the column-side key gradient
+  // is then written per query head and added up by k_bwd_finish
+  int bx, zy;
+  xcd_map(bx, zy);
   const int Lp = a.Lp, L = a.L, nT16 = Lp / 16, R = a.R;
+  const bool split_r = a.split_r != 0;
+  const int zk = split_r ? zy / R : zy, r_begin = split_r ? zy % R : 0, r_end = split_r ? r_begin + 1 : R;
   const int jt = gridDim.x - 1 - bx, tq = 8 * jt + w;
   char* sX = sXbuf + w * 2 * ST::BYTES;      // [dS of a 32-key half][dg of that half]
   const GroupMasks gm = group_masks(lane);
@@ -835,7 +840,7 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
   const int uk0_w = CH ? ((min((16 * tq) / a.c, a.nch - 1) + 1) * a.c) >> 6 : 0;
   const int uk1 = uniform_part ? max(uk0, L >> 6) : uk0;
 
-  for (int r = 0; r < R; ++r) {
+  for (int r = r_begin; r < r_end; ++r) {
     const long zq = (long)zk * R + r;
     Frag<T> qt[NK], gt[NK];
     f32x4 l2t, dlt;
@@ -1002,7 +1007,7 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
   for (int v = 0; v < 4; ++v) {
     const int t = 16 * tq + 4 * g + v;
 #pragma unroll
-    for (int n = 0; n < ND; ++n) a.dKdacc[((long)zk * Lp + t) * D + 16 * n + col] = dKc[n][v];
+    for (int n = 0; n < ND; ++n) a.dKdacc[((long)zy * Lp + t) * D + 16 * n + col] = dKc[n][v];
   }
 }
 

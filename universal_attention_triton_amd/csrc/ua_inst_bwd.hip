@@ -13,7 +13,7 @@ static BwdArgs<T> typed(const BwdArgsV& v) {
   a.dOp = (const T*)v.dOp; a.dOT = (const T*)v.dOT; a.lsrc = v.lsrc; a.ldest = v.ldest; a.lse2 = v.lse2; a.delta = v.delta;
   a.C = v.C;
   a.dQacc = v.dQacc; a.dKdacc = v.dKdacc; a.Dsuf = v.Dsuf; a.dKrow = v.dKrow; a.dVrow = v.dVrow; a.dsrc_raw = v.dsrc_raw;
-  a.R = v.R; a.L = v.L; a.Lp = v.Lp; a.c = v.c; a.nch = v.nch; a.chunked = v.chunked; a.skip_masked = v.skip_masked;
+  a.R = v.R; a.L = v.L; a.Lp = v.Lp; a.c = v.c; a.nch = v.nch; a.chunked = v.chunked; a.skip_masked = v.skip_masked; a.split_r = v.split_r;
   return a;
 }
 
@@ -69,8 +69,9 @@ UA_INST(bf16, 64, 2) UA_INST(bf16, 128, 2) UA_INST(float, 64, 1) UA_INST(float, 
 template <class T, int D, int NST>
 static hipError_t bwdq_t(const BwdArgsV& v, void* dq, int d, int Zk, hipStream_t s) {
   const BwdArgs<T> a = typed<T>(v);
-  if (v.chunked) hipLaunchKernelGGL((k_bwd_queries2<T, D, NST, true>), dim3(v.Lp / 128, Zk), dim3(512), 0, s, a, (T*)dq, d);
-  else hipLaunchKernelGGL((k_bwd_queries2<T, D, NST, false>), dim3(v.Lp / 128, Zk), dim3(512), 0, s, a, (T*)dq, d);
+  const dim3 grid(v.Lp / 128, v.split_r ? Zk * v.R : Zk);
+  if (v.chunked) hipLaunchKernelGGL((k_bwd_queries2<T, D, NST, true>), grid, dim3(512), 0, s, a, (T*)dq, d);
+  else hipLaunchKernelGGL((k_bwd_queries2<T, D, NST, false>), grid, dim3(512), 0, s, a, (T*)dq, d);
   return hipGetLastError();
 }
 hipError_t launch_bwd_queries(int dtype, int D, const BwdArgsV& a, void* dq, int d, int Zk, hipStream_t s) {

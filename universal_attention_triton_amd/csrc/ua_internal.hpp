@@ -12,7 +12,7 @@ struct BwdArgsV {
   const void *Kp, *Vp, *KT, *Qp, *QT, *dOp, *dOT;
   const float *lsrc, *ldest, *lse2, *delta, *C;
   float *dQacc, *dKdacc, *Dsuf, *dKrow, *dVrow, *dsrc_raw;
-  int R, L, Lp, c, nch, chunked, skip_masked;
+  int R, L, Lp, c, nch, chunked, skip_masked, split_r;
 };
 
 // Every launcher returns hipGetLastError() after enqueuing.  dtype: 0 fp32, 1 bf16.  D in {64,128}.
