@@ -788,6 +788,12 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
   constexpr int TILES = 4 * TN::BYTES + 2 * TT::BYTES, SB = TILES + 8 * 1024;   // + per wave [C: 64f][lsrc: 64f][Dsuf: 64f]
   UA_STAGES(SB);
   __shared__ __attribute__((aligned(256))) char sXbuf[8 * 2 * ST::BYTES];
+  // Chunked operator: the stationary upstream rows of the NEXT chunk are copied asynchronously into a wave-private
+  // LDS region one step ahead (where the 160 KB of LDS allow it), so that entering a chunk costs an LDS read instead
+  // of a round trip to memory; lse2 and delta of the step's chunk travel in the stats row.
+  constexpr int GBYTES = 16 * D * (int)sizeof(T), GH = (int)sizeof(Frag<T>) / 16;
+  constexpr bool PRE = CH && (NST == 2 ? 2 * SB : SB + 1024) + 8 * 2 * ST::BYTES + 8 * GBYTES <= 163840;
+  __shared__ __attribute__((aligned(1024))) char sGbuf[PRE ? 8 * GBYTES : 1024];
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
   // grid y: kv heads (the query groups of a head are then swept one after the other), or, when gridDim.y is the number
   // of query heads, one (kv head, query group) per workgroup: more, smaller workgroups; the column-side key gradient
@@ -822,7 +828,8 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
   // a tile that does not reach this wave's block gets a carry of -1e30, which zeroes its dS and dG
   const int tbq = tq >> 1;
   const int kt_min = (a.minkey[zk * (nT16 >> 1) + 4 * jt] >> 2) & ~1;
-  // per-wave stats row of a step: [C row: 64f][lsrc: 64f][Dsuf row: 64f][reach of the 4 key tiles: 4 ints]; source of
+  // per-wave stats row of a step: [C row: 64f][lsrc: 64f][Dsuf row: 64f][reach of the 4 key tiles: 4 ints] and, with
+  // the chunked operator, [lse2: 16f][delta: 16f] of this wave's queries in the step's chunk at floats 208 and 224; source of
   // each lane's 16 bytes as base + step * stride (in 4-byte units)
   const float* row_base;
   int row_step = 64;
@@ -844,14 +851,42 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
     const long zq = (long)zk * R + r;
     Frag<T> qt[NK], gt[NK];
     f32x4 l2t, dlt;
-    int cur_chunk = -1;
-    // upstream operands of chunk ch (chunked operator) or of the merged operator (ch = 0, nch = 1)
+    int cur_chunk = -1;      // chunk whose upstream rows gt holds
+    int in_lds = -1;         // chunk whose upstream rows are (being) copied into this wave's LDS region
+    char* sG = sGbuf + (PRE ? w * GBYTES : 0);
+    // upstream operands of chunk ch (chunked operator) or of the merged operator (ch = 0, nch = 1), straight from memory
     auto load_upstream = [&] __device__ (int ch) __attribute__((always_inline)) {
       const long zg = CH ? zq * a.nch + ch : zq;
 #pragma unroll
       for (int q = 0; q < NK; ++q) gt[q] = ld8(a.dOp + nat_off<D>(zg, Lp, 16 * tq + col, 32 * q + 8 * g));
-      l2t = load_t4(a.lse2 + zg * Lp + 16 * tq, g);
-      dlt = load_t4(a.delta + zg * Lp + 16 * tq, g);
+      if (!PRE) {
+        l2t = load_t4(a.lse2 + zg * Lp + 16 * tq, g);
+        dlt = load_t4(a.delta + zg * Lp + 16 * tq, g);
+      }
+      cur_chunk = ch;
+    };
+    // PRE: every lane copies the 16-byte pieces of its own operand fragments; the copy is complete after the next
+    // step's wait_async_loads()
+    auto prefetch_upstream = [&] __device__ (int ch) __attribute__((always_inline)) {
+      if (ch == in_lds) return;
+      const long zg = zq * a.nch + ch;
+#pragma unroll
+      for (int q = 0; q < NK; ++q)
+#pragma unroll
+        for (int hh = 0; hh < GH; ++hh)
+          issue_row(sG + (q * GH + hh) * 1024,
+                    reinterpret_cast<const char*>(a.dOp + nat_off<D>(zg, Lp, 16 * tq + col, 32 * q + 8 * g)) + 16 * hh);
+      in_lds = ch;
+    };
+    // PRE: fragments of chunk ch out of the LDS region (which must hold them, completely)
+    auto take_upstream = [&] __device__ (int ch) __attribute__((always_inline)) {
+      if (ch == cur_chunk) return;
+#pragma unroll
+      for (int q = 0; q < NK; ++q)
+#pragma unroll
+        for (int hh = 0; hh < GH; ++hh)
+          reinterpret_cast<uint4*>(&gt[q])[hh] = *reinterpret_cast<const uint4*>(sG + (q * GH + hh) * 1024 + 16 * lane);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // before the region may be refilled
       cur_chunk = ch;
     };
     {
@@ -866,13 +901,21 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
 #define UA_ISSUE(s, base)                                                                   \
   {                                                                                         \
     const int k0_ = 64 * ((s) < n_kt ? (s) : (s) - n_kt + uk0);                             \
+    const int ch_ = CH ? min(k0_ / a.c, a.nch - 1) : 0;                                     \
+    if (PRE && in_lds >= 0) take_upstream(in_lds);   /* rows of the step computed next */    \
     stN.issue((base), Kz + (long)k0_ * D, w);                                               \
     stN.issue((base) + TN::BYTES, Kz + (long)(k0_ + 32) * D, w);                            \
     stN.issue((base) + 2 * TN::BYTES, Vz + (long)k0_ * D, w);                               \
     stN.issue((base) + 3 * TN::BYTES, Vz + (long)(k0_ + 32) * D, w);                        \
     stT.issue((base) + 4 * TN::BYTES, KTz + (long)k0_ * D, w);                              \
     stT.issue((base) + 4 * TN::BYTES + TT::BYTES, KTz + (long)(k0_ + 32) * D, w);           \
-    issue_row((base) + TILES + w * 1024, row_base + (long)(k0_ >> 6) * row_step);           \
+    {                                                                                       \
+      const float* src_ = row_base + (long)(k0_ >> 6) * row_step;                           \
+      if (PRE && lane >= 52 && lane < 60)                                                   \
+        src_ = (lane < 56 ? a.lse2 : a.delta) + (zq * a.nch + ch_) * Lp + 16 * tq + 4 * (lane & 3); \
+      issue_row((base) + TILES + w * 1024, src_);                                           \
+    }                                                                                       \
+    if (PRE) prefetch_upstream(ch_);                                                        \
   }
 #define UA_COMPUTE_FAST(s, base) bq_step((s), (base), FalseC())
 #define UA_COMPUTE_SLOW(s, base)                                                            \
@@ -884,7 +927,12 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
     // dS = (dP - delta) / c (see k_bwd_keys2), no decay part.
     auto uniform_step = [&] __device__ (int kti, const char* base) __attribute__((always_inline)) {
       const int ch = min((64 * kti) / a.c, a.nch - 1);
-      if (ch != cur_chunk) load_upstream(ch);
+      if (PRE) {
+        take_upstream(ch);
+        dlt = load_t4(reinterpret_cast<const float*>(base + TILES + w * 1024) + 224, g);
+      } else if (ch != cur_chunk) {
+        load_upstream(ch);
+      }
 #pragma unroll
       for (int kq = 0; kq < 2; ++kq) {
         const T* sV = reinterpret_cast<const T*>(base + (2 + kq) * TN::BYTES);
@@ -908,7 +956,13 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
       const float* stats = reinterpret_cast<const float*>(base + TILES + w * 1024);
       if constexpr (CH) {
         const int ch = min((64 * kti) / a.c, a.nch - 1);
-        if (ch != cur_chunk) load_upstream(ch);
+        if (PRE) {
+          take_upstream(ch);
+          l2t = load_t4(stats + 208, g);
+          dlt = load_t4(stats + 224, g);
+        } else if (ch != cur_chunk) {
+          load_upstream(ch);
+        }
       }
       // the 64 keys of the step are handled as two halves of 32 (= one contraction step of the column products);
 #pragma unroll
