@@ -584,6 +584,10 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   const float* ldz = a.ldest + (long)zk * Lp;
   const float* Cz = a.C + (long)zk * nT16 * Lp + 128 * kg;
   float* Dz = a.Dsuf + (long)zk * nT16 * Lp + spos;
+  // where this lane's four values of a (16 keys, 16 queries) tile go inside the 1 KB tile of its 32-key half
+  const bool store_tiles = sizeof(T) == 2 && a.dS_st != nullptr;
+  const long st_row = (long)(Lp >> 5) << 10;                       // bytes between consecutive 16-query tiles
+  const long st_lane = ((long)(sb16 >> 1) << 10) + StageT<bf16>::addr(perm32(16 * (sb16 & 1) + col), 8 * g);
 
 #define UA_ISSUE(s, base)                                                                   \
   {                                                                                         \
@@ -712,6 +716,13 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
         }
       }
       const Frag<T> bp = as_operand16<T>(P[0], P[1]), bs = as_operand16<T>(dS[0], dS[1]);
+      if constexpr (sizeof(T) == 2) {
+        if (store_tiles) {     // the two halves of the operand are the two query tiles of the block
+          char* p = reinterpret_cast<char*>(a.dS_st) + (((long)zk * R + r) * nT16 + 2 * tb) * st_row + st_lane;
+          __builtin_nontemporal_store(reinterpret_cast<const uint2*>(&bs)[0], reinterpret_cast<uint2*>(p));
+          __builtin_nontemporal_store(reinterpret_cast<const uint2*>(&bs)[1], reinterpret_cast<uint2*>(p + st_row));
+        }
+      }
 #pragma unroll
       for (int n = 0; n < ND; ++n) mma16(dVt[n], ld8(sdOT + TT::at(n, col, 0, g)), bp);
 #pragma unroll
@@ -740,6 +751,13 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
       }
       dcar += tot;
       const Frag<T> b = as_operand16<T>(dB[0], dB[1]);
+      if constexpr (sizeof(T) == 2) {
+        if (store_tiles) {
+          char* p = reinterpret_cast<char*>(a.dG_st) + ((long)zk * nT16 + 2 * tb) * st_row + st_lane;
+          __builtin_nontemporal_store(reinterpret_cast<const uint2*>(&b)[0], reinterpret_cast<uint2*>(p));
+          __builtin_nontemporal_store(reinterpret_cast<const uint2*>(&b)[1], reinterpret_cast<uint2*>(p + st_row));
+        }
+      }
 #pragma unroll
       for (int n = 0; n < ND; ++n) mma16(dKt[n], ld8(sKT + TT::at(n, col, 0, g)), b);
     }
@@ -1062,6 +1080,98 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
     const int t = 16 * tq + 4 * g + v;
 #pragma unroll
     for (int n = 0; n < ND; ++n) a.dKdacc[((long)zy * Lp + t) * D + 16 * n + col] = dKc[n][v];
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Query side of the backward from the tiles k_bwd_keys2 left (16-bit dtypes, fused mode): pure matrix work.
+//   dQ[t,:] = sum_s dS[s,t] k_s        dkcol[u,:] = sum_s dG[s,u] k_s
+// grid (Lp/128, Zq); 8 waves; wave w owns queries 16*(8*jt+w)..+15 and streams its own row of 1 KB tiles (two
+// 32-key halves of dS and of dG per step of 64 keys) straight into LDS, where they are read transposed as A
+// operands; the transposed key tiles are shared by the workgroup.  dG belongs to the kv head: with r query groups
+// per head, group r accumulates the feature tiles n = r, r + R, ... of dkcol (its slice of dKdacc holds zeros
+// elsewhere; k_bwd_finish adds the slices).
+// ---------------------------------------------------------------------------------------------
+template <class T, int D, int NST>
+__global__ void __launch_bounds__(512) k_bwd_queries3(BwdArgs<T> a, T* __restrict__ dq, int d) {
+  static_assert(sizeof(T) == 2, "tiles are exchanged in 16-bit operand precision");
+  using TT = Tile<T, D, 32>;
+  using ST = StageT<T>;
+  constexpr int ND = D / 16;
+  // stage: [KT half 0][KT half 1][per wave: dS half 0, dS half 1, dG half 0, dG half 1][reach of the 4 key tiles]
+  constexpr int TILES = 2 * TT::BYTES, WAVE = 4 * ST::BYTES, SB = TILES + 8 * WAVE + 1024;
+  UA_STAGES(SB);
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
+  int bx, zq;
+  xcd_map(bx, zq);
+  const int Lp = a.Lp, L = a.L, nT16 = Lp / 16, R = a.R, zk = zq / R, r = zq % R;
+  const int jt = gridDim.x - 1 - bx, tq = 8 * jt + w, tbq = tq >> 1;
+  Stager<TT, 8> stT;
+  stT.init(w, lane, Lp * (long)sizeof(T), D);
+  f32x4 dQ[ND], dKc[ND];
+#pragma unroll
+  for (int n = 0; n < ND; ++n) { dQ[n] = (f32x4){0, 0, 0, 0}; dKc[n] = (f32x4){0, 0, 0, 0}; }
+  const T* KTz = a.KT + (long)zk * D * Lp;
+  const int n_kt = 2 * jt + 2;
+  const int kt_min = (a.minkey[zk * (nT16 >> 1) + 4 * jt] >> 2) & ~1;
+  const long st_row = (long)(Lp >> 5) << 10;
+  // this lane's 16 bytes of the wave's tiles of key half h: base + h * 1024
+  const char* pS = reinterpret_cast<const char*>(a.dS_st) + ((long)zq * nT16 + tq) * st_row + 16 * lane;
+  const char* pG = reinterpret_cast<const char*>(a.dG_st) + ((long)zk * nT16 + tq) * st_row + 16 * lane;
+  const int* reach_z = a.reach + zk * nT16;
+
+#define UA_ISSUE(s, base)                                                                   \
+  {                                                                                         \
+    const int k0_ = 64 * (s);                                                               \
+    stT.issue((base), KTz + (long)k0_ * D, w);                                              \
+    stT.issue((base) + TT::BYTES, KTz + (long)(k0_ + 32) * D, w);                           \
+    char* mine_ = (base) + TILES + w * WAVE;                                                \
+    const long h_ = (long)(2 * (s)) << 10;                                                  \
+    __builtin_amdgcn_global_load_lds(pS + h_, (lds_ptr_t)mine_, 16, 0, 0);                  \
+    __builtin_amdgcn_global_load_lds(pS + h_ + 1024, (lds_ptr_t)(mine_ + ST::BYTES), 16, 0, 0);     \
+    __builtin_amdgcn_global_load_lds(pG + h_, (lds_ptr_t)(mine_ + 2 * ST::BYTES), 16, 0, 0);        \
+    __builtin_amdgcn_global_load_lds(pG + h_ + 1024, (lds_ptr_t)(mine_ + 3 * ST::BYTES), 16, 0, 0); \
+    if (w == 0) issue_row((base) + TILES + 8 * WAVE, reach_z + 4 * (s));                    \
+  }
+#define UA_COMPUTE(s, base) bq_step((s), (base))
+  auto bq_step = [&] __device__ (int kti, char* base) {
+    char* mine = base + TILES + w * WAVE;
+    const int* rch = reinterpret_cast<const int*>(base + TILES + 8 * WAVE);
+#pragma unroll
+    for (int kq = 0; kq < 2; ++kq) {
+      // the half's two 16-key tiles: visited by k_bwd_keys2 (hence written) iff not after the queries and in reach
+      const int sbk = 4 * kti + 2 * kq;
+      const bool live0 = sbk <= tq && rch[2 * kq] >= tbq, live1 = sbk + 1 <= tq && rch[2 * kq + 1] >= tbq;
+      if (!live0 && !live1) continue;
+      Frag<T> as = ST::get(mine + kq * ST::BYTES, lane), ag = ST::get(mine + (2 + kq) * ST::BYTES, lane);
+      // elements 0-3 of an operand are keys of the first tile, 4-7 of the second (perm32)
+      if (!live0) { reinterpret_cast<uint2*>(&as)[0] = make_uint2(0, 0); reinterpret_cast<uint2*>(&ag)[0] = make_uint2(0, 0); }
+      if (!live1) { reinterpret_cast<uint2*>(&as)[1] = make_uint2(0, 0); reinterpret_cast<uint2*>(&ag)[1] = make_uint2(0, 0); }
+      const T* sKT = reinterpret_cast<const T*>(base + kq * TT::BYTES);
+#pragma unroll
+      for (int n = 0; n < ND; ++n) {
+        const Frag<T> kb = ld8(sKT + TT::at(n, col, 0, g));
+        mma16(dQ[n], as, kb);
+        if (n % R == r) mma16(dKc[n], ag, kb);
+      }
+    }
+  };
+  UA_PIPE_START_AT(kt_min, n_kt, UA_ISSUE);
+  UA_PIPE_RANGE(kt_min, n_kt, n_kt, UA_ISSUE, UA_COMPUTE);
+#undef UA_ISSUE
+#undef UA_COMPUTE
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    const int t = 16 * tq + 4 * g + v;
+    if (t < L) {
+#pragma unroll
+      for (int n = 0; n < ND; ++n) {
+        const int dd = 16 * n + col;
+        if (dd < d) dq[((long)zq * L + t) * d + dd] = cvt<T>(dQ[n][v]);
+      }
+    }
+#pragma unroll
+    for (int n = 0; n < ND; ++n) a.dKdacc[((long)zq * Lp + t) * D + 16 * n + col] = dKc[n][v];
   }
 }
 

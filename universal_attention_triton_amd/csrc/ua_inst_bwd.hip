@@ -12,6 +12,7 @@ static BwdArgs<T> typed(const BwdArgsV& v) {
   a.Kp = (const T*)v.Kp; a.Vp = (const T*)v.Vp; a.KT = (const T*)v.KT; a.Qp = (const T*)v.Qp; a.QT = (const T*)v.QT;
   a.dOp = (const T*)v.dOp; a.dOT = (const T*)v.dOT; a.lsrc = v.lsrc; a.ldest = v.ldest; a.lse2 = v.lse2; a.delta = v.delta;
   a.C = v.C;
+  a.dS_st = (T*)v.dS_st; a.dG_st = (T*)v.dG_st;
   a.dQacc = v.dQacc; a.dKdacc = v.dKdacc; a.Dsuf = v.Dsuf; a.dKrow = v.dKrow; a.dVrow = v.dVrow; a.dsrc_raw = v.dsrc_raw;
   a.R = v.R; a.L = v.L; a.Lp = v.Lp; a.c = v.c; a.nch = v.nch; a.chunked = v.chunked; a.skip_masked = v.skip_masked; a.split_r = v.split_r;
   return a;
@@ -77,6 +78,16 @@ static hipError_t bwdq_t(const BwdArgsV& v, void* dq, int d, int Zk, hipStream_t
 hipError_t launch_bwd_queries(int dtype, int D, const BwdArgsV& a, void* dq, int d, int Zk, hipStream_t s) {
   if (dtype == 1) return D == 64 ? bwdq_t<bf16, 64, 2>(a, dq, d, Zk, s) : bwdq_t<bf16, 128, 2>(a, dq, d, Zk, s);
   return D == 64 ? bwdq_t<float, 64, 1>(a, dq, d, Zk, s) : bwdq_t<float, 128, 1>(a, dq, d, Zk, s);
+}
+
+template __global__ void k_bwd_queries3<bf16, 64, 2>(BwdArgs<bf16>, bf16*, int);
+template __global__ void k_bwd_queries3<bf16, 128, 2>(BwdArgs<bf16>, bf16*, int);
+hipError_t launch_bwd_queries_from_tiles(int D, const BwdArgsV& v, void* dq, int d, int Zq, hipStream_t s) {
+  const BwdArgs<bf16> a = typed<bf16>(v);
+  const dim3 grid(v.Lp / 128, Zq);
+  if (D == 64) hipLaunchKernelGGL((k_bwd_queries3<bf16, 64, 2>), grid, dim3(512), 0, s, a, (bf16*)dq, d);
+  else hipLaunchKernelGGL((k_bwd_queries3<bf16, 128, 2>), grid, dim3(512), 0, s, a, (bf16*)dq, d);
+  return hipGetLastError();
 }
 
 }  // namespace ua

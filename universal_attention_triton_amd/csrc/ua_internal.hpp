@@ -12,6 +12,7 @@ struct BwdArgsV {
   const void *Kp, *Vp, *KT, *Qp, *QT, *dOp, *dOT;
   const float *lsrc, *ldest, *lse2, *delta, *C;
   float *dQacc, *dKdacc, *Dsuf, *dKrow, *dVrow, *dsrc_raw;
+  void *dS_st, *dG_st;
   int R, L, Lp, c, nch, chunked, skip_masked, split_r;
 };
 
@@ -39,5 +40,7 @@ hipError_t launch_fwd_chunked2(int dtype, int D, const void* Qp, const void* Kp,
 // with a.chunked set: the chunked operator for a chunk that is a multiple of 64).
 hipError_t launch_bwd_keys(int dtype, int D, const BwdArgsV& a, int Zk, int cols, hipStream_t s);
 hipError_t launch_bwd_queries(int dtype, int D, const BwdArgsV& a, void* dq, int d, int Zk, hipStream_t s);
+// bf16 only, a.dS_st / a.dG_st filled by launch_bwd_keys (cols == 0): the query side as pure matrix work over those tiles
+hipError_t launch_bwd_queries_from_tiles(int D, const BwdArgsV& a, void* dq, int d, int Zq, hipStream_t s);
 
 }  // namespace ua

@@ -40,10 +40,11 @@ class UniversalAttention(_ChunkedBase):
 
 class _FusedUniversalAttention(Function):
     @staticmethod
-    def forward(ctx, kc, vc, xq, static_src, static_dest, prune=False):
+    def forward(ctx, kc, vc, xq, static_src, static_dest, prune=False, recompute=False):
         need_grad = any(ctx.needs_input_grad)
-        O, lse, ws = ops.fused_forward(kc, vc, xq, static_src, static_dest, for_backward=need_grad, prune=prune)
-        ctx.prune = prune
+        O, lse, ws = ops.fused_forward(kc, vc, xq, static_src, static_dest, for_backward=need_grad, prune=prune,
+                                       recompute=recompute)
+        ctx.prune, ctx.recompute = prune, recompute
         ctx.save_for_backward(kc, vc, xq, static_src, static_dest, O, lse)
         ctx.ws = ws if need_grad else None
         ctx.mark_non_differentiable(lse)
@@ -54,16 +55,19 @@ class _FusedUniversalAttention(Function):
         kc, vc, xq, static_src, static_dest, O, lse = ctx.saved_tensors
         b, h, n, c, d = kc.shape
         dO = dO.reshape(b, h, xq.shape[2], n * c, d)
-        dk, dv, dq, dsrc, ddest = ops.fused_backward(kc, vc, xq, static_src, static_dest, O, lse, dO, ws=ctx.ws, prune=ctx.prune)
+        dk, dv, dq, dsrc, ddest = ops.fused_backward(kc, vc, xq, static_src, static_dest, O, lse, dO, ws=ctx.ws, prune=ctx.prune,
+                                                     recompute=ctx.recompute)
         ctx.ws = None
-        return dk, dv, dq.view(xq.shape), dsrc.view(static_src.shape), ddest.view(static_dest.shape), None
+        return dk, dv, dq.view(xq.shape), dsrc.view(static_src.shape), ddest.view(static_dest.shape), None, None
 
 
-def universal_attention(kc, vc, xq, static_src, static_dest, return_lse=False, prune=False):
+def universal_attention(kc, vc, xq, static_src, static_dest, return_lse=False, prune=False, recompute=False):
     """Fused forward/backward.  Accepts the 1-D (xq [b,h,r,l,d]) and the 2-D (xq [b,h,r,_n,_c,d]) layouts;
     the result has xq's shape.  prune=True skips (key, query) pairs whose softmax weight is provably below 2^-48
-    because of the accumulated decay: same results to float32 rounding, less work on long sequences."""
-    O, lse = _FusedUniversalAttention.apply(kc, vc, xq, static_src, static_dest, prune)
+    because of the accumulated decay: same results to float32 rounding, less work on long sequences.
+    recompute=True (bf16): the backward keeps its workspace at O(L*L/16) bytes per head by recomputing the score and
+    decay gradients in its second kernel instead of exchanging them through 2*L*L bytes per head (UA_FLAG_RECOMPUTE)."""
+    O, lse = _FusedUniversalAttention.apply(kc, vc, xq, static_src, static_dest, prune, recompute)
     return (O, lse) if return_lse else O
 
 
