@@ -76,6 +76,7 @@ __device__ __forceinline__ void issue_row(void* lds_base, const void* src_lane) 
 //   C[z][t16][s]    = sum_{u < 16*t16, u > s} log2(1 - A[s,u])        (t16 >= s/16 ... any t16 with 16*t16+15 >= s)
 //   Dsuf[z][t16][s] = sum_{t >= 16*(t16+1)} dBias[s,t]
 // ---------------------------------------------------------------------------------------------
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 struct TrueC { static constexpr bool value = true; };
 struct FalseC { static constexpr bool value = false; };
 
@@ -719,8 +720,8 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
       if constexpr (sizeof(T) == 2) {
         if (store_tiles) {     // the two halves of the operand are the two query tiles of the block
           char* p = reinterpret_cast<char*>(a.dS_st) + (((long)zk * R + r) * nT16 + 2 * tb) * st_row + st_lane;
-          __builtin_nontemporal_store(reinterpret_cast<const uint2*>(&bs)[0], reinterpret_cast<uint2*>(p));
-          __builtin_nontemporal_store(reinterpret_cast<const uint2*>(&bs)[1], reinterpret_cast<uint2*>(p + st_row));
+          __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&bs)[0], reinterpret_cast<u32x2*>(p));
+          __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&bs)[1], reinterpret_cast<u32x2*>(p + st_row));
         }
       }
 #pragma unroll
@@ -754,8 +755,8 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
       if constexpr (sizeof(T) == 2) {
         if (store_tiles) {
           char* p = reinterpret_cast<char*>(a.dG_st) + ((long)zk * nT16 + 2 * tb) * st_row + st_lane;
-          __builtin_nontemporal_store(reinterpret_cast<const uint2*>(&b)[0], reinterpret_cast<uint2*>(p));
-          __builtin_nontemporal_store(reinterpret_cast<const uint2*>(&b)[1], reinterpret_cast<uint2*>(p + st_row));
+          __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&b)[0], reinterpret_cast<u32x2*>(p));
+          __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&b)[1], reinterpret_cast<u32x2*>(p + st_row));
         }
       }
 #pragma unroll
