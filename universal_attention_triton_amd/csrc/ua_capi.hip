@@ -34,7 +34,7 @@ struct Layout {
   int D, Lp, nT, nch, Zk, Zq;
   size_t esz;
   // forward state
-  size_t Kp, KT, Vp, VT, Qp, QT, lsrc, ldest, C, lse2, knorm2, qnorm2, reach, minkey, fwd_end;
+  size_t Kp, KT, Vp, VT, Qp, QT, lsrc, ldest, C, lse2, knorm2, qnorm2, reach, minkey, Bt, fwd_end;
   // backward scratch
   size_t dOp, dOT, delta, dQacc, dKdacc, Dsuf, dKrow, dVrow, dsrc_raw, masked_nz, dS_st, dG_st, total;
   bool tiles;     // the backward exchanges dS / dG tiles between its two kernels
@@ -75,6 +75,11 @@ Layout make_layout(const ua_desc& d, bool chunked) {
   // pruning state of the fused mode: largest squared row norm of every 32-row block of K and Q, reach of every key
   // tile, first key tile reaching every query block
   l.knorm2 = take((size_t)l.Zk * (l.nT / 2) * 4); l.qnorm2 = take((size_t)l.Zq * (l.nT / 2) * 4); l.reach = take((size_t)l.Zk * l.nT * 4); l.minkey = take((size_t)l.Zk * (l.nT / 2) * 4);
+  // bf16 fused operator: the kernels exchange tiles through the workspace instead of recomputing them (fp16 bias of every
+  // (16 keys, 32 queries) tile here; score and decay gradients in the backward part), 1 KB per tile, full square
+  l.tiles = !chunked && d.dtype == UA_BF16 && !(d.flags & UA_FLAG_RECOMPUTE);
+  const size_t sq = (size_t)l.nT * (l.Lp / 32) * 1024;
+  l.Bt = l.tiles ? take((size_t)l.Zk * sq) : 0;
   l.fwd_end = off;
   const size_t gbytes = (size_t)l.Zq * l.nch * l.Lp * l.D * l.esz;
   l.dOp = take(gbytes); l.dOT = take(gbytes);
@@ -86,9 +91,7 @@ Layout make_layout(const ua_desc& d, bool chunked) {
   l.dKdacc = take((size_t)(atomics ? l.Zk : l.Zq) * l.Lp * l.D * 4);   // one slice per query group without atomics
   l.Dsuf = atomics ? 0 : take((size_t)l.Zk * l.nT * l.Lp * 4);
   l.masked_nz = take(256);
-  // bf16 fused backward: score and decay gradients of every (32 keys, 16 queries) tile, 1 KB each, full square
-  l.tiles = !chunked && d.dtype == UA_BF16 && !(d.flags & UA_FLAG_RECOMPUTE);
-  const size_t sq = (size_t)l.nT * (l.Lp / 32) * 1024;
+  // score and decay gradients of every (32 keys, 16 queries) tile
   l.dS_st = l.tiles ? take((size_t)l.Zq * sq) : 0;
   l.dG_st = l.tiles ? take((size_t)l.Zk * sq) : 0;
   l.dKrow = take((size_t)l.Zk * l.Lp * l.D * 4);
@@ -242,12 +245,14 @@ int run_fused_fwd_kernels(const ua_desc& d, const Layout& l, char* ws, void* O, 
     UA_PROF("k_carry", s);
     UA_HIP(ua::launch_carry(d.dtype, l.D, ws + l.Kp, (const float*)(ws + l.lsrc), (const float*)(ws + l.ldest),
                             (float*)(ws + l.C), l.Lp, l.Zk, 1, (d.flags & UA_FLAG_PRUNE) ? (const float*)(ws + l.knorm2) : nullptr,
-                            (const float*)(ws + l.qnorm2), d.r, (int*)(ws + l.reach), (int*)(ws + l.minkey), s));
+                            (const float*)(ws + l.qnorm2), d.r, (int*)(ws + l.reach), (int*)(ws + l.minkey), s,
+                            l.tiles ? ws + l.Bt : nullptr));
   }
   UA_PROF("k_fwd_fused", s);
   UA_HIP(ua::launch_fwd_fused(d.dtype, l.D, variant, ws + l.Qp, ws + l.Kp, ws + l.VT, (const float*)(ws + l.lsrc),
                               (const float*)(ws + l.ldest), (const float*)(ws + l.C), O, lse, (float*)(ws + l.lse2),
-                              (const int*)(ws + l.reach), (const int*)(ws + l.minkey), d.r, d.L, l.Lp, d.d, l.Zq, s));
+                              (const int*)(ws + l.reach), (const int*)(ws + l.minkey), d.r, d.L, l.Lp, d.d, l.Zq, s,
+                              l.tiles ? ws + l.Bt : nullptr));
   return UA_OK;
 }
 
@@ -290,7 +295,7 @@ int run_bwd_common(const ua_desc& d, const Layout& l, char* ws, bool chunked, co
   a.dKrow = (float*)(ws + l.dKrow);
   a.dVrow = (float*)(ws + l.dVrow); a.dsrc_raw = (float*)(ws + l.dsrc_raw);
   a.masked_nz = (const int*)(ws + l.masked_nz);
-  a.dS_st = l.tiles ? ws + l.dS_st : nullptr; a.dG_st = l.tiles ? ws + l.dG_st : nullptr;
+  a.dS_st = l.tiles ? ws + l.dS_st : nullptr; a.dG_st = l.tiles ? ws + l.dG_st : nullptr; a.Bt = l.tiles ? ws + l.Bt : nullptr;
   a.R = d.r; a.L = d.L; a.Lp = l.Lp; a.c = is_chunked ? d.chunk : 128; a.nch = l.nch; a.chunked = is_chunked ? 1 : 0;
   a.skip_masked = (d.flags & UA_FLAG_SKIP_MASKED) ? 1 : 0;
   a.split_r = (!chunked && d.r > 1) ? 1 : 0;
@@ -350,7 +355,8 @@ int ua_fused_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, cons
     if (int e = pack_inputs(d, l, false, kc, vc, xq, static_src, static_dest, w, s)) return e;
     UA_HIP(ua::launch_carry(d.dtype, l.D, w + l.Kp, (const float*)(w + l.lsrc), (const float*)(w + l.ldest),
                             (float*)(w + l.C), l.Lp, l.Zk, 1, (d.flags & UA_FLAG_PRUNE) ? (const float*)(w + l.knorm2) : nullptr,
-                            (const float*)(w + l.qnorm2), d.r, (int*)(w + l.reach), (int*)(w + l.minkey), s));
+                            (const float*)(w + l.qnorm2), d.r, (int*)(w + l.reach), (int*)(w + l.minkey), s,
+                            l.tiles ? w + l.Bt : nullptr));
   }
   const long rowsz = (long)d.L * d.d;
   const ua::RowsView Ov = contiguous_view(O, rowsz, d.d), dOv = contiguous_view(dO, rowsz, d.d);

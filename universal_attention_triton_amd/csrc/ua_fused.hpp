@@ -87,11 +87,17 @@ struct FalseC { static constexpr bool value = false; };
 // cannot contribute a softmax weight above 2^-kPruneLog2 to any later query (the bias only decreases, a score
 // is at most max|k| max|q|, and a query's normaliser is at least its own score); a wave stops once all its 16
 // keys are there and records the last 32-query block it reached in reach[z][key tile].
-template <class T, int D, int NST, bool CM>
+// BO: instead of the carries C, leave the bias of every visited (16 keys, 32 queries) tile itself, as fp16, in
+// Bt[z][Lp/32 query blocks][Lp/16 key tiles][1 KB]: lane l of the key tile's wave owns bytes 16 l .. 16 l + 15 = its
+// key's bias towards queries 4g..4g+3 of the block's first 16-query tile, then of the second (g = l / 16).  The
+// 16-bit forward and backward kernels then read the bias instead of recomputing the affinity chain; fp16 resolves
+// the bias of every pair that carries weight (|bias| < 16: 2^-7 at worst) to better than the bf16 rounding of the
+// softmax weight itself.
+template <class T, int D, int NST, bool CM, bool BO>
 __global__ void __launch_bounds__(512) k_carry2(const T* __restrict__ Kp, const float* __restrict__ lsrc,
                                                 const float* __restrict__ ldest, float* __restrict__ C, int Lp,
                                                 const float* __restrict__ knorm2, const float* __restrict__ qnorm2, int R,
-                                                int* __restrict__ reach) {
+                                                int* __restrict__ reach, _Float16* __restrict__ Bt) {
   using TN = Tile<T, 32, D, CM>;
   constexpr int NK = D / 32, SB = TN::BYTES + 1024;   // tile + [ldest of the block: 32 floats]
   UA_STAGES(SB);
@@ -168,14 +174,25 @@ __global__ void __launch_bounds__(512) k_carry2(const T* __restrict__ Kp, const 
         x[i][v] = l2;
       }
     }
-    float b0, a0, t0, b1, a1, t1;
-    group_scan((x[0][0] + x[0][1]) + (x[0][2] + x[0][3]), gm, b0, a0, t0);
-    group_scan((x[1][0] + x[1][1]) + (x[1][2] + x[1][3]), gm, b1, a1, t1);
-    if (g == 0) {
-      Cz[(long)(2 * tb) * Lp] = carry;
-      Cz[(long)(2 * tb + 1) * Lp] = carry + t0;
+    if constexpr (BO) {
+      const float tot = prefix32(x[0], x[1], gm);
+      typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+      f16x8 hb;
+#pragma unroll
+      for (int v = 0; v < 4; ++v) { hb[v] = (_Float16)(x[0][v] + carry); hb[4 + v] = (_Float16)(x[1][v] + carry); }
+      char* dst = reinterpret_cast<char*>(Bt) + ((((long)z * nT + tb) * nT16 + sb16) << 10) + 16 * lane;
+      __builtin_nontemporal_store(hb, reinterpret_cast<f16x8*>(dst));
+      carry += tot;
+    } else {
+      float b0, a0, t0, b1, a1, t1;
+      group_scan((x[0][0] + x[0][1]) + (x[0][2] + x[0][3]), gm, b0, a0, t0);
+      group_scan((x[1][0] + x[1][1]) + (x[1][2] + x[1][3]), gm, b1, a1, t1);
+      if (g == 0) {
+        Cz[(long)(2 * tb) * Lp] = carry;
+        Cz[(long)(2 * tb + 1) * Lp] = carry + t0;
+      }
+      carry += t0 + t1;
     }
-    carry += t0 + t1;
   };
   {
     // segments of 16 blocks, so that the workgroup can leave once all its waves have stopped
@@ -291,18 +308,24 @@ __global__ void __launch_bounds__(256) k_chunk_masked_denom(T* __restrict__ deno
 // ---------------------------------------------------------------------------------------------
 // CHUNKED: the reference's chunked operator instead of the merged one: the softmax restarts at every chunk of
 // co.c keys (a multiple of 64) and each chunk's result goes to out[.., i] / denom[.., i] / lse2[zq*nch + i][t].
-template <class T, int D, int NST, int NW, bool CHUNKED>
+// BI (8 waves): the decay bias comes from the fp16 tiles k_carry2<BO> left in Bt instead of being recomputed (no key-key
+// product, no affinity chain, no scan).  The two waves that share a 32-query block copy its four key tiles (two each)
+// into one LDS region per step.
+template <class T, int D, int NST, int NW, bool CHUNKED, bool BI = false>
 __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW >= 8 ? NW / 4 : 2, NW >= 8 ? NW / 4 : 2))) k_fwd_fused2(const T* __restrict__ Qp, const T* __restrict__ Kp,
                                                     const T* __restrict__ VT, const float* __restrict__ lsrc,
                                                     const float* __restrict__ ldest, const float* __restrict__ C,
                                                     T* __restrict__ O, float* __restrict__ lse, float* __restrict__ lse2,
                                                     const int* __restrict__ reach, const int* __restrict__ minkey,
-                                                    int R, int L, int Lp, int d, ChunkOut<T> co) {
+                                                    int R, int L, int Lp, int d, ChunkOut<T> co,
+                                                    const _Float16* __restrict__ Bt = nullptr) {
+  static_assert(!BI || (NW == 8 && !CHUNKED), "bias tiles: 8 waves, merged operator");
   using TN = Tile<T, 32, D>;
   using TT = Tile<T, D, 32>;
   constexpr int NK = D / 32, ND = D / 16;
   using ST = StageT<T>;
-  constexpr int TILES = 2 * TN::BYTES + 2 * TT::BYTES, SB = TILES + NW * 1024;   // + per wave [C row: 64f][lsrc: 64f]
+  // + per wave [C row: 64f][lsrc: 64f][reach], or (BI) per pair of waves 4 bias tiles of 1 KB, then one reach row
+  constexpr int TILES = 2 * TN::BYTES + 2 * TT::BYTES, SB = TILES + (BI ? NW * 2048 + 1024 : NW * 1024);
   UA_STAGES(SB);
   __shared__ __attribute__((aligned(256))) char sPbuf[NW * 2 * ST::BYTES];
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
@@ -327,10 +350,11 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW
 #pragma unroll
     for (int q = 0; q < NK; ++q) {
       qf[q] = ld8(Qp + nat_off<D>(zq, Lp, 16 * tq + col, 32 * q + 8 * g));
-      kf[q] = ld8(Kp + nat_off<D>(zk, Lp, 16 * tq + col, 32 * q + 8 * g));
+      if (!BI) kf[q] = ld8(Kp + nat_off<D>(zk, Lp, 16 * tq + col, 32 * q + 8 * g));
     }
   }
-  const f32x4 lb = load_t4(ldest + (long)zk * Lp + 16 * tq, g);
+  f32x4 lb = {0, 0, 0, 0};
+  if (!BI) lb = load_t4(ldest + (long)zk * Lp + 16 * tq, g);
   f32x4 o[ND];
 #pragma unroll
   for (int n = 0; n < ND; ++n) o[n] = (f32x4){0, 0, 0, 0};
@@ -351,6 +375,8 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW
   if (lane < 16) row_base = C + ((long)zk * nT16 + tq) * Lp + 4 * lane;
   else if (lane < 32) row_base = lsrc + (long)zk * Lp + 4 * (lane - 16);
   else { row_base = reinterpret_cast<const float*>(reach + zk * nT16); row_step = 4; }
+  // BI: this lane's 16 bytes of key tile 0 of the wave's query block
+  const char* bt_src = reinterpret_cast<const char*>(Bt) + ((((long)zk * (Lp >> 5) + tbq) * nT16) << 10) + 16 * lane;
 
 #define UA_ISSUE(s, base)                                                                   \
   {                                                                                         \
@@ -359,7 +385,15 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW
     stN.issue((base) + TN::BYTES, Kz + (long)(64 * kt_ + 32) * D, w);                       \
     stT.issue((base) + 2 * TN::BYTES, Vz + (long)(2 * kt_) * (32 * D), w);                  \
     stT.issue((base) + 2 * TN::BYTES + TT::BYTES, Vz + (long)(2 * kt_ + 1) * (32 * D), w);  \
-    issue_row((base) + TILES + w * 1024, row_base + (long)kt_ * row_step);                  \
+    if (BI) {                                                                               \
+      const char* src_ = bt_src + ((long)(4 * kt_ + 2 * (w & 1)) << 10);                    \
+      char* dst_ = (base) + TILES + (w >> 1) * 4096 + (w & 1) * 2048;                       \
+      issue_row(dst_, src_);                                                                \
+      issue_row(dst_ + 1024, src_ + 1024);                                                  \
+      if (w == 0) issue_row((base) + TILES + NW * 2048, reach + zk * nT16 + 4 * kt_);        \
+    } else {                                                                                \
+      issue_row((base) + TILES + w * 1024, row_base + (long)kt_ * row_step);                \
+    }                                                                                       \
   }
 #define UA_COMPUTE_FAST(s, base) fwd_tile(n_kt - 1 - (s), (base), FalseC())
 #define UA_COMPUTE_SLOW(s, base) fwd_tile(n_kt - 1 - (s), (base), TrueC())
@@ -413,7 +447,24 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW
     for (int j = 0; j < 4; ++j) {
       const int sbk = 4 * kt + j;                      // 16-key tile
       const T* sK = reinterpret_cast<const T*>(base + (j >> 1) * TN::BYTES);
-      if (!MASKED || sbk <= tq) {
+      if constexpr (BI) {
+        if (!MASKED || sbk <= tq) {
+          f32x4 sc = {0, 0, 0, 0};
+#pragma unroll
+          for (int q = 0; q < NK; ++q) mma16(sc, qf[q], ld8(sK + TN::at(j & 1, col, q, g)));
+          typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+          const f16x4 hb = *reinterpret_cast<const f16x4*>(base + TILES + (w >> 1) * 4096 + j * 1024 + 16 * lane + 8 * (w & 1));
+          const bool in_reach = reinterpret_cast<const int*>(base + TILES + NW * 2048)[j] >= tbq;
+          const bool diag = MASKED && (sbk == tq);
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            const float x = in_reach ? __builtin_fmaf(sc[v], kLog2e, (float)hb[v]) : -1.0e30f;
+            s2[j][v] = (MASKED && diag && 4 * g + v < col) ? -1.0e30f : x;
+          }
+        } else {
+          s2[j] = (f32x4){-1.0e30f, -1.0e30f, -1.0e30f, -1.0e30f};
+        }
+      } else if (!MASKED || sbk <= tq) {
         const float c = reinterpret_cast<const int*>(stats)[128 + j] >= tbq ? stats[16 * j + col] : -1.0e30f;
         const float la = stats[64 + 16 * j + col];
         f32x4 gt = {0, 0, 0, 0}, sc = {0, 0, 0, 0};
@@ -524,12 +575,16 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW
 // ---------------------------------------------------------------------------------------------
 // CH: chunked operator (a.c a multiple of 64): the upstream gradient, delta and the normaliser depend on the key's chunk
 // (z index zq*nch + chunk); the 128 keys of a workgroup lie in at most two chunks, whose dO tiles are both staged.
-template <class T, int D, int NST, bool MR, bool CH>
+// TO (16-bit dtypes): leave the score gradient dS and the decay gradient dG of every visited tile, in operand precision,
+// in a.dS_st / a.dG_st for k_bwd_queries3 (which then needs no suffix carries Dsuf).
+template <class T, int D, int NST, bool MR, bool CH, bool TO>
 __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   using TN = Tile<T, 32, D>;
   using TT = Tile<T, D, 32>;
   constexpr int NK = D / 32, ND = D / 16;
-  constexpr int TILES = (CH ? 4 : 3) * (TN::BYTES + TT::BYTES), SB = TILES + (CH ? 2048 : 1024);
+  static_assert(!TO || !CH, "tile exchange is for the merged operator");
+  // TO: the bias comes from the fp16 tiles of k_carry2<BO> (a.Bt), one 1 KB tile per wave and step after the stats row
+  constexpr int TILES = (CH ? 4 : 3) * (TN::BYTES + TT::BYTES), SB = TILES + (CH ? 2048 : 1024) + (TO ? 8 * 1024 : 0);
   // tiles of a stage: Kt, Q, dO | KT, QT, dOT | (CH) dO, dOT of the workgroup's second chunk
   // stats row of a stage: [lse2: 32f][delta: 32f][ldest: 32f][unused: 32f][forward carries of the 128 keys: 128f]
   // (CH) followed by [lse2: 32f][delta: 32f] of the second chunk
@@ -586,7 +641,9 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   const float* Cz = a.C + (long)zk * nT16 * Lp + 128 * kg;
   float* Dz = a.Dsuf + (long)zk * nT16 * Lp + spos;
   // where this lane's four values of a (16 keys, 16 queries) tile go inside the 1 KB tile of its 32-key half
-  const bool store_tiles = sizeof(T) == 2 && a.dS_st != nullptr;
+  static_assert(!TO || sizeof(T) == 2, "tiles are exchanged in 16-bit operand precision");
+  // this lane's 16 bytes of the wave's bias tile of query block 0
+  const char* bt_src = reinterpret_cast<const char*>(a.Bt) + ((((long)zk * (Lp >> 5)) * nT16 + sb16) << 10) + 16 * lane;
   const long st_row = (long)(Lp >> 5) << 10;                       // bytes between consecutive 16-query tiles
   const long st_lane = ((long)(sb16 >> 1) << 10) + StageT<bf16>::addr(perm32(16 * (sb16 & 1) + col), 8 * g);
 
@@ -611,6 +668,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
       else src_ = Cz + (long)(2 * tb_) * Lp + 4 * (lane - 32);                              \
       issue_row((base) + TILES, src_);                                                      \
     }                                                                                       \
+    if (TO) issue_row((base) + TILES + 1024 + w * 1024, bt_src + ((long)tb_ * nT16 << 10)); \
     if (CH && two) {                                                                        \
       stN.issue((base) + 3 * TN::BYTES + 3 * TT::BYTES, a.dOp + go_ + (long)Lp * D, w);     \
       stT.issue((base) + 4 * TN::BYTES + 3 * TT::BYTES, a.dOT + go_ + (long)Lp * D, w);     \
@@ -677,7 +735,9 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
     f32x4 (&dB)[2] = MR ? dB_s : dB_l;
     const int tl0 = 32 * tb + 4 * g - spos;        // query position minus key position for (tile 0, v = 0)
     if (!MR || r == 0) {
-      const float cin = stats[128 + 16 * w + col];
+      typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+      f16x8 hb;
+      if constexpr (TO) hb = *reinterpret_cast<const f16x8*>(base + TILES + 1024 + w * 1024 + 16 * lane);
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         f32x4 acc = {0, 0, 0, 0};
@@ -688,15 +748,23 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
         for (int v = 0; v < 4; ++v) {
           gk[i][v] = fmaxf(acc[v], 0.f);
           aff[i][v] = affinity(__builtin_amdgcn_logf(gk[i][v]), lab[v] + la);
-          const float l2 = log2_one_minus(aff[i][v]);
-          bias[i][v] = (MASKED && diag && tl0 + 16 * i + v <= 0) ? 0.f : l2;
+          if constexpr (TO) {
+            bias[i][v] = (float)hb[4 * i + v];
+          } else {
+            const float l2 = log2_one_minus(aff[i][v]);
+            bias[i][v] = (MASKED && diag && tl0 + 16 * i + v <= 0) ? 0.f : l2;
+          }
+          if (MR) dB[i][v] = 0.f;
         }
       }
-      prefix32(bias[0], bias[1], gm);
+      if constexpr (!TO) {
+        const float cin = stats[128 + 16 * w + col];
+        prefix32(bias[0], bias[1], gm);
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) { bias[i][v] += cin; if (MR) dB[i][v] = 0.f; }
+          for (int v = 0; v < 4; ++v) bias[i][v] += cin;
+      }
     }
     {
       f32x4 P[2], dS[2];
@@ -717,12 +785,10 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
         }
       }
       const Frag<T> bp = as_operand16<T>(P[0], P[1]), bs = as_operand16<T>(dS[0], dS[1]);
-      if constexpr (sizeof(T) == 2) {
-        if (store_tiles) {     // the two halves of the operand are the two query tiles of the block
-          char* p = reinterpret_cast<char*>(a.dS_st) + (((long)zk * R + r) * nT16 + 2 * tb) * st_row + st_lane;
-          __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&bs)[0], reinterpret_cast<u32x2*>(p));
-          __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&bs)[1], reinterpret_cast<u32x2*>(p + st_row));
-        }
+      if constexpr (TO) {     // the two halves of the operand are the two query tiles of the block
+        char* p = reinterpret_cast<char*>(a.dS_st) + (((long)zk * R + r) * nT16 + 2 * tb) * st_row + st_lane;
+        __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&bs)[0], reinterpret_cast<u32x2*>(p));
+        __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&bs)[1], reinterpret_cast<u32x2*>(p + st_row));
       }
 #pragma unroll
       for (int n = 0; n < ND; ++n) mma16(dVt[n], ld8(sdOT + TT::at(n, col, 0, g)), bp);
@@ -736,7 +802,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
     if (!MR || r == R - 1) {
       float t1;
       const float tot = suffix32(dB[0], dB[1], gm, t1);
-      if (g == 0) {
+      if (!TO && g == 0) {
         Dz[(long)(2 * tb + 1) * Lp] = dcar;
         Dz[(long)(2 * tb) * Lp] = dcar + t1;
       }
@@ -752,12 +818,10 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
       }
       dcar += tot;
       const Frag<T> b = as_operand16<T>(dB[0], dB[1]);
-      if constexpr (sizeof(T) == 2) {
-        if (store_tiles) {
-          char* p = reinterpret_cast<char*>(a.dG_st) + ((long)zk * nT16 + 2 * tb) * st_row + st_lane;
-          __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&b)[0], reinterpret_cast<u32x2*>(p));
-          __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&b)[1], reinterpret_cast<u32x2*>(p + st_row));
-        }
+      if constexpr (TO) {
+        char* p = reinterpret_cast<char*>(a.dG_st) + ((long)zk * nT16 + 2 * tb) * st_row + st_lane;
+        __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&b)[0], reinterpret_cast<u32x2*>(p));
+        __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&b)[1], reinterpret_cast<u32x2*>(p + st_row));
       }
 #pragma unroll
       for (int n = 0; n < ND; ++n) mma16(dKt[n], ld8(sKT + TT::at(n, col, 0, g)), b);

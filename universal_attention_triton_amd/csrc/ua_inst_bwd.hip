@@ -12,7 +12,7 @@ static BwdArgs<T> typed(const BwdArgsV& v) {
   a.Kp = (const T*)v.Kp; a.Vp = (const T*)v.Vp; a.KT = (const T*)v.KT; a.Qp = (const T*)v.Qp; a.QT = (const T*)v.QT;
   a.dOp = (const T*)v.dOp; a.dOT = (const T*)v.dOT; a.lsrc = v.lsrc; a.ldest = v.ldest; a.lse2 = v.lse2; a.delta = v.delta;
   a.C = v.C;
-  a.dS_st = (T*)v.dS_st; a.dG_st = (T*)v.dG_st;
+  a.dS_st = (T*)v.dS_st; a.dG_st = (T*)v.dG_st; a.Bt = (const _Float16*)v.Bt;
   a.dQacc = v.dQacc; a.dKdacc = v.dKdacc; a.Dsuf = v.Dsuf; a.dKrow = v.dKrow; a.dVrow = v.dVrow; a.dsrc_raw = v.dsrc_raw;
   a.R = v.R; a.L = v.L; a.Lp = v.Lp; a.c = v.c; a.nch = v.nch; a.chunked = v.chunked; a.skip_masked = v.skip_masked; a.split_r = v.split_r;
   return a;
@@ -29,24 +29,32 @@ static hipError_t bwd_t(const BwdArgsV& v, int Zk, hipStream_t s) {
   return hipGetLastError();
 }
 // explicit instantiations (the implicit ones are not emitted on the host side for kernels holding lambdas)
-#define UA_INST(T, D, NST)                                                   \
-  template __global__ void k_bwd_keys2<T, D, NST, false, false>(BwdArgs<T>); \
-  template __global__ void k_bwd_keys2<T, D, NST, true, false>(BwdArgs<T>);  \
-  template __global__ void k_bwd_keys2<T, D, NST, false, true>(BwdArgs<T>);  \
-  template __global__ void k_bwd_keys2<T, D, NST, true, true>(BwdArgs<T>);
+#define UA_INST(T, D, NST)                                                          \
+  template __global__ void k_bwd_keys2<T, D, NST, false, false, false>(BwdArgs<T>); \
+  template __global__ void k_bwd_keys2<T, D, NST, true, false, false>(BwdArgs<T>);  \
+  template __global__ void k_bwd_keys2<T, D, NST, false, true, false>(BwdArgs<T>);  \
+  template __global__ void k_bwd_keys2<T, D, NST, true, true, false>(BwdArgs<T>);
 UA_INST(bf16, 64, 2) UA_INST(bf16, 128, 2) UA_INST(float, 64, 1) UA_INST(float, 128, 1)
 #undef UA_INST
+template __global__ void k_bwd_keys2<bf16, 64, 2, false, false, true>(BwdArgs<bf16>);
+template __global__ void k_bwd_keys2<bf16, 64, 2, true, false, true>(BwdArgs<bf16>);
+template __global__ void k_bwd_keys2<bf16, 128, 2, false, false, true>(BwdArgs<bf16>);
+template __global__ void k_bwd_keys2<bf16, 128, 2, true, false, true>(BwdArgs<bf16>);
 
-template <class T, int D, int NST, bool MR, bool CH>
+template <class T, int D, int NST, bool MR, bool CH, bool TO>
 static hipError_t bwd2_mr(const BwdArgs<T>& a, int Lp, int Zk, hipStream_t s) {
-  hipLaunchKernelGGL((k_bwd_keys2<T, D, NST, MR, CH>), dim3(Lp / 128, Zk), dim3(512), 0, s, a);
+  hipLaunchKernelGGL((k_bwd_keys2<T, D, NST, MR, CH, TO>), dim3(Lp / 128, Zk), dim3(512), 0, s, a);
   return hipGetLastError();
 }
 template <class T, int D, int NST>
 static hipError_t bwd2_t(const BwdArgsV& v, int Zk, hipStream_t s) {
   const BwdArgs<T> a = typed<T>(v);
-  if (v.chunked) return v.R > 1 ? bwd2_mr<T, D, NST, true, true>(a, v.Lp, Zk, s) : bwd2_mr<T, D, NST, false, true>(a, v.Lp, Zk, s);
-  return v.R > 1 ? bwd2_mr<T, D, NST, true, false>(a, v.Lp, Zk, s) : bwd2_mr<T, D, NST, false, false>(a, v.Lp, Zk, s);
+  if constexpr (sizeof(T) == 2) {
+    if (v.dS_st && !v.chunked)
+      return v.R > 1 ? bwd2_mr<T, D, NST, true, false, true>(a, v.Lp, Zk, s) : bwd2_mr<T, D, NST, false, false, true>(a, v.Lp, Zk, s);
+  }
+  if (v.chunked) return v.R > 1 ? bwd2_mr<T, D, NST, true, true, false>(a, v.Lp, Zk, s) : bwd2_mr<T, D, NST, false, true, false>(a, v.Lp, Zk, s);
+  return v.R > 1 ? bwd2_mr<T, D, NST, true, false, false>(a, v.Lp, Zk, s) : bwd2_mr<T, D, NST, false, false, false>(a, v.Lp, Zk, s);
 }
 template <class T, int D>
 static hipError_t bwd_nw(const BwdArgsV& v, int Zk, int cols, hipStream_t s) {

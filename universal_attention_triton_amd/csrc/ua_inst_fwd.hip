@@ -14,10 +14,12 @@ static void allow_lds(K kernel, size_t bytes) {
 
 template <class T, int D>
 static hipError_t carry_t(const void* Kp, const float* lsrc, const float* ldest, float* C, int Lp, int Zk, int tiled,
-                          const float* knorm2, const float* qnorm2, int R, int* reach, int* minkey, hipStream_t s) {
+                          const float* knorm2, const float* qnorm2, int R, int* reach, int* minkey, hipStream_t s, void* Bt) {
   constexpr int NST = 2;
-  if (tiled) hipLaunchKernelGGL((k_carry2<T, D, NST, true>), dim3(Lp / 128, Zk), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, C, Lp, knorm2, qnorm2, R, reach);
-  else hipLaunchKernelGGL((k_carry2<T, D, NST, false>), dim3(Lp / 128, Zk), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, C, Lp, knorm2, qnorm2, R, reach);
+  _Float16* none = nullptr;
+  if (tiled && Bt && sizeof(T) == 2) hipLaunchKernelGGL((k_carry2<T, D, NST, true, true>), dim3(Lp / 128, Zk), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, C, Lp, knorm2, qnorm2, R, reach, (_Float16*)Bt);
+  else if (tiled) hipLaunchKernelGGL((k_carry2<T, D, NST, true, false>), dim3(Lp / 128, Zk), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, C, Lp, knorm2, qnorm2, R, reach, none);
+  else hipLaunchKernelGGL((k_carry2<T, D, NST, false, false>), dim3(Lp / 128, Zk), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, C, Lp, knorm2, qnorm2, R, reach, none);
   hipError_t e = hipGetLastError();
   if (e == hipSuccess && reach && minkey) {
     hipLaunchKernelGGL((k_minkey<>), dim3((Lp / 32 + 255) / 256, Zk), dim3(256), 0, s, (const int*)reach, minkey, Lp / 16);
@@ -26,30 +28,45 @@ static hipError_t carry_t(const void* Kp, const float* lsrc, const float* ldest,
   return e;
 }
 hipError_t launch_carry(int dtype, int D, const void* Kp, const float* lsrc, const float* ldest, float* C, int Lp, int Zk,
-                        int tiled, const float* knorm2, const float* qnorm2, int R, int* reach, int* minkey, hipStream_t s) {
-#define UA_ARGS Kp, lsrc, ldest, C, Lp, Zk, tiled, knorm2, qnorm2, R, reach, minkey, s
+                        int tiled, const float* knorm2, const float* qnorm2, int R, int* reach, int* minkey, hipStream_t s,
+                        void* Bt) {
+#define UA_ARGS Kp, lsrc, ldest, C, Lp, Zk, tiled, knorm2, qnorm2, R, reach, minkey, s, Bt
   if (dtype == 1) return D == 64 ? carry_t<bf16, 64>(UA_ARGS) : carry_t<bf16, 128>(UA_ARGS);
   return D == 64 ? carry_t<float, 64>(UA_ARGS) : carry_t<float, 128>(UA_ARGS);
 #undef UA_ARGS
 }
 
 // explicit instantiations (the implicit ones are not emitted on the host side for these kernels)
-#define UA_INST(T, D, NST, NW, CH)                                                                                    \
-  template __global__ void k_fwd_fused2<T, D, NST, NW, CH>(const T*, const T*, const T*, const float*, const float*,  \
-                                                           const float*, T*, float*, float*, const int*, const int*, \
-                                                           int, int, int, int, ChunkOut<T>);
+#define UA_INST2(T, D, NST, NW, CH, BI)                                                                                  \
+  template __global__ void k_fwd_fused2<T, D, NST, NW, CH, BI>(const T*, const T*, const T*, const float*, const float*, \
+                                                               const float*, T*, float*, float*, const int*, const int*, \
+                                                               int, int, int, int, ChunkOut<T>, const _Float16*);
+#define UA_INST(T, D, NST, NW, CH) UA_INST2(T, D, NST, NW, CH, false)
+UA_INST2(bf16, 64, 2, 8, false, true) UA_INST2(bf16, 128, 2, 8, false, true)
 UA_INST(bf16, 64, 1, 8, false) UA_INST(bf16, 64, 2, 8, false) UA_INST(bf16, 64, 2, 12, false) UA_INST(bf16, 64, 2, 16, false)
 UA_INST(bf16, 128, 2, 4, false) UA_INST(bf16, 64, 2, 4, false) UA_INST(bf16, 128, 1, 8, false) UA_INST(bf16, 128, 2, 8, false) UA_INST(bf16, 128, 2, 12, false) UA_INST(bf16, 128, 2, 16, false)
 UA_INST(float, 64, 1, 8, false) UA_INST(float, 128, 1, 8, false)
 UA_INST(bf16, 64, 2, 8, true) UA_INST(bf16, 128, 2, 8, true) UA_INST(float, 64, 1, 8, true) UA_INST(float, 128, 1, 8, true)
 #undef UA_INST
+#undef UA_INST2
 
 template <class T, int D, int NST, int NW>
 static hipError_t fused_t(const void* Qp, const void* Kp, const void* VT, const float* lsrc, const float* ldest,
                           const float* C, void* O, float* lse, float* lse2, const int* reach, const int* minkey, int R, int L,
                           int Lp, int d, int Zq, hipStream_t s) {
+  const _Float16* none = nullptr;
   hipLaunchKernelGGL((k_fwd_fused2<T, D, NST, NW, false>), dim3((Lp / 16 + NW - 1) / NW, Zq), dim3(64 * NW), 0, s, (const T*)Qp,
-                     (const T*)Kp, (const T*)VT, lsrc, ldest, C, (T*)O, lse, lse2, reach, minkey, R, L, Lp, d, ChunkOut<T>{});
+                     (const T*)Kp, (const T*)VT, lsrc, ldest, C, (T*)O, lse, lse2, reach, minkey, R, L, Lp, d, ChunkOut<T>{}, none);
+  return hipGetLastError();
+}
+// bf16 with bias tiles from launch_carry
+template <int D>
+static hipError_t fused_bi(const void* Qp, const void* Kp, const void* VT, const float* lsrc, const float* ldest,
+                           const float* C, void* O, float* lse, float* lse2, const int* reach, const int* minkey, int R, int L,
+                           int Lp, int d, int Zq, hipStream_t s, const void* Bt) {
+  using T = bf16;
+  hipLaunchKernelGGL((k_fwd_fused2<T, D, 2, 8, false, true>), dim3(Lp / 128, Zq), dim3(512), 0, s, (const T*)Qp, (const T*)Kp,
+                     (const T*)VT, lsrc, ldest, C, (T*)O, lse, lse2, reach, minkey, R, L, Lp, d, ChunkOut<T>{}, (const _Float16*)Bt);
   return hipGetLastError();
 }
 // variants (bf16): 0 = 8 waves, double-buffered stages; 1 = 8 waves, single stage; 2 = 12 waves; 3 = 16 waves
@@ -71,8 +88,10 @@ static hipError_t fused_v(int variant, const void* Qp, const void* Kp, const voi
 }
 hipError_t launch_fwd_fused(int dtype, int D, int variant, const void* Qp, const void* Kp, const void* VT,
                             const float* lsrc, const float* ldest, const float* C, void* O, float* lse, float* lse2,
-                            const int* reach, const int* minkey, int R, int L, int Lp, int d, int Zq, hipStream_t s) {
+                            const int* reach, const int* minkey, int R, int L, int Lp, int d, int Zq, hipStream_t s,
+                            const void* Bt) {
 #define UA_ARGS Qp, Kp, VT, lsrc, ldest, C, O, lse, lse2, reach, minkey, R, L, Lp, d, Zq, s
+  if (dtype == 1 && Bt) return D == 64 ? fused_bi<64>(UA_ARGS, Bt) : fused_bi<128>(UA_ARGS, Bt);
   if (dtype == 1) return D == 64 ? fused_v<bf16, 64>(variant, UA_ARGS) : fused_v<bf16, 128>(variant, UA_ARGS);
   return D == 64 ? fused_t<float, 64, 1, 8>(UA_ARGS) : fused_t<float, 128, 1, 8>(UA_ARGS);
 #undef UA_ARGS
@@ -88,7 +107,7 @@ static hipError_t chunked2_t(const void* Qp, const void* Kp, const void* Vp, con
   const int ovec = out && o_sd == 1 && d % VV == 0 && (uintptr_t)out % 16 == 0 && o_sz % VV == 0 && o_st % VV == 0 && o_si % VV == 0;
   ChunkOut<T> co{(T*)out, (T*)denom, o_sz, o_st, o_sd, o_si, c, nch, ovec};
   hipLaunchKernelGGL((k_fwd_fused2<T, D, NST, NW, true>), dim3((Lp / 16 + NW - 1) / NW, Zq), dim3(64 * NW), 0, s, (const T*)Qp,
-                     (const T*)Kp, (const T*)VT, lsrc, ldest, C, (T*)nullptr, (float*)nullptr, lse2, reach, minkey, R, L, Lp, d, co);
+                     (const T*)Kp, (const T*)VT, lsrc, ldest, C, (T*)nullptr, (float*)nullptr, lse2, reach, minkey, R, L, Lp, d, co, (const _Float16*)nullptr);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
   if (out && nch > 1) {

@@ -13,6 +13,7 @@ struct BwdArgsV {
   const float *lsrc, *ldest, *lse2, *delta, *C;
   float *dQacc, *dKdacc, *Dsuf, *dKrow, *dVrow, *dsrc_raw;
   void *dS_st, *dG_st;
+  const void* Bt;
   int R, L, Lp, c, nch, chunked, skip_masked, split_r;
 };
 
@@ -20,12 +21,15 @@ struct BwdArgsV {
 // tiled: Kp is stored in tiles of 32 keys, k-group-major (fused mode) instead of row-major (chunked mode)
 // knorm2 [Zk][Lp/32], qnorm2 [Zk*R][Lp/32] (optional): largest squared row norm of every block of 32 keys / queries,
 // enables pruning; reach (optional): [Zk][Lp/16] out.  With reach given, minkey [Zk][Lp/32] is filled as well.
+// Bt (optional, bf16 + tiled): fp16 bias tiles [Zk][Lp/32][Lp/16][1 KB] are written instead of the carries C
 hipError_t launch_carry(int dtype, int D, const void* Kp, const float* lsrc, const float* ldest, float* C, int Lp, int Zk,
-                        int tiled, const float* knorm2, const float* qnorm2, int R, int* reach, int* minkey, hipStream_t s);
+                        int tiled, const float* knorm2, const float* qnorm2, int R, int* reach, int* minkey, hipStream_t s,
+                        void* Bt = nullptr);
 int fwd_fused_variants(int dtype, int D);
 hipError_t launch_fwd_fused(int dtype, int D, int variant, const void* Qp, const void* Kp, const void* VT,
                             const float* lsrc, const float* ldest, const float* C, void* O, float* lse, float* lse2,
-                            const int* reach, const int* minkey, int R, int L, int Lp, int d, int Zq, hipStream_t s);
+                            const int* reach, const int* minkey, int R, int L, int Lp, int d, int Zq, hipStream_t s,
+                            const void* Bt = nullptr);   // Bt (bf16): bias tiles of launch_carry; overrides the variant
 hipError_t launch_fwd_chunked(int dtype, int D, const void* Qp, const void* Kp, const void* VT, const float* lsrc,
                               const float* ldest, void* out, void* denom, float* lse2, long o_sz, long o_st, long o_sd,
                               long o_si, int R, int L, int Lp, int d, int c, int nch, int Zk, hipStream_t s);
