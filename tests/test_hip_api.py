@@ -124,7 +124,7 @@ def test_every_forward_variant_gives_the_same_result_and_autotune_records_one():
     for v in range(n):
         ops.tune_set(a[0], a[2], v)
         assert ops.tune_get(a[0], a[2]) == v
-        O, lse, _ = ops.fused_forward(*a)
+        O, lse, _ = ops.fused_forward(*a, recompute=True)      # the variants belong to the recomputing forward
         torch.cuda.synchronize()
         assert rel_err(O, O_ref) <= TOL[torch.bfloat16], (v, rel_err(O, O_ref))
         assert float((lse.cpu().double() - lse_ref).abs().max()) <= 2e-2
@@ -133,9 +133,43 @@ def test_every_forward_variant_gives_the_same_result_and_autotune_records_one():
         assert rel_err(results[v], results[0]) <= 2e-3, v            # same arithmetic, different summation order
     best = ops.autotune(*a)
     assert 0 <= best < n and ops.tune_get(a[0], a[2]) == best
-    O, _, _ = ops.fused_forward(*a)
+    O, _, _ = ops.fused_forward(*a, recompute=True)
     assert rel_err(O, O_ref) <= TOL[torch.bfloat16]
     ops.tune_set(a[0], a[2], 0)
+
+
+@pytest.mark.parametrize("shape", [(1, 2, 1, 1024 + 64, 128, 32), (2, 1, 3, 640, 48, 64)])
+@pytest.mark.parametrize("prune", [False, True])
+def test_recomputing_and_tile_exchanging_bf16_kernels_agree(shape, prune):
+    """bf16: by default the kernels pass the decay bias (fp16) and the score / decay gradients (bf16) through the
+    workspace; UA_FLAG_RECOMPUTE makes every kernel recompute them.  Both must meet the oracle, and each other far
+    inside the tolerance; the workspace of the recomputing mode is the small one."""
+    import ctypes
+    from universal_attention_triton_amd import _lib, ops
+    b, h, r, L, d, c = shape
+    dtype = torch.bfloat16
+    inp = orc.make_inputs(b, h, r, L, d, c, dtype=dtype, seed=91)
+    print("case recompute", shape, prune, flush=True)
+    dev = {k: v.cuda() for k, v in inp.items()}
+    a = [dev[k] for k in NAMES]
+    res = {}
+    for rec in (False, True):
+        O, lse, ws = ops.fused_forward(*a, for_backward=True, prune=prune, recompute=rec)
+        grads = ops.fused_backward(*a, O, lse, dev["dO"], ws=ws, prune=prune, recompute=rec)
+        g2 = ops.fused_backward(*a, O, lse, dev["dO"], ws=None, prune=prune, recompute=rec)     # without the forward's state
+        torch.cuda.synchronize()
+        res[rec] = (O, lse) + tuple(grads)
+        for x, y in zip(grads, g2):
+            assert rel_err(y, x) <= 1e-3
+        res[rec, "bytes"] = ws.numel()
+    assert res[True, "bytes"] < res[False, "bytes"]
+    O_ref, lse_ref, g_ref = dense_reference(inp)
+    for rec in (False, True):
+        assert rel_err(res[rec][0], O_ref) <= TOL[dtype]
+        for k, g, gr in zip(NAMES, res[rec][2:], g_ref):
+            assert rel_err(g.reshape(gr.shape), gr) <= TOL[dtype], (rec, k, rel_err(g.reshape(gr.shape), gr))
+    for name, x, y in zip(("O", "lse", "dk", "dv", "dq", "dsrc", "ddest"), res[False], res[True]):
+        assert rel_err(y, x) <= 6e-3, (name, rel_err(y, x))
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
