@@ -37,7 +37,8 @@ struct Layout {
   size_t Kp, KT, Vp, VT, Qp, QT, lsrc, ldest, C, lse2, knorm2, qnorm2, reach, minkey, Bt, fwd_end;
   // backward scratch
   size_t dOp, dOT, delta, dQacc, dKdacc, Dsuf, dKrow, dVrow, dsrc_raw, masked_nz, dS_st, dG_st, total;
-  bool tiles;     // the backward exchanges dS / dG tiles between its two kernels
+  bool tiles;       // bf16 merged operator: bias, dS and dG tiles are exchanged through the workspace
+  bool grad_tiles;  // ... dS and dG tiles (also the chunked operator with a chunk that is a multiple of 64)
 };
 
 int check_desc(const ua_desc* d, bool chunked) {
@@ -92,8 +93,9 @@ Layout make_layout(const ua_desc& d, bool chunked) {
   l.Dsuf = atomics ? 0 : take((size_t)l.Zk * l.nT * l.Lp * 4);
   l.masked_nz = take(256);
   // score and decay gradients of every (32 keys, 16 queries) tile
-  l.dS_st = l.tiles ? take((size_t)l.Zq * sq) : 0;
-  l.dG_st = l.tiles ? take((size_t)l.Zk * sq) : 0;
+  l.grad_tiles = l.tiles || (chunked && d.chunk % 64 == 0 && d.dtype == UA_BF16 && !(d.flags & UA_FLAG_RECOMPUTE));
+  l.dS_st = l.grad_tiles ? take((size_t)l.Zq * sq) : 0;
+  l.dG_st = l.grad_tiles ? take((size_t)l.Zk * sq) : 0;
   l.dKrow = take((size_t)l.Zk * l.Lp * l.D * 4);
   l.dVrow = take((size_t)l.Zk * l.Lp * l.D * 4);
   l.dsrc_raw = take((size_t)l.Zk * l.Lp * 4);
@@ -295,7 +297,7 @@ int run_bwd_common(const ua_desc& d, const Layout& l, char* ws, bool chunked, co
   a.dKrow = (float*)(ws + l.dKrow);
   a.dVrow = (float*)(ws + l.dVrow); a.dsrc_raw = (float*)(ws + l.dsrc_raw);
   a.masked_nz = (const int*)(ws + l.masked_nz);
-  a.dS_st = l.tiles ? ws + l.dS_st : nullptr; a.dG_st = l.tiles ? ws + l.dG_st : nullptr; a.Bt = l.tiles ? ws + l.Bt : nullptr;
+  a.dS_st = l.grad_tiles ? ws + l.dS_st : nullptr; a.dG_st = l.grad_tiles ? ws + l.dG_st : nullptr; a.Bt = l.tiles ? ws + l.Bt : nullptr;
   a.R = d.r; a.L = d.L; a.Lp = l.Lp; a.c = is_chunked ? d.chunk : 128; a.nch = l.nch; a.chunked = is_chunked ? 1 : 0;
   a.skip_masked = (d.flags & UA_FLAG_SKIP_MASKED) ? 1 : 0;
   a.split_r = (!chunked && d.r > 1) ? 1 : 0;
@@ -305,8 +307,9 @@ int run_bwd_common(const ua_desc& d, const Layout& l, char* ws, bool chunked, co
   }
   if (!chunked) {
     UA_PROF("k_bwd_queries", s);
-    if (l.tiles) UA_HIP(ua::launch_bwd_queries_from_tiles(l.D, a, dxq, d.d, l.Zq, s));
-    else UA_HIP(ua::launch_bwd_queries(d.dtype, l.D, a, dxq, d.d, l.Zk, s));
+    // chunked operator with tiles: both are enqueued, the flag k_delta left on the device decides which one works
+    if (l.grad_tiles) UA_HIP(ua::launch_bwd_queries_from_tiles(l.D, a, dxq, d.d, l.Zq, s));
+    if (!l.tiles) UA_HIP(ua::launch_bwd_queries(d.dtype, l.D, a, dxq, d.d, l.Zk, s));
   }
   UA_PROF("k_bwd_finish", s);
   if (d.dtype == UA_BF16) UA_HIP(finish_t<ua::bf16>(l, d, ws, chunked, src, dest, dkc, dvc, dxq, dsrc, ddest, s));

@@ -582,9 +582,10 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   using TN = Tile<T, 32, D>;
   using TT = Tile<T, D, 32>;
   constexpr int NK = D / 32, ND = D / 16;
-  static_assert(!TO || !CH, "tile exchange is for the merged operator");
-  // TO: the bias comes from the fp16 tiles of k_carry2<BO> (a.Bt), one 1 KB tile per wave and step after the stats row
-  constexpr int TILES = (CH ? 4 : 3) * (TN::BYTES + TT::BYTES), SB = TILES + (CH ? 2048 : 1024) + (TO ? 8 * 1024 : 0);
+  // merged operator with tile exchange: the bias comes from the fp16 tiles of k_carry2<BO> (a.Bt), one 1 KB tile per wave
+  // and step after the stats row (the chunked operator keeps the carries C, and Dsuf for the recomputing query side)
+  constexpr bool BI = TO && !CH;
+  constexpr int TILES = (CH ? 4 : 3) * (TN::BYTES + TT::BYTES), SB = TILES + (CH ? 2048 : 1024) + (BI ? 8 * 1024 : 0);
   // tiles of a stage: Kt, Q, dO | KT, QT, dOT | (CH) dO, dOT of the workgroup's second chunk
   // stats row of a stage: [lse2: 32f][delta: 32f][ldest: 32f][unused: 32f][forward carries of the 128 keys: 128f]
   // (CH) followed by [lse2: 32f][delta: 32f] of the second chunk
@@ -668,7 +669,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
       else src_ = Cz + (long)(2 * tb_) * Lp + 4 * (lane - 32);                              \
       issue_row((base) + TILES, src_);                                                      \
     }                                                                                       \
-    if (TO) issue_row((base) + TILES + 1024 + w * 1024, bt_src + ((long)tb_ * nT16 << 10)); \
+    if (BI) issue_row((base) + TILES + 1024 + w * 1024, bt_src + ((long)tb_ * nT16 << 10)); \
     if (CH && two) {                                                                        \
       stN.issue((base) + 3 * TN::BYTES + 3 * TT::BYTES, a.dOp + go_ + (long)Lp * D, w);     \
       stT.issue((base) + 4 * TN::BYTES + 3 * TT::BYTES, a.dOT + go_ + (long)Lp * D, w);     \
@@ -737,7 +738,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
     if (!MR || r == 0) {
       typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
       f16x8 hb;
-      if constexpr (TO) hb = *reinterpret_cast<const f16x8*>(base + TILES + 1024 + w * 1024 + 16 * lane);
+      if constexpr (BI) hb = *reinterpret_cast<const f16x8*>(base + TILES + 1024 + w * 1024 + 16 * lane);
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         f32x4 acc = {0, 0, 0, 0};
@@ -748,7 +749,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
         for (int v = 0; v < 4; ++v) {
           gk[i][v] = fmaxf(acc[v], 0.f);
           aff[i][v] = affinity(__builtin_amdgcn_logf(gk[i][v]), lab[v] + la);
-          if constexpr (TO) {
+          if constexpr (BI) {
             bias[i][v] = (float)hb[4 * i + v];
           } else {
             const float l2 = log2_one_minus(aff[i][v]);
@@ -757,7 +758,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
           if (MR) dB[i][v] = 0.f;
         }
       }
-      if constexpr (!TO) {
+      if constexpr (!BI) {
         const float cin = stats[128 + 16 * w + col];
         prefix32(bias[0], bias[1], gm);
 #pragma unroll
@@ -802,7 +803,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
     if (!MR || r == R - 1) {
       float t1;
       const float tot = suffix32(dB[0], dB[1], gm, t1);
-      if (!TO && g == 0) {
+      if (!BI && g == 0) {
         Dz[(long)(2 * tb + 1) * Lp] = dcar;
         Dz[(long)(2 * tb) * Lp] = dcar + t1;
       }
@@ -926,6 +927,7 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
   // wave's queries); they are swept only when some upstream gradient there is non-zero (flag set by k_delta)
   const float inv_c = CH ? 1.0f / (float)a.c : 0.f;
   const bool uniform_part = CH && !a.skip_masked && *a.masked_nz != 0;
+  if (CH && a.dS_st && !uniform_part) return;      // k_bwd_queries3 does the query side from the tiles
   const int uk0 = CH ? ((min((128 * jt) / a.c, a.nch - 1) + 1) * a.c) >> 6 : 0;
   const int uk0_w = CH ? ((min((16 * tq) / a.c, a.nch - 1) + 1) * a.c) >> 6 : 0;
   const int uk1 = uniform_part ? max(uk0, L >> 6) : uk0;
@@ -1170,6 +1172,8 @@ __global__ void __launch_bounds__(512) k_bwd_queries3(BwdArgs<T> a, T* __restric
   int bx, zq;
   xcd_map(bx, zq);
   const int Lp = a.Lp, L = a.L, nT16 = Lp / 16, R = a.R, zk = zq / R, r = zq % R;
+  // chunked operator with live (query, later chunk) pairs: their tiles are not exchanged, k_bwd_queries2 runs instead
+  if (a.chunked && !a.skip_masked && *a.masked_nz != 0) return;
   const int jt = gridDim.x - 1 - bx, tq = 8 * jt + w, tbq = tq >> 1;
   Stager<TT, 8> stT;
   stT.init(w, lane, Lp * (long)sizeof(T), D);

@@ -40,6 +40,10 @@ template __global__ void k_bwd_keys2<bf16, 64, 2, false, false, true>(BwdArgs<bf
 template __global__ void k_bwd_keys2<bf16, 64, 2, true, false, true>(BwdArgs<bf16>);
 template __global__ void k_bwd_keys2<bf16, 128, 2, false, false, true>(BwdArgs<bf16>);
 template __global__ void k_bwd_keys2<bf16, 128, 2, true, false, true>(BwdArgs<bf16>);
+template __global__ void k_bwd_keys2<bf16, 64, 2, false, true, true>(BwdArgs<bf16>);
+template __global__ void k_bwd_keys2<bf16, 64, 2, true, true, true>(BwdArgs<bf16>);
+template __global__ void k_bwd_keys2<bf16, 128, 2, false, true, true>(BwdArgs<bf16>);
+template __global__ void k_bwd_keys2<bf16, 128, 2, true, true, true>(BwdArgs<bf16>);
 
 template <class T, int D, int NST, bool MR, bool CH, bool TO>
 static hipError_t bwd2_mr(const BwdArgs<T>& a, int Lp, int Zk, hipStream_t s) {
@@ -52,6 +56,8 @@ static hipError_t bwd2_t(const BwdArgsV& v, int Zk, hipStream_t s) {
   if constexpr (sizeof(T) == 2) {
     if (v.dS_st && !v.chunked)
       return v.R > 1 ? bwd2_mr<T, D, NST, true, false, true>(a, v.Lp, Zk, s) : bwd2_mr<T, D, NST, false, false, true>(a, v.Lp, Zk, s);
+    if (v.dS_st)
+      return v.R > 1 ? bwd2_mr<T, D, NST, true, true, true>(a, v.Lp, Zk, s) : bwd2_mr<T, D, NST, false, true, true>(a, v.Lp, Zk, s);
   }
   if (v.chunked) return v.R > 1 ? bwd2_mr<T, D, NST, true, true, false>(a, v.Lp, Zk, s) : bwd2_mr<T, D, NST, false, true, false>(a, v.Lp, Zk, s);
   return v.R > 1 ? bwd2_mr<T, D, NST, true, false, false>(a, v.Lp, Zk, s) : bwd2_mr<T, D, NST, false, false, false>(a, v.Lp, Zk, s);
