@@ -43,10 +43,12 @@ enum {
                               flag ua_bwd finds this out by itself for chunks that are multiples of 64 (one pass
                               over g_out and g_denom that it makes anyway); the flag saves that check and, for the
                               other chunk sizes, the sweep over those pairs. */
-  UA_FLAG_RECOMPUTE = 4,   /* fused backward, bf16 (ua_fused_bwd and ua_workspace_bytes): by default the key-side kernel
-                              leaves the score and decay gradients of every tile in the workspace (Lp*Lp*2 bytes per
-                              query head and per kv head) and the query side is pure matrix work over them; with
-                              this flag the query-side kernel recomputes them instead: slower, workspace O(L*L/16). */
+  UA_FLAG_RECOMPUTE = 4,   /* bf16 (all ops and ua_workspace_bytes): by default the kernels of the fused operator pass the
+                              decay bias and the score / decay gradients of every tile to one another through the
+                              workspace (2 bytes per (key, query) pair and tensor: Lp*Lp*2 bytes per kv head for the
+                              bias, per query head and per kv head for the gradients; the chunked backward with a
+                              chunk that is a multiple of 64 does the same for the gradients).  With this flag every
+                              kernel recomputes what it needs instead: slower, workspace O(L*L/16). */
   UA_FLAG_PRUNE = 2        /* fused ops: skip (key, query) pairs whose softmax weight is provably below 2^-48 because
                               of the accumulated decay (no counterpart in the reference, which visits every pair).
                               The bound uses the largest key and query norms of the head; results change by less

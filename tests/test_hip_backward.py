@@ -162,6 +162,9 @@ def test_chunked_backward_chunk_multiple_of_64(shape, dtype):
     got = ops.chunked_backward(*ins, out, g_out.cuda(), g_denom.cuda(), ws=None)
     torch.cuda.synchronize()
     _report("recompute", got, want, TOL[dtype], tol_dkc)
+    got = ops.chunked_backward(*ins, out, g_out.cuda(), g_denom.cuda(), ws=None, recompute=True)
+    torch.cuda.synchronize()
+    _report("UA_FLAG_RECOMPUTE", got, want, TOL[dtype], tol_dkc)
     # upstream that vanishes wherever a query precedes the chunk
     t = torch.arange(L).view(L, 1, 1)
     live = (t >= torch.arange(n).view(1, 1, n) * c)
@@ -172,3 +175,6 @@ def test_chunked_backward_chunk_multiple_of_64(shape, dtype):
         got0 = ops.chunked_backward(*ins, out, g_out0.cuda(), g_denom0.cuda(), ws=ws, skip_masked=skip)
         torch.cuda.synchronize()
         _report("zero before chunk, skip=%s" % skip, got0, want0, TOL[dtype], tol_dkc)
+    got0 = ops.chunked_backward(*ins, out, g_out0.cuda(), g_denom0.cuda(), ws=None, recompute=True)
+    torch.cuda.synchronize()
+    _report("zero before chunk, UA_FLAG_RECOMPUTE", got0, want0, TOL[dtype], tol_dkc)

@@ -78,14 +78,15 @@ def _prep(kc, vc, xq, static_src, static_dest):
     return kc, vc, xq, src, dest
 
 
-def chunked_forward(kc, vc, xq, static_src, static_dest, for_backward=False):
-    """-> out [b,h,r,l,d,n] (chunk-major storage, returned as a permuted view), denom [b,h,r,l,n], state"""
+def chunked_forward(kc, vc, xq, static_src, static_dest, for_backward=False, recompute=False):
+    """-> out [b,h,r,l,d,n] (chunk-major storage, returned as a permuted view), denom [b,h,r,l,n], state
+    recompute: size the state for a backward that runs with UA_FLAG_RECOMPUTE (pass the same value to chunked_backward)."""
     kc, vc, xq, src, dest = _prep(kc, vc, xq, static_src, static_dest)
     lib = _lib.load()
     b, h, n, c, d = kc.shape
     r = xq.shape[2]
     L = n * c
-    desc = _desc(kc, xq, True)
+    desc = _desc(kc, xq, True, _lib.UA_FLAG_RECOMPUTE if recompute else 0)
     ws = _workspace(desc, _lib.UA_OP_BWD if for_backward else _lib.UA_OP_FWD, xq.device)
     store = torch.empty(b, h, r, n, L, d, dtype=xq.dtype, device=xq.device)
     out = store.permute(0, 1, 2, 4, 5, 3)
@@ -97,13 +98,13 @@ def chunked_forward(kc, vc, xq, static_src, static_dest, for_backward=False):
     return out, denom, ws
 
 
-def chunked_backward(kc, vc, xq, static_src, static_dest, out, g_out, g_denom, ws=None, skip_masked=False):
+def chunked_backward(kc, vc, xq, static_src, static_dest, out, g_out, g_denom, ws=None, skip_masked=False, recompute=False):
     kc, vc, xq, src, dest = _prep(kc, vc, xq, static_src, static_dest)
     lib = _lib.load()
     b, h, n, c, d = kc.shape
     r = xq.shape[2]
     L = n * c
-    desc = _desc(kc, xq, True, _lib.UA_FLAG_SKIP_MASKED if skip_masked else 0)
+    desc = _desc(kc, xq, True, (_lib.UA_FLAG_SKIP_MASKED if skip_masked else 0) | (_lib.UA_FLAG_RECOMPUTE if recompute else 0))
     has_fwd = ws is not None
     need = lib.ua_workspace_bytes(ctypes.byref(desc), _lib.UA_OP_BWD)
     if ws is None or ws.numel() < need:

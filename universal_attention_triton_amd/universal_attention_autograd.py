@@ -20,11 +20,15 @@ class _ChunkedBase(Function):
     # gradients of (query, chunk) pairs whose query precedes the chunk are propagated exactly as the
     # reference does; set to True only when the upstream gradient is known to vanish there
     skip_masked = False
+    # bf16, chunk a multiple of 64: True keeps the backward's workspace small (UA_FLAG_RECOMPUTE: its second kernel
+    # recomputes the score and decay gradients instead of reading them from 2*L*L bytes per head)
+    recompute = False
 
     @staticmethod
     def forward(ctx, kc, vc, xq, static_src, static_dest):
         need_grad = any(ctx.needs_input_grad)
-        out, denom, ws = ops.chunked_forward(kc, vc, xq, static_src, static_dest, for_backward=need_grad)
+        out, denom, ws = ops.chunked_forward(kc, vc, xq, static_src, static_dest, for_backward=need_grad,
+                                             recompute=_ChunkedBase.recompute)
         ctx.save_for_backward(kc, vc, xq, static_src, static_dest, out)
         ctx.ws = ws if need_grad else None
         return out, denom
@@ -33,7 +37,8 @@ class _ChunkedBase(Function):
     def backward(ctx, g_out, g_denom):
         kc, vc, xq, static_src, static_dest, out = ctx.saved_tensors
         dk, dv, dq, dsrc, ddest = ops.chunked_backward(kc, vc, xq, static_src, static_dest, out, g_out, g_denom,
-                                                       ws=ctx.ws, skip_masked=_ChunkedBase.skip_masked)
+                                                       ws=ctx.ws, skip_masked=_ChunkedBase.skip_masked,
+                                                       recompute=_ChunkedBase.recompute)
         ctx.ws = None
         return dk, dv, dq.view(xq.shape), dsrc.view(static_src.shape), ddest.view(static_dest.shape)
 
