@@ -283,3 +283,37 @@ def test_pruning_of_negligible_pairs_changes_nothing(case, dtype):
     assert rel_err(res[True][0], O_ref) <= TOL[dtype]
     for k, g, gr in zip(NAMES, res[True][2:], g_ref):
         assert rel_err(g.reshape(gr.shape), gr) <= (TOL[dtype] if k != "kc" else max(TOL[dtype], 4e-4)), (k, rel_err(g.reshape(gr.shape), gr))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_decoder_front_end_takes_sequence_major_projections_without_copies(dtype):
+    """[b, s, heads, d] projections and the fused gate tensor of the reference's driver (main.py:19-31): the views
+    built from them reach the kernels as they are (keys / values / queries are read through their strides)."""
+    from universal_attention_triton_amd import frontend, ops
+    b, s, n_kv, rep, d, c = 2, 256, 2, 2, 64, 64
+    inp = orc.make_inputs(b, n_kv, rep, s, d, c, dtype=dtype, seed=61)
+    O_ref, _, g_ref = dense_reference(inp)
+    # sequence-major tensors holding the same values
+    q = inp["xq"].flatten(1, 2).transpose(1, 2).contiguous().cuda().requires_grad_()          # [b, s, n, d]
+    k = inp["kc"].flatten(2, 3).transpose(1, 2).contiguous().cuda().requires_grad_()          # [b, s, n_kv, d]
+    v = inp["vc"].flatten(2, 3).transpose(1, 2).contiguous().cuda().requires_grad_()
+    static = torch.stack([inp["static_src"].flatten(2, 3), inp["static_dest"]], 0).permute(1, 3, 0, 2).reshape(b, s, 2 * n_kv)
+    static = static.contiguous().cuda().requires_grad_()
+    seen = []
+    real = ops._rows_k
+    ops._rows_k = lambda t: (seen.append((t.data_ptr(), t.is_contiguous())), real(t))[1]
+    try:
+        out = frontend.decoder_attention(q, k, v, static, chunk=c)
+    finally:
+        ops._rows_k = real
+    assert out.shape == (b, s, n_kv * rep, d)
+    assert (k.data_ptr(), False) in seen and (v.data_ptr(), False) in seen          # the kernels saw the strided views themselves
+    dO = inp["dO"].flatten(1, 2).transpose(1, 2).cuda()
+    gq, gk, gv, gs = torch.autograd.grad(out, [q, k, v, static], dO)
+    assert rel_err(out.transpose(1, 2).reshape(O_ref.shape), O_ref) <= TOL[dtype]
+    assert rel_err(gq.transpose(1, 2).reshape(g_ref[2].shape), g_ref[2]) <= TOL[dtype]
+    assert rel_err(gv.transpose(1, 2).reshape(g_ref[1].shape), g_ref[1]) <= TOL[dtype]
+    assert rel_err(gk.transpose(1, 2).reshape(g_ref[0].shape), g_ref[0]) <= max(TOL[dtype], 4e-4)
+    gs = gs.view(b, s, 2, n_kv).permute(2, 0, 3, 1)
+    assert rel_err(gs[0].reshape(g_ref[3].shape), g_ref[3]) <= TOL[dtype]
+    assert rel_err(gs[1].reshape(g_ref[4].shape), g_ref[4]) <= TOL[dtype]
