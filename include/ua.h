@@ -45,8 +45,8 @@ enum {
                               other chunk sizes, the sweep over those pairs. */
   UA_FLAG_RECOMPUTE = 4,   /* bf16 (all ops and ua_workspace_bytes): by default the kernels of the fused operator pass the
                               decay bias and the score / decay gradients of every tile to one another through the
-                              workspace (2 bytes per (key, query) pair and tensor: Lp*Lp*2 bytes per kv head for the
-                              bias, per query head and per kv head for the gradients; the chunked backward with a
+                              workspace (2 bytes per causal (key, query) pair and tensor: about Lp*Lp bytes per kv head for
+                              the bias, per query head and per kv head for the gradients; the chunked backward with a
                               chunk that is a multiple of 64 does the same for the gradients).  With this flag every
                               kernel recomputes what it needs instead: slower, workspace O(L*L/16). */
   UA_FLAG_PRUNE = 2        /* fused ops: skip (key, query) pairs whose softmax weight is provably below 2^-48 because

@@ -38,10 +38,10 @@ struct BwdArgs {
   float *dKrow, *dVrow;         // [Zk][Lp][D]
   float* dsrc_raw;              // [Zk][Lp]
   // optional (16-bit dtypes, fused mode): k_bwd_keys2 leaves the score gradient dS [Zq] and the decay gradient dG [Zk]
-  // of every visited (16 keys, 32 queries) tile, in operand precision, as [z][Lp/16 query tiles][Lp/32 key halves]
-  // tiles of 1 KB laid out like StageT (32 keys x 16 queries); k_bwd_queries3 turns them into dQ and the column side of dK
+  // of every visited (16 keys, 32 queries) tile, in operand precision, as [z][causal triangle of (16-query tile, 32-key half)
+  // pairs, see tri_grad_row] tiles of 1 KB laid out like StageT (32 keys x 16 queries); k_bwd_queries3 turns them into dQ and the column side of dK
   T *dS_st, *dG_st;
-  const _Float16* Bt;           // with dS_st: fp16 bias tiles of k_carry2<BO>, [Zk][Lp/32][Lp/16][1 KB]
+  const _Float16* Bt;           // with dS_st: fp16 bias tiles of k_carry2<BO>, [Zk][triangle, see tri_bias_row][1 KB]
   int R, L, Lp, c, nch, chunked, skip_masked;
   int split_r;                  // k_bwd_queries2: one workgroup per (kv head, query group); dKdacc is then [Zq][Lp][D]
 };

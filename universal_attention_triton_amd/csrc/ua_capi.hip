@@ -77,9 +77,9 @@ Layout make_layout(const ua_desc& d, bool chunked) {
   // tile, first key tile reaching every query block
   l.knorm2 = take((size_t)l.Zk * (l.nT / 2) * 4); l.qnorm2 = take((size_t)l.Zq * (l.nT / 2) * 4); l.reach = take((size_t)l.Zk * l.nT * 4); l.minkey = take((size_t)l.Zk * (l.nT / 2) * 4);
   // bf16 fused operator: the kernels exchange tiles through the workspace instead of recomputing them (fp16 bias of every
-  // (16 keys, 32 queries) tile here; score and decay gradients in the backward part), 1 KB per tile, full square
+  // (16 keys, 32 queries) tile here; score and decay gradients in the backward part), 1 KB per tile
   l.tiles = !chunked && d.dtype == UA_BF16 && !(d.flags & UA_FLAG_RECOMPUTE);
-  const size_t sq = (size_t)l.nT * (l.Lp / 32) * 1024;
+  const size_t sq = (size_t)ua::tri_tiles(l.Lp / 32) * 1024;     // the causal triangle of 1 KB tiles, per head
   l.Bt = l.tiles ? take((size_t)l.Zk * sq) : 0;
   l.fwd_end = off;
   const size_t gbytes = (size_t)l.Zq * l.nch * l.Lp * l.D * l.esz;

@@ -88,7 +88,8 @@ struct FalseC { static constexpr bool value = false; };
 // is at most max|k| max|q|, and a query's normaliser is at least its own score); a wave stops once all its 16
 // keys are there and records the last 32-query block it reached in reach[z][key tile].
 // BO: instead of the carries C, leave the bias of every visited (16 keys, 32 queries) tile itself, as fp16, in
-// Bt[z][Lp/32 query blocks][Lp/16 key tiles][1 KB]: lane l of the key tile's wave owns bytes 16 l .. 16 l + 15 = its
+// Bt[z][causal triangle of (32-query block, 16-key tile) pairs, see tri_bias_row][1 KB]: lane l of the key tile's wave owns
+// bytes 16 l .. 16 l + 15 = its
 // key's bias towards queries 4g..4g+3 of the block's first 16-query tile, then of the second (g = l / 16).  The
 // 16-bit forward and backward kernels then read the bias instead of recomputing the affinity chain; fp16 resolves
 // the bias of every pair that carries weight (|bias| < 16: 2^-7 at worst) to better than the bf16 rounding of the
@@ -180,7 +181,7 @@ __global__ void __launch_bounds__(512) k_carry2(const T* __restrict__ Kp, const 
       f16x8 hb;
 #pragma unroll
       for (int v = 0; v < 4; ++v) { hb[v] = (_Float16)(x[0][v] + carry); hb[4 + v] = (_Float16)(x[1][v] + carry); }
-      char* dst = reinterpret_cast<char*>(Bt) + ((((long)z * nT + tb) * nT16 + sb16) << 10) + 16 * lane;
+      char* dst = reinterpret_cast<char*>(Bt) + (((long)z * tri_tiles(nT) + tri_bias_row(tb) + sb16) << 10) + 16 * lane;
       __builtin_nontemporal_store(hb, reinterpret_cast<f16x8*>(dst));
       carry += tot;
     } else {
@@ -376,7 +377,7 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW
   else if (lane < 32) row_base = lsrc + (long)zk * Lp + 4 * (lane - 16);
   else { row_base = reinterpret_cast<const float*>(reach + zk * nT16); row_step = 4; }
   // BI: this lane's 16 bytes of key tile 0 of the wave's query block
-  const char* bt_src = reinterpret_cast<const char*>(Bt) + ((((long)zk * (Lp >> 5) + tbq) * nT16) << 10) + 16 * lane;
+  const char* bt_src = reinterpret_cast<const char*>(Bt) + (((long)zk * tri_tiles(Lp >> 5) + tri_bias_row(tbq)) << 10) + 16 * lane;
 
 #define UA_ISSUE(s, base)                                                                   \
   {                                                                                         \
@@ -644,8 +645,8 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   // where this lane's four values of a (16 keys, 16 queries) tile go inside the 1 KB tile of its 32-key half
   static_assert(!TO || sizeof(T) == 2, "tiles are exchanged in 16-bit operand precision");
   // this lane's 16 bytes of the wave's bias tile of query block 0
-  const char* bt_src = reinterpret_cast<const char*>(a.Bt) + ((((long)zk * (Lp >> 5)) * nT16 + sb16) << 10) + 16 * lane;
-  const long st_row = (long)(Lp >> 5) << 10;                       // bytes between consecutive 16-query tiles
+  const char* bt_src = reinterpret_cast<const char*>(a.Bt) + (((long)zk * tri_tiles(Lp >> 5) + sb16) << 10) + 16 * lane;
+  const long st_head = tri_tiles(Lp >> 5) << 10;                   // bytes of gradient tiles per head
   const long st_lane = ((long)(sb16 >> 1) << 10) + StageT<bf16>::addr(perm32(16 * (sb16 & 1) + col), 8 * g);
 
 #define UA_ISSUE(s, base)                                                                   \
@@ -669,7 +670,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
       else src_ = Cz + (long)(2 * tb_) * Lp + 4 * (lane - 32);                              \
       issue_row((base) + TILES, src_);                                                      \
     }                                                                                       \
-    if (BI) issue_row((base) + TILES + 1024 + w * 1024, bt_src + ((long)tb_ * nT16 << 10)); \
+    if (BI) issue_row((base) + TILES + 1024 + w * 1024, bt_src + (tri_bias_row(tb_) << 10)); \
     if (CH && two) {                                                                        \
       stN.issue((base) + 3 * TN::BYTES + 3 * TT::BYTES, a.dOp + go_ + (long)Lp * D, w);     \
       stT.issue((base) + 4 * TN::BYTES + 3 * TT::BYTES, a.dOT + go_ + (long)Lp * D, w);     \
@@ -787,9 +788,10 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
       }
       const Frag<T> bp = as_operand16<T>(P[0], P[1]), bs = as_operand16<T>(dS[0], dS[1]);
       if constexpr (TO) {     // the two halves of the operand are the two query tiles of the block
-        char* p = reinterpret_cast<char*>(a.dS_st) + (((long)zk * R + r) * nT16 + 2 * tb) * st_row + st_lane;
+        // query tiles 2 tb and 2 tb + 1: their rows start tb + 1 tiles apart
+        char* p = reinterpret_cast<char*>(a.dS_st) + ((long)zk * R + r) * st_head + (tri_grad_row(2 * tb) << 10) + st_lane;
         __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&bs)[0], reinterpret_cast<u32x2*>(p));
-        __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&bs)[1], reinterpret_cast<u32x2*>(p + st_row));
+        __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&bs)[1], reinterpret_cast<u32x2*>(p + ((long)(tb + 1) << 10)));
       }
 #pragma unroll
       for (int n = 0; n < ND; ++n) mma16(dVt[n], ld8(sdOT + TT::at(n, col, 0, g)), bp);
@@ -820,9 +822,9 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
       dcar += tot;
       const Frag<T> b = as_operand16<T>(dB[0], dB[1]);
       if constexpr (TO) {
-        char* p = reinterpret_cast<char*>(a.dG_st) + ((long)zk * nT16 + 2 * tb) * st_row + st_lane;
+        char* p = reinterpret_cast<char*>(a.dG_st) + (long)zk * st_head + (tri_grad_row(2 * tb) << 10) + st_lane;
         __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&b)[0], reinterpret_cast<u32x2*>(p));
-        __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&b)[1], reinterpret_cast<u32x2*>(p + st_row));
+        __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&b)[1], reinterpret_cast<u32x2*>(p + ((long)(tb + 1) << 10)));
       }
 #pragma unroll
       for (int n = 0; n < ND; ++n) mma16(dKt[n], ld8(sKT + TT::at(n, col, 0, g)), b);
@@ -1183,10 +1185,10 @@ __global__ void __launch_bounds__(512) k_bwd_queries3(BwdArgs<T> a, T* __restric
   const T* KTz = a.KT + (long)zk * D * Lp;
   const int n_kt = 2 * jt + 2;
   const int kt_min = (a.minkey[zk * (nT16 >> 1) + 4 * jt] >> 2) & ~1;
-  const long st_row = (long)(Lp >> 5) << 10;
   // this lane's 16 bytes of the wave's tiles of key half h: base + h * 1024
-  const char* pS = reinterpret_cast<const char*>(a.dS_st) + ((long)zq * nT16 + tq) * st_row + 16 * lane;
-  const char* pG = reinterpret_cast<const char*>(a.dG_st) + ((long)zk * nT16 + tq) * st_row + 16 * lane;
+  const long st_head = tri_tiles(Lp >> 5) << 10;
+  const char* pS = reinterpret_cast<const char*>(a.dS_st) + (long)zq * st_head + (tri_grad_row(tq) << 10) + 16 * lane;
+  const char* pG = reinterpret_cast<const char*>(a.dG_st) + (long)zk * st_head + (tri_grad_row(tq) << 10) + 16 * lane;
   const int* reach_z = a.reach + zk * nT16;
 
 #define UA_ISSUE(s, base)                                                                   \
