@@ -309,18 +309,18 @@ __global__ void __launch_bounds__(256) k_chunk_masked_denom(T* __restrict__ deno
 // ---------------------------------------------------------------------------------------------
 // CHUNKED: the reference's chunked operator instead of the merged one: the softmax restarts at every chunk of
 // co.c keys (a multiple of 64) and each chunk's result goes to out[.., i] / denom[.., i] / lse2[zq*nch + i][t].
-// BI (8 waves): the decay bias comes from the fp16 tiles k_carry2<BO> left in Bt instead of being recomputed (no key-key
+// BI (4 or 8 waves): the decay bias comes from the fp16 tiles k_carry2<BO> left in Bt instead of being recomputed (no key-key
 // product, no affinity chain, no scan).  The two waves that share a 32-query block copy its four key tiles (two each)
 // into one LDS region per step.
 template <class T, int D, int NST, int NW, bool CHUNKED, bool BI = false>
-__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW >= 8 ? NW / 4 : 2, NW >= 8 ? NW / 4 : 2))) k_fwd_fused2(const T* __restrict__ Qp, const T* __restrict__ Kp,
+__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW >= 8 ? NW / 4 : (BI ? 3 : 2), NW >= 8 ? NW / 4 : (BI ? 3 : 2)))) k_fwd_fused2(const T* __restrict__ Qp, const T* __restrict__ Kp,
                                                     const T* __restrict__ VT, const float* __restrict__ lsrc,
                                                     const float* __restrict__ ldest, const float* __restrict__ C,
                                                     T* __restrict__ O, float* __restrict__ lse, float* __restrict__ lse2,
                                                     const int* __restrict__ reach, const int* __restrict__ minkey,
                                                     int R, int L, int Lp, int d, ChunkOut<T> co,
                                                     const _Float16* __restrict__ Bt = nullptr) {
-  static_assert(!BI || (NW == 8 && !CHUNKED), "bias tiles: 8 waves, merged operator");
+  static_assert(!BI || ((NW == 8 || NW == 4) && !CHUNKED), "bias tiles: 4 or 8 waves, merged operator");
   using TN = Tile<T, 32, D>;
   using TT = Tile<T, D, 32>;
   constexpr int NK = D / 32, ND = D / 16;
