@@ -128,6 +128,17 @@ int ua_merge_fwd(int dtype, int64_t rows, int32_t L, int32_t d, int32_t n, const
 int ua_merge_bwd(int dtype, int64_t rows, int32_t L, int32_t d, int32_t n, const ua_chunked* mat, const void* vec,
                  const void* g, const ua_chunked* d_mat, void* d_vec, ua_stream_t stream);
 
+/* Stand-alone decay bias ("affinity scores"): replaces _affinity_fwd / _affinity_bwd and the AffinityScores wrapper
+ * (Universal_Attention/triton/affinity_kernel_opt.py:100-127, :130-423, :425-450).  desc: b, h, L, d, dtype (r, chunk and
+ * flags are ignored).  k: [b,h,L,d] rows; src, dest: contiguous [b,h,L]; aff / daff: contiguous [b,h,L,L] in the
+ * dtype, aff[b,h,t,s] = bias of key s towards query t in natural-log units (0 on the diagonal, -1e12 where s > t).
+ * dk contiguous [b,h,L,d]; dsrc, ddest contiguous [b,h,L].  Workspace: ua_affinity_workspace_bytes(desc, backward). */
+size_t ua_affinity_workspace_bytes(const ua_desc* desc, int backward);
+int ua_affinity_fwd(const ua_desc* desc, const ua_rows* k, const void* src, const void* dest, void* aff, void* ws,
+                    size_t ws_bytes, ua_stream_t stream);
+int ua_affinity_bwd(const ua_desc* desc, const ua_rows* k, const void* src, const void* dest, const void* daff, void* dk,
+                    void* dsrc, void* ddest, void* ws, size_t ws_bytes, ua_stream_t stream);
+
 /* On-device autotune table: replaces the @triton.autotune wrappers
  * (universal_attention_kernel.py:10-25, universal_attention_kernel_opt.py:8-36).  Times the kernel variants
  * available for (op, desc) on `stream` using `ws` and records the fastest in the process-wide table that

@@ -161,6 +161,16 @@ def dense_bias(k, static_src, static_dest):
     return torch.cumsum(logs, dim=-1)
 
 
+def affinity_scores(k, static_src, static_dest):
+    """The bias as the L x L additive mask of the reference's stand-alone op (affinity_kernel_opt.py:457-462,
+    _gen_affinity_scores_torch): [b,h,t,s], cumulative sum cast to k.dtype, -1e12 where the key comes after the query.
+    Built on dense_bias, which the brute-force and closed-form tests pin."""
+    B = dense_bias(k, static_src, static_dest).to(k.dtype)                      # [b,h,s,t]
+    l = k.shape[-2]
+    after = torch.ones(l, l, dtype=torch.bool, device=k.device).tril(-1)        # s > t
+    return B.masked_fill(after, NEG_FILL).transpose(-1, -2).contiguous()
+
+
 def dense_forward(k, v, q, static_src, static_dest, return_lse=False):
     """O[r,t] = sum_{s<=t} softmax_s(k_s.q_t + B[s,t]) v_s.
 

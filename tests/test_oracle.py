@@ -175,3 +175,29 @@ def test_merge_backward_equals_autograd():
     torch.testing.assert_close(got[0], want[0])
     torch.testing.assert_close(got[1], want[1])
     torch.testing.assert_close(orc.merge(out.detach(), denom.detach()), O.detach())
+
+
+def test_affinity_scores_restatement_matches_dense_bias_and_the_reference_mask():
+    """orc.affinity_scores (reference affinity_kernel_opt.py:457-462): transposed dense_bias where the key does not
+    come after the query, -1e12 elsewhere, in the input dtype; a brute-force loop on a tiny case pins the layout."""
+    import math
+    g = torch.Generator().manual_seed(11)
+    b, h, L, d = 1, 2, 12, 8
+    k = torch.randn(b, h, L, d, generator=g, dtype=torch.float64)
+    k = k / k.norm(dim=-1, keepdim=True)
+    src = torch.sigmoid(torch.randn(b, h, L, generator=g, dtype=torch.float64))
+    dest = torch.sigmoid(torch.randn(b, h, L, generator=g, dtype=torch.float64))
+    aff = orc.affinity_scores(k, src, dest)
+    assert aff.shape == (b, h, L, L)
+    for hh in range(h):
+        for t in range(L):
+            for s in range(L):
+                if s > t:
+                    assert aff[0, hh, t, s] == -1e12
+                    continue
+                tot = 0.0
+                for u in range(s + 1, t + 1):
+                    a = max(float(k[0, hh, s] @ k[0, hh, u]), 0.0) ** (2 / 3) * float(src[0, hh, s] * dest[0, hh, u]) ** (1 / 3)
+                    tot += math.log1p(-min(a, 1 - 1e-6))
+                assert abs(float(aff[0, hh, t, s]) - tot) <= 1e-12 * max(1.0, abs(tot))
+    assert orc.affinity_scores(k.to(torch.bfloat16), src.to(torch.bfloat16), dest.to(torch.bfloat16)).dtype == torch.bfloat16

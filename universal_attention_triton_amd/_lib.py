@@ -45,6 +45,10 @@ SIGNATURES = {
                              c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
     "ua_merge_fwd": (c_int, [c_int, c_int64, c_int32, c_int32, c_int32, P(UaChunked), c_void_p, c_void_p, c_void_p]),
     "ua_merge_bwd": (c_int, [c_int, c_int64, c_int32, c_int32, c_int32, P(UaChunked), c_void_p, c_void_p, P(UaChunked), c_void_p, c_void_p]),
+    "ua_affinity_workspace_bytes": (c_size_t, [P(UaDesc), c_int]),
+    "ua_affinity_fwd": (c_int, [P(UaDesc), P(UaRows), c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "ua_affinity_bwd": (c_int, [P(UaDesc), P(UaRows), c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
+                                c_void_p]),
     "ua_autotune": (c_int, [P(UaDesc), c_int, c_void_p, c_size_t, c_void_p]),
     "ua_tune_get": (c_int, [P(UaDesc), c_int]),
     "ua_tune_set": (c_int, [P(UaDesc), c_int, c_int]),

@@ -505,6 +505,83 @@ int ua_merge_bwd(int dtype, int64_t rows, int32_t L, int32_t d, int32_t n, const
   return UA_OK;
 }
 
+// ---- stand-alone decay bias (affinity scores) ------------------------------------------------
+namespace {
+struct AffLayout { int D, Lp, Z; size_t Kp, KT, lsrc, ldest, fwd_end, DL, row, colp, gs_row, gs_col, total; };
+AffLayout make_aff_layout(const ua_desc& d) {
+  AffLayout l{};
+  l.D = d.d <= 64 ? 64 : 128;
+  l.Lp = (int)align_up((size_t)d.L, 128);
+  l.Z = d.b * d.h;
+  const size_t esz = d.dtype == UA_BF16 ? 2 : 4;
+  size_t off = 0;
+  auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
+  const size_t kbytes = (size_t)l.Z * l.Lp * l.D * esz;
+  l.Kp = take(kbytes); l.KT = take(kbytes);
+  l.lsrc = take((size_t)l.Z * l.Lp * 4); l.ldest = take((size_t)l.Z * l.Lp * 4);
+  l.fwd_end = off;
+  l.DL = take((size_t)l.Z * d.L * d.L * 4);
+  l.row = take((size_t)l.Z * l.Lp * l.D * 4); l.colp = take((size_t)l.Z * l.Lp * l.D * 4);
+  l.gs_row = take((size_t)l.Z * l.Lp * 4); l.gs_col = take((size_t)l.Z * l.Lp * 4);
+  l.total = off;
+  return l;
+}
+int aff_prepare(const ua_desc* desc, const ua_rows* k, const void* src, const void* dest, void* ws, size_t ws_bytes, bool bwd,
+                AffLayout& l, hipStream_t s) {
+  if (int e = check_desc(desc, false)) return e;
+  l = make_aff_layout(*desc);
+  if (!k || !k->ptr || !src || !dest) return fail(UA_EINVAL, "null input tensor");
+  if (!ws) return fail(UA_EWORKSPACE, "null workspace");
+  if ((uintptr_t)ws % 256 != 0) return fail(UA_EWORKSPACE, "workspace must be 256-byte aligned");
+  const size_t need = bwd ? l.total : l.fwd_end;
+  if (ws_bytes < need) return fail(UA_EWORKSPACE, "workspace has %zu bytes, %zu needed", ws_bytes, need);
+  const ua_desc& d = *desc;
+  char* w = (char*)ws;
+  const ua::RowsView K = rows_view(*k, d.h, 1);
+  UA_HIP(pack(d.dtype, l.D, K, w + l.Kp, w + l.KT, d.d, d.L, l.Lp, l.Z, TR_PERM32, s));
+  const dim3 grid((l.Lp + 255) / 256, l.Z);
+  if (d.dtype == UA_BF16)
+    hipLaunchKernelGGL((ua::k_gates<ua::bf16>), grid, dim3(256), 0, s, (const ua::bf16*)src, (const ua::bf16*)dest,
+                       (float*)(w + l.lsrc), (float*)(w + l.ldest), d.L, l.Lp);
+  else
+    hipLaunchKernelGGL((ua::k_gates<float>), grid, dim3(256), 0, s, (const float*)src, (const float*)dest,
+                       (float*)(w + l.lsrc), (float*)(w + l.ldest), d.L, l.Lp);
+  UA_HIP(hipGetLastError());
+  return UA_OK;
+}
+}  // namespace
+
+size_t ua_affinity_workspace_bytes(const ua_desc* desc, int backward) {
+  if (check_desc(desc, false) != UA_OK) return 0;
+  const AffLayout l = make_aff_layout(*desc);
+  return backward ? l.total : l.fwd_end;
+}
+
+int ua_affinity_fwd(const ua_desc* desc, const ua_rows* k, const void* src, const void* dest, void* aff, void* ws,
+                    size_t ws_bytes, ua_stream_t stream) {
+  AffLayout l;
+  hipStream_t s = (hipStream_t)stream;
+  if (!aff) return fail(UA_EINVAL, "null output tensor");
+  if (int e = aff_prepare(desc, k, src, dest, ws, ws_bytes, false, l, s)) return e;
+  char* w = (char*)ws;
+  UA_HIP(ua::launch_aff_fwd(desc->dtype, l.D, w + l.Kp, (const float*)(w + l.lsrc), (const float*)(w + l.ldest), aff, desc->L, l.Lp,
+                            l.Z, s));
+  return UA_OK;
+}
+
+int ua_affinity_bwd(const ua_desc* desc, const ua_rows* k, const void* src, const void* dest, const void* daff, void* dk,
+                    void* dsrc, void* ddest, void* ws, size_t ws_bytes, ua_stream_t stream) {
+  AffLayout l;
+  hipStream_t s = (hipStream_t)stream;
+  if (!daff || !dk || !dsrc || !ddest) return fail(UA_EINVAL, "null tensor");
+  if (int e = aff_prepare(desc, k, src, dest, ws, ws_bytes, true, l, s)) return e;
+  char* w = (char*)ws;
+  UA_HIP(ua::launch_aff_bwd(desc->dtype, l.D, w + l.Kp, w + l.KT, (const float*)(w + l.lsrc), (const float*)(w + l.ldest), daff,
+                            (float*)(w + l.DL), (float*)(w + l.row), (float*)(w + l.colp), (float*)(w + l.gs_row),
+                            (float*)(w + l.gs_col), src, dest, dk, dsrc, ddest, desc->L, l.Lp, desc->d, l.Z, s));
+  return UA_OK;
+}
+
 void ua_prof_enable(int on) {
   std::lock_guard<std::mutex> g(g_prof_mu);
   g_prof_on = on != 0;

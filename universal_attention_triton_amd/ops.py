@@ -246,3 +246,43 @@ def tune_set(kc, xq, variant, op=_lib.UA_OP_FUSED_FWD):
 
 def tune_get(kc, xq, op=_lib.UA_OP_FUSED_FWD):
     return _lib.load().ua_tune_get(ctypes.byref(_desc(kc, xq, False)), op)
+
+
+def _affinity_args(k, src, dest):
+    _require_gpu(k, src, dest)
+    if not (k.dtype == src.dtype == dest.dtype):
+        raise TypeError("k, src and dest must share one dtype")
+    b, h, L, d = k.shape
+    assert src.shape == (b, h, L) and dest.shape == (b, h, L)
+    k = _last_contig(k)
+    desc = UaDesc(b, h, 1, L, d, 0, _dtype_code(k), 0)
+    rows = UaRows(k.data_ptr(), k.stride(0), k.stride(1), 0, 0, k.stride(2), L)
+    return k, src.contiguous(), dest.contiguous(), desc, rows
+
+
+def affinity_forward(k, src, dest):
+    """k [b,h,L,d], src, dest [b,h,L] -> aff [b,h,L,L] (k.dtype): bias of key s towards query t at aff[b,h,t,s]"""
+    k, src, dest, desc, rows = _affinity_args(k, src, dest)
+    lib = _lib.load()
+    b, h, L, _ = k.shape
+    ws = torch.empty(lib.ua_affinity_workspace_bytes(ctypes.byref(desc), 0), dtype=torch.uint8, device=k.device)
+    aff = torch.empty(b, h, L, L, dtype=k.dtype, device=k.device)
+    _lib.check(lib.ua_affinity_fwd(ctypes.byref(desc), ctypes.byref(rows), src.data_ptr(), dest.data_ptr(), aff.data_ptr(),
+                                   ws.data_ptr(), ws.numel(), _stream()), "ua_affinity_fwd")
+    return aff
+
+
+def affinity_backward(k, src, dest, daff):
+    """-> dk [b,h,L,d], dsrc, ddest [b,h,L]"""
+    k, src, dest, desc, rows = _affinity_args(k, src, dest)
+    lib = _lib.load()
+    b, h, L, d = k.shape
+    daff = daff.to(k.dtype).contiguous()
+    ws = torch.empty(lib.ua_affinity_workspace_bytes(ctypes.byref(desc), 1), dtype=torch.uint8, device=k.device)
+    dk = torch.empty(b, h, L, d, dtype=k.dtype, device=k.device)
+    dsrc = torch.empty(b, h, L, dtype=k.dtype, device=k.device)
+    ddest = torch.empty_like(dsrc)
+    _lib.check(lib.ua_affinity_bwd(ctypes.byref(desc), ctypes.byref(rows), src.data_ptr(), dest.data_ptr(), daff.data_ptr(),
+                                   dk.data_ptr(), dsrc.data_ptr(), ddest.data_ptr(), ws.data_ptr(), ws.numel(), _stream()),
+               "ua_affinity_bwd")
+    return dk, dsrc, ddest
