@@ -172,6 +172,39 @@ def test_recomputing_and_tile_exchanging_bf16_kernels_agree(shape, prune):
         assert rel_err(y, x) <= 6e-3, (name, rel_err(y, x))
 
 
+@pytest.mark.parametrize("shape", [(1, 2, 4, 512 + 32, 128, 32), (2, 1, 3, 640, 48, 64), (1, 3, 2, 300, 64, 4)])
+@pytest.mark.parametrize("prune", [False, True])
+def test_grouped_queries_shared_and_separate_key_sweeps_agree(shape, prune):
+    """bf16, r > 1: with few kv heads the key side of the backward gives every query group a sweep of its own and adds
+    the partial key gradients up afterwards; UA_FLAG_SHARE_GROUPS keeps one sweep per kv head.  Both must meet the
+    oracle and agree with each other up to bf16 rounding of the per-group decay gradients; the forward is the same."""
+    from universal_attention_triton_amd import ops
+    b, h, r, L, d, c = shape
+    dtype = torch.bfloat16
+    inp = orc.make_inputs(b, h, r, L, d, c, dtype=dtype, seed=77)
+    print("case groups", shape, prune, flush=True)
+    dev = {k: v.cuda() for k, v in inp.items()}
+    a = [dev[k] for k in NAMES]
+    res = {}
+    for share in (False, True):
+        O, lse, ws = ops.fused_forward(*a, for_backward=True, prune=prune, share_groups=share)
+        grads = ops.fused_backward(*a, O, lse, dev["dO"], ws=ws, prune=prune, share_groups=share)
+        g2 = ops.fused_backward(*a, O, lse, dev["dO"], ws=None, prune=prune, share_groups=share)
+        torch.cuda.synchronize()
+        res[share] = (O, lse) + tuple(grads)
+        for x, y in zip(grads, g2):
+            assert rel_err(y, x) <= 1e-3
+        res[share, "bytes"] = ws.numel()
+    assert res[True, "bytes"] < res[False, "bytes"]       # separate sweeps keep the key-side sums per query head
+    assert torch.equal(res[False][0], res[True][0]) and torch.equal(res[False][1], res[True][1])
+    O_ref, lse_ref, g_ref = dense_reference(inp)
+    for share in (False, True):
+        for k, g, gr in zip(NAMES, res[share][2:], g_ref):
+            assert rel_err(g.reshape(gr.shape), gr) <= TOL[dtype], (share, k, rel_err(g.reshape(gr.shape), gr))
+    for name, x, y in zip(("dk", "dv", "dq", "dsrc", "ddest"), res[False][2:], res[True][2:]):
+        assert rel_err(y, x) <= 6e-3, (name, rel_err(y, x))
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("case", ["L1", "L16", "L17_ragged", "gates_near_one", "gates_near_zero", "identical_keys", "orthogonal_keys"])
 def test_edge_cases_of_the_inputs(case, dtype):

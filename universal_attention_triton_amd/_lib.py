@@ -15,6 +15,7 @@ UA_OP_FWD, UA_OP_BWD, UA_OP_FUSED_FWD, UA_OP_FUSED_BWD = 0, 1, 2, 3
 UA_FLAG_SKIP_MASKED = 1
 UA_FLAG_RECOMPUTE = 4
 UA_FLAG_PRUNE = 2
+UA_FLAG_SHARE_GROUPS = 8
 
 c_void_p, c_int, c_size_t, c_int64, c_int32 = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_int64, ctypes.c_int32
 

@@ -44,6 +44,7 @@ struct BwdArgs {
   const _Float16* Bt;           // with dS_st: fp16 bias tiles of k_carry2<BO>, [Zk][triangle, see tri_bias_row][1 KB]
   int R, L, Lp, c, nch, chunked, skip_masked;
   int split_r;                  // k_bwd_queries2: one workgroup per (kv head, query group); dKdacc is then [Zq][Lp][D]
+  int split_keys;               // k_bwd_keys2<!MR>: likewise; dKrow, dVrow, dsrc_raw and dG_st then hold one slice per query head
 };
 
 // grid (key groups, Zk).  chunked == 0: key group = 128 consecutive keys, 4 waves.
@@ -282,7 +283,7 @@ __global__ void __launch_bounds__(256) k_bwd_finish(const float* __restrict__ dK
                                                     const T* __restrict__ src, const T* __restrict__ dest,
                                                     T* __restrict__ dk, T* __restrict__ dv, T* __restrict__ dq,
                                                     T* __restrict__ dsrc, T* __restrict__ ddest, int Zk, int Zq, int L,
-                                                    int Lp, int D, int d, int tiled, int RS) {
+                                                    int Lp, int D, int d, int tiled, int RS, int RK) {
   const int z = blockIdx.y, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + wave;
   if (t >= L) return;
@@ -300,14 +301,23 @@ __global__ void __launch_bounds__(256) k_bwd_finish(const float* __restrict__ dK
       // the packed keys are row-major in chunked mode and tiled (nat_off) in fused mode
       const long ik = !tiled ? i : (D == 64 ? nat_off<64>(z, Lp, t, c) : nat_off<128>(z, Lp, t, c));
       dot += kd * (float)Kp[ik];
-      dk[((long)z * L + t) * d + c] = cvt<T>(dKrow[i] + kd);
-      dv[((long)z * L + t) * d + c] = cvt<T>(dVrow[i]);
+      // RK > 1: so does the row side, and dV
+      float kr = 0.f, vr = 0.f;
+      for (int r = 0; r < RK; ++r) {
+        const long ir = (((long)z * RK + r) * Lp + t) * D + c;
+        kr += dKrow[ir];
+        vr += dVrow[ir];
+      }
+      dk[((long)z * L + t) * d + c] = cvt<T>(kr + kd);
+      dv[((long)z * L + t) * d + c] = cvt<T>(vr);
     }
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) dot += __shfl_xor(dot, m, 64);
     if (lane == 0) {
       ddest[(long)z * L + t] = cvt<T>(dot / (2.0f * sd));
-      dsrc[(long)z * L + t] = cvt<T>(dsrc_raw[(long)z * Lp + t] / (3.0f * (float)src[(long)z * L + t]));
+      float sr = 0.f;
+      for (int r = 0; r < RK; ++r) sr += dsrc_raw[((long)z * RK + r) * Lp + t];
+      dsrc[(long)z * L + t] = cvt<T>(sr / (3.0f * (float)src[(long)z * L + t]));
     }
   }
 }

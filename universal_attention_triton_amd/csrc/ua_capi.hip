@@ -39,6 +39,7 @@ struct Layout {
   size_t dOp, dOT, delta, dQacc, dKdacc, Dsuf, dKrow, dVrow, dsrc_raw, masked_nz, dS_st, dG_st, total;
   bool tiles;       // bf16 merged operator: bias, dS and dG tiles are exchanged through the workspace
   bool grad_tiles;  // ... dS and dG tiles (also the chunked operator with a chunk that is a multiple of 64)
+  bool split_keys;  // key side of the backward: one sweep per query head instead of per kv head (see make_layout)
 };
 
 int check_desc(const ua_desc* d, bool chunked) {
@@ -94,11 +95,18 @@ Layout make_layout(const ua_desc& d, bool chunked) {
   l.masked_nz = take(256);
   // score and decay gradients of every (32 keys, 16 queries) tile
   l.grad_tiles = l.tiles || (chunked && d.chunk % 64 == 0 && d.dtype == UA_BF16 && !(d.flags & UA_FLAG_RECOMPUTE));
+  // Grouped queries with few kv heads: the key-stationary kernel's longest workgroup sweeps Lp/32 * r steps while the
+  // device-wide average is Zk * (Lp/128) / CUs times half of that, so with fewer than about 1.5 workgroups per CU (256
+  // CUs) the launch waits for that one workgroup.  Each query group then gets a sweep of its own (r times the
+  // workgroups, a longest one r times shorter, the key-key part of a step repeated per group) and the key-side sums are
+  // kept per query head.  UA_FLAG_SHARE_GROUPS keeps the shared sweep.
+  l.split_keys = l.tiles && d.r > 1 && !(d.flags & UA_FLAG_SHARE_GROUPS) && (long)l.Zk * (l.Lp / 128) <= 384;
+  const size_t Zs = l.split_keys ? l.Zq : l.Zk;
   l.dS_st = l.grad_tiles ? take((size_t)l.Zq * sq) : 0;
-  l.dG_st = l.grad_tiles ? take((size_t)l.Zk * sq) : 0;
-  l.dKrow = take((size_t)l.Zk * l.Lp * l.D * 4);
-  l.dVrow = take((size_t)l.Zk * l.Lp * l.D * 4);
-  l.dsrc_raw = take((size_t)l.Zk * l.Lp * 4);
+  l.dG_st = l.grad_tiles ? take(Zs * sq) : 0;
+  l.dKrow = take(Zs * l.Lp * l.D * 4);
+  l.dVrow = take(Zs * l.Lp * l.D * 4);
+  l.dsrc_raw = take(Zs * l.Lp * 4);
   l.total = off;
   return l;
 }
@@ -265,7 +273,8 @@ hipError_t finish_t(const Layout& l, const ua_desc& d, char* ws, bool chunked, c
   hipLaunchKernelGGL((ua::k_bwd_finish<T>), dim3((d.L + 3) / 4, Z), dim3(256), 0, s, (const float*)(ws + l.dKrow),
                      (const float*)(ws + l.dVrow), (const float*)(ws + l.dKdacc), chunked ? (const float*)(ws + l.dQacc) : nullptr,
                      (const float*)(ws + l.dsrc_raw), (const T*)(ws + l.Kp), (const T*)src, (const T*)dest, (T*)dk, (T*)dv,
-                     (T*)dq, (T*)dsrc, (T*)ddest, l.Zk, l.Zq, d.L, l.Lp, l.D, d.d, chunked ? 0 : 1, chunked ? 1 : d.r);
+                     (T*)dq, (T*)dsrc, (T*)ddest, l.Zk, l.Zq, d.L, l.Lp, l.D, d.d, chunked ? 0 : 1, chunked ? 1 : d.r,
+                     l.split_keys ? d.r : 1);
   return hipGetLastError();
 }
 
@@ -301,6 +310,7 @@ int run_bwd_common(const ua_desc& d, const Layout& l, char* ws, bool chunked, co
   a.R = d.r; a.L = d.L; a.Lp = l.Lp; a.c = is_chunked ? d.chunk : 128; a.nch = l.nch; a.chunked = is_chunked ? 1 : 0;
   a.skip_masked = (d.flags & UA_FLAG_SKIP_MASKED) ? 1 : 0;
   a.split_r = (!chunked && d.r > 1) ? 1 : 0;
+  a.split_keys = l.split_keys ? 1 : 0;
   {
     UA_PROF("k_bwd_keys", s);
     UA_HIP(ua::launch_bwd_keys(d.dtype, l.D, a, l.Zk, chunked ? 1 : 0, s));

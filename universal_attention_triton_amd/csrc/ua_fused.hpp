@@ -592,8 +592,14 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   // (CH) followed by [lse2: 32f][delta: 32f] of the second chunk
   UA_STAGES(SB);
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
-  int bx, zk;
-  xcd_map(bx, zk);
+  // grid y: kv heads (MR: the query groups of a head are swept one after the other, sharing the key-key part of a
+  // step), or, with a.split_keys, query heads: one workgroup per (kv head, query group), each a sweep of its own whose
+  // key-side sums land in slice zo of dKrow / dVrow / dsrc_raw / dG_st (k_bwd_finish and k_bwd_queries3 add them up).
+  // That repeats the key-key part per group but cuts the longest workgroup of the launch by the factor r, which is
+  // what bounds the launch when there are few kv heads.
+  int bx, zo;
+  xcd_map(bx, zo);
+  const int zk = (!MR && a.split_keys) ? zo / a.R : zo;
   const int Lp = a.Lp, L = a.L, nT16 = Lp / 16, R = MR ? a.R : 1;
   const int kg = bx, sb16 = 8 * kg + w, spos = 16 * sb16 + col;      // key group 0 sweeps the most query blocks: first
   const int nTr = (L + 31) / 32, first = 4 * kg;
@@ -652,7 +658,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
 #define UA_ISSUE(s, base)                                                                   \
   {                                                                                         \
     const int tb_ = top - (s) / R;                                                          \
-    const long zq_ = (long)zk * R + (s) % R;                                                \
+    const long zq_ = MR ? (long)zk * R + (s) % R : (long)zo;                                \
     const long qo_ = (zq_ * Lp + 32 * tb_) * D;   /* tile base, natural and transposed */      \
     const long zg_ = zq_ * nch + ch0;             /* z index of dO, delta, lse2 */             \
     const long go_ = (zg_ * Lp + 32 * tb_) * D;                                             \
@@ -789,7 +795,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
       const Frag<T> bp = as_operand16<T>(P[0], P[1]), bs = as_operand16<T>(dS[0], dS[1]);
       if constexpr (TO) {     // the two halves of the operand are the two query tiles of the block
         // query tiles 2 tb and 2 tb + 1: their rows start tb + 1 tiles apart
-        char* p = reinterpret_cast<char*>(a.dS_st) + ((long)zk * R + r) * st_head + (tri_grad_row(2 * tb) << 10) + st_lane;
+        char* p = reinterpret_cast<char*>(a.dS_st) + (MR ? (long)zk * R + r : (long)zo) * st_head + (tri_grad_row(2 * tb) << 10) + st_lane;
         __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&bs)[0], reinterpret_cast<u32x2*>(p));
         __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&bs)[1], reinterpret_cast<u32x2*>(p + ((long)(tb + 1) << 10)));
       }
@@ -822,7 +828,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
       dcar += tot;
       const Frag<T> b = as_operand16<T>(dB[0], dB[1]);
       if constexpr (TO) {
-        char* p = reinterpret_cast<char*>(a.dG_st) + (long)zk * st_head + (tri_grad_row(2 * tb) << 10) + st_lane;
+        char* p = reinterpret_cast<char*>(a.dG_st) + (long)zo * st_head + (tri_grad_row(2 * tb) << 10) + st_lane;
         __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&b)[0], reinterpret_cast<u32x2*>(p));
         __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&b)[1], reinterpret_cast<u32x2*>(p + ((long)(tb + 1) << 10)));
       }
@@ -845,11 +851,11 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   {
     float b, af, tot;
     group_scan(dsrc_acc, gm, b, af, tot);
-    if (g == 0) a.dsrc_raw[(long)zk * Lp + spos] = 1.5f * tot;    // sum dA A = 3/2 sum dG G
+    if (g == 0) a.dsrc_raw[(long)zo * Lp + spos] = 1.5f * tot;    // sum dA A = 3/2 sum dG G
   }
 #pragma unroll
   for (int n = 0; n < ND; ++n) {
-    const long o = ((long)zk * Lp + spos) * D + 16 * n + 4 * g;
+    const long o = ((long)zo * Lp + spos) * D + 16 * n + 4 * g;
     *reinterpret_cast<float4*>(a.dVrow + o) = make_float4(dVt[n][0], dVt[n][1], dVt[n][2], dVt[n][3]);
     *reinterpret_cast<float4*>(a.dKrow + o) = make_float4(dKt[n][0], dKt[n][1], dKt[n][2], dKt[n][3]);
   }
@@ -1159,7 +1165,8 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
 // 32-key halves of dS and of dG per step of 64 keys) straight into LDS, where they are read transposed as A
 // operands; the transposed key tiles are shared by the workgroup.  dG belongs to the kv head: with r query groups
 // per head, group r accumulates the feature tiles n = r, r + R, ... of dkcol (its slice of dKdacc holds zeros
-// elsewhere; k_bwd_finish adds the slices).
+// elsewhere; k_bwd_finish adds the slices).  With a.split_keys every query head has a dG of its own (the part of
+// its group) and accumulates all feature tiles.
 // ---------------------------------------------------------------------------------------------
 template <class T, int D, int NST>
 __global__ void __launch_bounds__(512) k_bwd_queries3(BwdArgs<T> a, T* __restrict__ dq, int d) {
@@ -1188,7 +1195,8 @@ __global__ void __launch_bounds__(512) k_bwd_queries3(BwdArgs<T> a, T* __restric
   // this lane's 16 bytes of the wave's tiles of key half h: base + h * 1024
   const long st_head = tri_tiles(Lp >> 5) << 10;
   const char* pS = reinterpret_cast<const char*>(a.dS_st) + (long)zq * st_head + (tri_grad_row(tq) << 10) + 16 * lane;
-  const char* pG = reinterpret_cast<const char*>(a.dG_st) + (long)zk * st_head + (tri_grad_row(tq) << 10) + 16 * lane;
+  const bool own_dg = a.split_keys != 0;
+  const char* pG = reinterpret_cast<const char*>(a.dG_st) + (long)(own_dg ? zq : zk) * st_head + (tri_grad_row(tq) << 10) + 16 * lane;
   const int* reach_z = a.reach + zk * nT16;
 
 #define UA_ISSUE(s, base)                                                                   \
@@ -1223,7 +1231,7 @@ __global__ void __launch_bounds__(512) k_bwd_queries3(BwdArgs<T> a, T* __restric
       for (int n = 0; n < ND; ++n) {
         const Frag<T> kb = ld8(sKT + TT::at(n, col, 0, g));
         mma16(dQ[n], as, kb);
-        if (n % R == r) mma16(dKc[n], ag, kb);
+        if (own_dg || n % R == r) mma16(dKc[n], ag, kb);
       }
     }
   };

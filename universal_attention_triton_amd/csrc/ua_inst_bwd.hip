@@ -14,7 +14,7 @@ static BwdArgs<T> typed(const BwdArgsV& v) {
   a.C = v.C;
   a.dS_st = (T*)v.dS_st; a.dG_st = (T*)v.dG_st; a.Bt = (const _Float16*)v.Bt;
   a.dQacc = v.dQacc; a.dKdacc = v.dKdacc; a.Dsuf = v.Dsuf; a.dKrow = v.dKrow; a.dVrow = v.dVrow; a.dsrc_raw = v.dsrc_raw;
-  a.R = v.R; a.L = v.L; a.Lp = v.Lp; a.c = v.c; a.nch = v.nch; a.chunked = v.chunked; a.skip_masked = v.skip_masked; a.split_r = v.split_r;
+  a.R = v.R; a.L = v.L; a.Lp = v.Lp; a.c = v.c; a.nch = v.nch; a.chunked = v.chunked; a.skip_masked = v.skip_masked; a.split_r = v.split_r; a.split_keys = v.split_keys;
   return a;
 }
 
@@ -54,6 +54,7 @@ template <class T, int D, int NST>
 static hipError_t bwd2_t(const BwdArgsV& v, int Zk, hipStream_t s) {
   const BwdArgs<T> a = typed<T>(v);
   if constexpr (sizeof(T) == 2) {
+    if (v.dS_st && !v.chunked && v.split_keys) return bwd2_mr<T, D, NST, false, false, true>(a, v.Lp, Zk * v.R, s);
     if (v.dS_st && !v.chunked)
       return v.R > 1 ? bwd2_mr<T, D, NST, true, false, true>(a, v.Lp, Zk, s) : bwd2_mr<T, D, NST, false, false, true>(a, v.Lp, Zk, s);
     if (v.dS_st)

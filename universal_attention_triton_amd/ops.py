@@ -125,22 +125,24 @@ def chunked_backward(kc, vc, xq, static_src, static_dest, out, g_out, g_denom, w
     return dk, dv, dq, dsrc, ddest
 
 
-def _fused_flags(prune, recompute):
-    return (_lib.UA_FLAG_PRUNE if prune else 0) | (_lib.UA_FLAG_RECOMPUTE if recompute else 0)
+def _fused_flags(prune, recompute, share_groups=False):
+    return ((_lib.UA_FLAG_PRUNE if prune else 0) | (_lib.UA_FLAG_RECOMPUTE if recompute else 0)
+            | (_lib.UA_FLAG_SHARE_GROUPS if share_groups else 0))
 
 
-def fused_forward(kc, vc, xq, static_src, static_dest, for_backward=False, prune=False, recompute=False):
+def fused_forward(kc, vc, xq, static_src, static_dest, for_backward=False, prune=False, recompute=False, share_groups=False):
     """-> O [b,h,r,l,d], lse [b,h,r,l] (float32), state
 
     prune: skip (key, query) pairs whose softmax weight is provably below 2^-48 because of the accumulated decay
     (UA_FLAG_PRUNE); the backward that receives the returned state follows the same selection.
-    recompute: size the state for a backward that runs with UA_FLAG_RECOMPUTE (pass the same value to fused_backward)."""
+    recompute: size the state for a backward that runs with UA_FLAG_RECOMPUTE (pass the same value to fused_backward).
+    share_groups: likewise for UA_FLAG_SHARE_GROUPS (grouped queries: one key-side sweep per kv head whatever the shape)."""
     kc, vc, xq, src, dest = _prep(kc, vc, xq, static_src, static_dest)
     lib = _lib.load()
     b, h, n, c, d = kc.shape
     r = xq.shape[2]
     L = n * c
-    desc = _desc(kc, xq, False, _fused_flags(prune, recompute))
+    desc = _desc(kc, xq, False, _fused_flags(prune, recompute, share_groups))
     ws = _workspace(desc, _lib.UA_OP_FUSED_BWD if for_backward else _lib.UA_OP_FUSED_FWD, xq.device)
     O = torch.empty(b, h, r, L, d, dtype=xq.dtype, device=xq.device)
     lse = torch.empty(b, h, r, L, dtype=torch.float32, device=xq.device)
@@ -150,7 +152,7 @@ def fused_forward(kc, vc, xq, static_src, static_dest, for_backward=False, prune
     return O, lse, ws
 
 
-def fused_backward(kc, vc, xq, static_src, static_dest, O, lse, dO, ws=None, prune=False, recompute=False):
+def fused_backward(kc, vc, xq, static_src, static_dest, O, lse, dO, ws=None, prune=False, recompute=False, share_groups=False):
     """ws: the state fused_forward returned for the same inputs (skips the recompute and keeps its pruning);
     prune only matters when ws is None.  recompute: UA_FLAG_RECOMPUTE (small workspace, slower; bf16 only)."""
     kc, vc, xq, src, dest = _prep(kc, vc, xq, static_src, static_dest)
@@ -158,7 +160,7 @@ def fused_backward(kc, vc, xq, static_src, static_dest, O, lse, dO, ws=None, pru
     b, h, n, c, d = kc.shape
     r = xq.shape[2]
     L = n * c
-    desc = _desc(kc, xq, False, _fused_flags(prune, recompute))
+    desc = _desc(kc, xq, False, _fused_flags(prune, recompute, share_groups))
     has_fwd = ws is not None
     need = lib.ua_workspace_bytes(ctypes.byref(desc), _lib.UA_OP_FUSED_BWD)
     if ws is None or ws.numel() < need:
