@@ -72,7 +72,7 @@ Layout make_layout(const ua_desc& d, bool chunked) {
   l.Kp = take(kbytes); l.KT = take(kbytes); l.Vp = take(kbytes); l.VT = take(kbytes);
   l.Qp = take(qbytes); l.QT = take(qbytes);
   l.lsrc = take((size_t)l.Zk * l.Lp * 4); l.ldest = take((size_t)l.Zk * l.Lp * 4);
-  l.C = take((size_t)l.Zk * l.nT * l.Lp * 4);
+  const size_t carries = (size_t)l.Zk * l.nT * l.Lp * 4;     // one float per (16-query tile, key)
   l.lse2 = take((size_t)l.Zq * l.nch * l.Lp * 4);
   // pruning state of the fused mode: largest squared row norm of every 32-row block of K and Q, reach of every key
   // tile, first key tile reaching every query block
@@ -82,6 +82,7 @@ Layout make_layout(const ua_desc& d, bool chunked) {
   l.tiles = !chunked && d.dtype == UA_BF16 && !(d.flags & UA_FLAG_RECOMPUTE);
   const size_t sq = (size_t)ua::tri_tiles(l.Lp / 32) * 1024;     // the causal triangle of 1 KB tiles, per head
   l.Bt = l.tiles ? take((size_t)l.Zk * sq) : 0;
+  l.C = l.tiles ? 0 : take(carries);      // the bias tiles replace the forward carries
   l.fwd_end = off;
   const size_t gbytes = (size_t)l.Zq * l.nch * l.Lp * l.D * l.esz;
   l.dOp = take(gbytes); l.dOT = take(gbytes);
@@ -91,7 +92,7 @@ Layout make_layout(const ua_desc& d, bool chunked) {
   const bool atomics = chunked && d.chunk % 64 != 0;
   l.dQacc = atomics ? take((size_t)l.Zq * l.Lp * l.D * 4) : 0;
   l.dKdacc = take((size_t)(atomics ? l.Zk : l.Zq) * l.Lp * l.D * 4);   // one slice per query group without atomics
-  l.Dsuf = atomics ? 0 : take((size_t)l.Zk * l.nT * l.Lp * 4);
+  l.Dsuf = (atomics || l.tiles) ? 0 : take(carries);     // ... and the gradient tiles the suffix carries
   l.masked_nz = take(256);
   // score and decay gradients of every (32 keys, 16 queries) tile
   l.grad_tiles = l.tiles || (chunked && d.chunk % 64 == 0 && d.dtype == UA_BF16 && !(d.flags & UA_FLAG_RECOMPUTE));

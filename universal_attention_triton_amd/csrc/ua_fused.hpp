@@ -673,7 +673,8 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
       if (lane < 8) src_ = a.lse2 + zg_ * Lp + 32 * tb_ + 4 * lane;                         \
       else if (lane < 16) src_ = a.delta + zg_ * Lp + 32 * tb_ + 4 * (lane - 8);            \
       else if (lane < 32) src_ = ldz + 32 * tb_ + 4 * (lane & 7);                           \
-      else src_ = Cz + (long)(2 * tb_) * Lp + 4 * (lane - 32);                              \
+      else src_ = BI ? ldz + 32 * tb_ + 4 * (lane & 7)   /* no carries with bias tiles */      \
+                     : Cz + (long)(2 * tb_) * Lp + 4 * (lane - 32);                         \
       issue_row((base) + TILES, src_);                                                      \
     }                                                                                       \
     if (BI) issue_row((base) + TILES + 1024 + w * 1024, bt_src + (tri_bias_row(tb_) << 10)); \
