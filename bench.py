@@ -46,6 +46,39 @@ def kernel_flops(cfg, name):
     return {"k_carry": 1, "k_fwd_fused": 2 * r, "k_bwd_keys": 2 + 4 * r, "k_bwd_queries": 5 * r}[name] * base
 
 
+def hbm_kernels(cfg, kern):
+    """Achieved GB/s of the kernels of the fused bf16 step whose algorithmic work is moving bytes: bytes they must read and
+    write once (tile tensors of 1 KB tiles over the causal triangle, fp32 partial gradients, packed inputs) over their
+    measured time, against the 8 TB/s of HBM3E."""
+    if cfg["dtype"] != "bf16":
+        return None
+    Zk = cfg["b"] * cfg["h"]
+    Zq = Zk * cfg["r"]
+    L, d = cfg["L"], cfg["d"]
+    Lp, D = -(-L // 128) * 128, 64 if d <= 64 else 128
+    n32 = Lp // 32
+    tri = (n32 * (n32 + 1) + 8) * 1024                     # bytes of one tile tensor per head
+    split = cfg["r"] > 1 and Zk * (Lp // 128) <= 384       # separate key sweeps per query group
+    Zs = Zq if split else Zk
+    rows = lambda Z, width, esz: Z * Lp * width * esz
+    bytes_of = {
+        "k_carry": Zk * tri + rows(Zk, D, 2),
+        "pack_inputs": (2 * Zk + Zq) * (L * d * 2 + 2 * Lp * D * 2),
+    }
+    if cfg["bwd"]:
+        bytes_of.update({
+            "k_bwd_queries": (Zq + Zs) * tri + rows(Zk, D, 2) + Zq * L * d * 2 + rows(Zq, D, 4),
+            "k_bwd_finish": rows(2 * Zs + Zq, D, 4) + rows(Zk, D, 2) + 2 * Zk * L * d * 2,
+            "pack_dO+delta": Zq * (2 * L * d * 2 + 2 * Lp * D * 2),
+        })
+    out = {}
+    for k, nbytes in bytes_of.items():
+        if k in kern and kern[k] > 0:
+            gbs = nbytes / (kern[k] * 1e-3) / 1e9
+            out[k] = {"GB": round(nbytes / 1e9, 3), "GB/s": round(gbs, 1), "frac_of_8TB/s": round(gbs / 8000.0, 3)}
+    return out
+
+
 def cpu_baseline(cfg, index, budget_s=10.0):
     """Oracle forward + backward (merge included) on whole kv heads of the workload, one at a time."""
     from oracle import ua_oracle as orc
@@ -83,6 +116,44 @@ def cpu_baseline(cfg, index, budget_s=10.0):
 MEASURED_TRAFFIC = {(2, "k_bwd_keys"): 8.32e9}
 
 
+def bench_affinity(args, cfg, inp):
+    """The stand-alone decay bias (AffinityScores: k, src, dest -> aff [b,h,L,L]) forward and backward at the config's
+    key shape; both directions are bound by the L x L tensor they write or read."""
+    from universal_attention_triton_amd import ops
+    b, h, L, d = cfg["b"], cfg["h"], cfg["L"], cfg["d"]
+    k = inp["kc"].reshape(b, h, L, d).cuda()
+    src = inp["static_src"].reshape(b, h, L).cuda()
+    dest = inp["static_dest"].reshape(b, h, L).cuda()
+    esz = k.element_size()
+    daff = torch.empty(b, h, L, L, dtype=k.dtype, device="cuda").normal_()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+    t_f = t_b = 0.0
+    for i in range(args.warmup + args.steps):
+        ev[0].record()
+        aff = ops.affinity_forward(k, src, dest)
+        ev[1].record()
+        grads = ops.affinity_backward(k, src, dest, daff)
+        ev[2].record()
+        torch.cuda.synchronize()
+        if i >= args.warmup:
+            t_f += ev[0].elapsed_time(ev[1])
+            t_b += ev[1].elapsed_time(ev[2])
+        del aff, grads
+    t_f /= args.steps
+    t_b /= args.steps
+    nbytes = b * h * L * L * esz
+    gbs_f, gbs_b = nbytes / (t_f * 1e-3) / 1e9, nbytes / (t_b * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "stand-alone decay bias forward+backward", "value": round(t_f + t_b, 4), "unit": "ms", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(t_f + t_b, 4), "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": None, "dtype": cfg["dtype"], "data": "synthetic",
+        "config": {"workload": "AffinityScores forward+backward, keys of BASELINE config %d: b=%d h=%d L=%d d=%d"
+                               % (args.config, b, h, L, d), "forward_ms": round(t_f, 4), "backward_ms": round(t_b, 4),
+                   "backward_GB/s_of_daff": round(gbs_b, 1)},
+        "roofline": {"bound": "hbm", "kernel": "k_aff_fwd", "achieved": round(gbs_f, 1), "peak": 8000.0, "unit": "GB/s",
+                     "frac": round(gbs_f / 8000.0, 4), "traffic": None}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -90,7 +161,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", type=int, default=2)
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--api", choices=["fused", "chunked"], default="fused",
+    ap.add_argument("--api", choices=["fused", "chunked", "affinity"], default="fused",
                     help="fused (default): universal_attention(); chunked: the reference's call sequence "
                          "UniversalAttention.apply + SMVecMatMul.apply, which materialises out[b,h,r,L,d,n]")
     ap.add_argument("--no-pruned", action="store_true",
@@ -115,6 +186,8 @@ def main():
     leaves = [inp[k].cuda().requires_grad_() for k in names]
     dO = inp["dO"].cuda()
 
+    if args.api == "affinity":
+        return bench_affinity(args, cfg, inp)
     if args.api == "chunked":
         import universal_attention_autograd as ref_api
 
@@ -181,6 +254,10 @@ def main():
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
                      "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get((args.config, dom))},
     }
+    if args.api == "fused":
+        hk = hbm_kernels(cfg, kern)
+        if hk:
+            out["config"]["hbm_kernels"] = hk
     if args.api == "chunked":
         out["roofline"] = roof
         out["config"]["workload"] += "; chunked API (reference call sequence, chunk %d)" % cfg["c"]

@@ -137,7 +137,8 @@ int ua_merge_bwd(int dtype, int64_t rows, int32_t L, int32_t d, int32_t n, const
  * (Universal_Attention/triton/affinity_kernel_opt.py:100-127, :130-423, :425-450).  desc: b, h, L, d, dtype (r, chunk and
  * flags are ignored).  k: [b,h,L,d] rows; src, dest: contiguous [b,h,L]; aff / daff: contiguous [b,h,L,L] in the
  * dtype, aff[b,h,t,s] = bias of key s towards query t in natural-log units (0 on the diagonal, -1e12 where s > t).
- * dk contiguous [b,h,L,d]; dsrc, ddest contiguous [b,h,L].  Workspace: ua_affinity_workspace_bytes(desc, backward). */
+ * dk contiguous [b,h,L,d]; dsrc, ddest contiguous [b,h,L].  Workspace: ua_affinity_workspace_bytes(desc, backward).
+ * bf16 with L a multiple of 8: daff must be 16-byte aligned (UA_EINVAL otherwise). */
 size_t ua_affinity_workspace_bytes(const ua_desc* desc, int backward);
 int ua_affinity_fwd(const ua_desc* desc, const ua_rows* k, const void* src, const void* dest, void* aff, void* ws,
                     size_t ws_bytes, ua_stream_t stream);

@@ -8,7 +8,9 @@ from tests.util import TOL, rel_err
 
 pytestmark = pytest.mark.gpu
 
-SHAPES = [(1, 2, 64, 16), (2, 2, 192, 64), (1, 1, 320, 80), (1, 2, 517, 128)]     # b, h, L, d (ragged L, padded d)
+# b, h, L, d (ragged L, padded d).  bf16 with L a multiple of 8 runs the tile-exchanging backward, everything else the one
+# with the float L x L running sum.
+SHAPES = [(1, 2, 64, 16), (2, 2, 192, 64), (1, 1, 320, 80), (1, 2, 517, 128), (1, 2, 1032, 128)]
 
 
 def _inputs(b, h, L, d, dtype, seed):
@@ -41,9 +43,15 @@ def test_affinity_scores_forward_and_backward(shape, dtype):
     # the bias grows to hundreds: a relative bar on the tensor, as everywhere else
     lower = visible[None, None].expand_as(a)
     assert rel_err(a[lower], want.detach()[lower]) <= (TOL[dtype] if dtype == torch.float32 else 4e-3)
+    # dk: (2/3) G^(-1/3) amplifies the float32 rounding of tiny positive key-key products G, and here every pair carries
+    # an upstream gradient of order sqrt(L); the bar follows how far a float32 evaluation of the oracle itself lands
+    # from the float64 one (2e-4 at L = 517, 2e-3 at L = 1032)
+    leaves32 = [x.float().requires_grad_() for x in (k, src, dest)]
+    g32 = torch.autograd.grad(orc.affinity_scores(*leaves32), leaves32, daff.float() * visible)
+    tol_dk = max(TOL[dtype], 4e-4, 3 * rel_err(g32[0], gw[0]))
     for name, got, ref in zip(("dk", "dsrc", "ddest"), grads, gw):
-        tol = TOL[dtype] if name != "dk" else max(TOL[dtype], 4e-4)
-        assert rel_err(got, ref) <= tol, (name, rel_err(got, ref))
+        tol = TOL[dtype] if name != "dk" else tol_dk
+        assert rel_err(got, ref) <= tol, (name, rel_err(got, ref), tol)
 
 
 def test_affinity_scores_agree_with_the_bias_inside_the_fused_operator():

@@ -518,7 +518,7 @@ int ua_merge_bwd(int dtype, int64_t rows, int32_t L, int32_t d, int32_t n, const
 
 // ---- stand-alone decay bias (affinity scores) ------------------------------------------------
 namespace {
-struct AffLayout { int D, Lp, Z; size_t Kp, KT, lsrc, ldest, fwd_end, DL, row, colp, gs_row, gs_col, total; };
+struct AffLayout { int D, Lp, Z; bool tiles; size_t Kp, KT, lsrc, ldest, fwd_end, DL, Wst, row, colp, gs_row, gs_col, total; };
 AffLayout make_aff_layout(const ua_desc& d) {
   AffLayout l{};
   l.D = d.d <= 64 ? 64 : 128;
@@ -531,7 +531,11 @@ AffLayout make_aff_layout(const ua_desc& d) {
   l.Kp = take(kbytes); l.KT = take(kbytes);
   l.lsrc = take((size_t)l.Z * l.Lp * 4); l.ldest = take((size_t)l.Z * l.Lp * 4);
   l.fwd_end = off;
-  l.DL = take((size_t)l.Z * d.L * d.L * 4);
+  // bf16 with rows of daff that can be 16-byte aligned: the backward exchanges bf16 tiles over the causal triangle
+  // (2 bytes per pair) instead of a float L x L running sum
+  l.tiles = d.dtype == UA_BF16 && d.L % 8 == 0;
+  l.DL = l.tiles ? 0 : take((size_t)l.Z * d.L * d.L * 4);
+  l.Wst = l.tiles ? take((size_t)l.Z * ua::tri_tiles(l.Lp / 32) * 1024) : 0;
   l.row = take((size_t)l.Z * l.Lp * l.D * 4); l.colp = take((size_t)l.Z * l.Lp * l.D * 4);
   l.gs_row = take((size_t)l.Z * l.Lp * 4); l.gs_col = take((size_t)l.Z * l.Lp * 4);
   l.total = off;
@@ -586,10 +590,12 @@ int ua_affinity_bwd(const ua_desc* desc, const ua_rows* k, const void* src, cons
   hipStream_t s = (hipStream_t)stream;
   if (!daff || !dk || !dsrc || !ddest) return fail(UA_EINVAL, "null tensor");
   if (int e = aff_prepare(desc, k, src, dest, ws, ws_bytes, true, l, s)) return e;
+  if (l.tiles && (uintptr_t)daff % 16 != 0) return fail(UA_EINVAL, "daff must be 16-byte aligned (bf16, L a multiple of 8)");
   char* w = (char*)ws;
   UA_HIP(ua::launch_aff_bwd(desc->dtype, l.D, w + l.Kp, w + l.KT, (const float*)(w + l.lsrc), (const float*)(w + l.ldest), daff,
                             (float*)(w + l.DL), (float*)(w + l.row), (float*)(w + l.colp), (float*)(w + l.gs_row),
-                            (float*)(w + l.gs_col), src, dest, dk, dsrc, ddest, desc->L, l.Lp, desc->d, l.Z, s));
+                            (float*)(w + l.gs_col), src, dest, dk, dsrc, ddest, desc->L, l.Lp, desc->d, l.Z, s,
+                            l.tiles ? w + l.Wst : nullptr));
   return UA_OK;
 }
 

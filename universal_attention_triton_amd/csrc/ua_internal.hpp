@@ -51,9 +51,10 @@ hipError_t launch_bwd_queries_from_tiles(int D, const BwdArgsV& a, void* dq, int
 // Stand-alone decay bias (affinity scores): aff [Z][L][L] in the dtype; working tensors tiled like the fused operator's.
 hipError_t launch_aff_fwd(int dtype, int D, const void* Kp, const float* lsrc, const float* ldest, void* aff, int L, int Lp, int Z,
                           hipStream_t s);
-// DL [Z][L][L] float scratch; row, colp [Z][Lp][D] and gs_row, gs_col [Z][Lp] float scratch; src, dest: the caller's gates
+// DL [Z][L][L] float scratch; row, colp [Z][Lp][D] and gs_row, gs_col [Z][Lp] float scratch; src, dest: the caller's gates.
+// Wst (bf16, L a multiple of 8, daff 16-byte aligned): [Z][tri_tiles(Lp/32)][1 KB] scratch that replaces DL and gs_col
 hipError_t launch_aff_bwd(int dtype, int D, const void* Kp, const void* KT, const float* lsrc, const float* ldest, const void* daff,
                           float* DL, float* row, float* colp, float* gs_row, float* gs_col, const void* src, const void* dest,
-                          void* dk, void* dsrc, void* ddest, int L, int Lp, int d, int Z, hipStream_t s);
+                          void* dk, void* dsrc, void* ddest, int L, int Lp, int d, int Z, hipStream_t s, void* Wst = nullptr);
 
 }  // namespace ua

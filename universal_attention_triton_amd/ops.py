@@ -280,6 +280,8 @@ def affinity_backward(k, src, dest, daff):
     lib = _lib.load()
     b, h, L, d = k.shape
     daff = daff.to(k.dtype).contiguous()
+    if daff.data_ptr() % 16:        # a contiguous view at an odd offset of its storage
+        daff = daff.clone()
     ws = torch.empty(lib.ua_affinity_workspace_bytes(ctypes.byref(desc), 1), dtype=torch.uint8, device=k.device)
     dk = torch.empty(b, h, L, d, dtype=k.dtype, device=k.device)
     dsrc = torch.empty(b, h, L, dtype=k.dtype, device=k.device)
