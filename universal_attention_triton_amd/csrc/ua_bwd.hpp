@@ -45,6 +45,12 @@ struct BwdArgs {
   int R, L, Lp, c, nch, chunked, skip_masked;
   int split_r;                  // k_bwd_queries2: one workgroup per (kv head, query group); dKdacc is then [Zq][Lp][D]
   int split_keys;               // k_bwd_keys2<!MR>: likewise; dKrow, dVrow, dsrc_raw and dG_st then hold one slice per query head
+  // direct (tile exchange, r = 1): the two kernels write the caller's gradients themselves and k_bwd_finish is not run:
+  // k_bwd_keys2 dv and dsrc, k_bwd_queries3 dk (row side from dKrow + its own column side) and ddest.
+  // dk_out, dv_out [Z][L][d_out]; dsrc_out, ddest_out and the caller's gates src_in, dest_in [Z][L].
+  int direct, d_out;
+  T *dk_out, *dv_out, *dsrc_out, *ddest_out;
+  const T *src_in, *dest_in;
 };
 
 // grid (key groups, Zk).  chunked == 0: key group = 128 consecutive keys, 4 waves.

@@ -312,6 +312,10 @@ int run_bwd_common(const ua_desc& d, const Layout& l, char* ws, bool chunked, co
   a.skip_masked = (d.flags & UA_FLAG_SKIP_MASKED) ? 1 : 0;
   a.split_r = (!chunked && d.r > 1) ? 1 : 0;
   a.split_keys = l.split_keys ? 1 : 0;
+  // merged bf16 operator with one query group: the two kernels write the caller's gradients themselves
+  const bool direct = l.tiles && d.r == 1;
+  a.direct = direct ? 1 : 0; a.d_out = d.d; a.dk_out = dkc; a.dv_out = dvc; a.dsrc_out = dsrc; a.ddest_out = ddest;
+  a.src_in = src; a.dest_in = dest;
   {
     UA_PROF("k_bwd_keys", s);
     UA_HIP(ua::launch_bwd_keys(d.dtype, l.D, a, l.Zk, chunked ? 1 : 0, s));
@@ -322,6 +326,7 @@ int run_bwd_common(const ua_desc& d, const Layout& l, char* ws, bool chunked, co
     if (l.grad_tiles) UA_HIP(ua::launch_bwd_queries_from_tiles(l.D, a, dxq, d.d, l.Zq, s));
     if (!l.tiles) UA_HIP(ua::launch_bwd_queries(d.dtype, l.D, a, dxq, d.d, l.Zk, s));
   }
+  if (direct) return UA_OK;
   UA_PROF("k_bwd_finish", s);
   if (d.dtype == UA_BF16) UA_HIP(finish_t<ua::bf16>(l, d, ws, chunked, src, dest, dkc, dvc, dxq, dsrc, ddest, s));
   else UA_HIP(finish_t<float>(l, d, ws, chunked, src, dest, dkc, dvc, dxq, dsrc, ddest, s));

@@ -852,13 +852,25 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   {
     float b, af, tot;
     group_scan(dsrc_acc, gm, b, af, tot);
-    if (g == 0) a.dsrc_raw[(long)zo * Lp + spos] = 1.5f * tot;    // sum dA A = 3/2 sum dG G
+    if (BI && !MR && a.direct) {      // straight into the caller's tensor: dsrc = sum dA A / (3 src)
+      if (g == 0 && spos < L) a.dsrc_out[(long)zo * L + spos] = cvt<T>(1.5f * tot / (3.0f * (float)a.src_in[(long)zo * L + spos]));
+    } else if (g == 0) {
+      a.dsrc_raw[(long)zo * Lp + spos] = 1.5f * tot;    // sum dA A = 3/2 sum dG G
+    }
   }
+  const bool direct = BI && !MR && a.direct;
 #pragma unroll
   for (int n = 0; n < ND; ++n) {
     const long o = ((long)zo * Lp + spos) * D + 16 * n + 4 * g;
-    *reinterpret_cast<float4*>(a.dVrow + o) = make_float4(dVt[n][0], dVt[n][1], dVt[n][2], dVt[n][3]);
     *reinterpret_cast<float4*>(a.dKrow + o) = make_float4(dKt[n][0], dKt[n][1], dKt[n][2], dKt[n][3]);
+    if (!direct) {
+      *reinterpret_cast<float4*>(a.dVrow + o) = make_float4(dVt[n][0], dVt[n][1], dVt[n][2], dVt[n][3]);
+    } else if (spos < L) {
+      T* dst = a.dv_out + ((long)zo * L + spos) * a.d_out + 16 * n + 4 * g;
+#pragma unroll
+      for (int v = 0; v < 4; ++v)
+        if (16 * n + 4 * g + v < a.d_out) dst[v] = cvt<T>(dVt[n][v]);
+    }
   }
 }
 
@@ -1250,8 +1262,24 @@ __global__ void __launch_bounds__(512) k_bwd_queries3(BwdArgs<T> a, T* __restric
         if (dd < d) dq[((long)zq * L + t) * d + dd] = cvt<T>(dQ[n][v]);
       }
     }
+    if (a.direct) {       // r = 1: dk = row side (k_bwd_keys2) + column side, ddest = (k_u . dkcol_u) / (2 dest_u)
+      float dot = 0.f;
+      if (t < L) {
 #pragma unroll
-    for (int n = 0; n < ND; ++n) a.dKdacc[((long)zq * Lp + t) * D + 16 * n + col] = dKc[n][v];
+        for (int n = 0; n < ND; ++n) {
+          const int dd = 16 * n + col;
+          if (dd < d) {
+            dot = __builtin_fmaf(dKc[n][v], (float)a.Kp[nat_off<D>(zq, Lp, t, dd)], dot);
+            a.dk_out[((long)zq * L + t) * d + dd] = cvt<T>(a.dKrow[((long)zq * Lp + t) * D + dd] + dKc[n][v]);
+          }
+        }
+      }
+      dot = allsum16(dot);
+      if (col == 0 && t < L) a.ddest_out[(long)zq * L + t] = cvt<T>(dot / (2.0f * (float)a.dest_in[(long)zq * L + t]));
+    } else {
+#pragma unroll
+      for (int n = 0; n < ND; ++n) a.dKdacc[((long)zq * Lp + t) * D + 16 * n + col] = dKc[n][v];
+    }
   }
 }
 

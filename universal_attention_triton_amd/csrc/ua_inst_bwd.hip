@@ -15,6 +15,8 @@ static BwdArgs<T> typed(const BwdArgsV& v) {
   a.dS_st = (T*)v.dS_st; a.dG_st = (T*)v.dG_st; a.Bt = (const _Float16*)v.Bt;
   a.dQacc = v.dQacc; a.dKdacc = v.dKdacc; a.Dsuf = v.Dsuf; a.dKrow = v.dKrow; a.dVrow = v.dVrow; a.dsrc_raw = v.dsrc_raw;
   a.R = v.R; a.L = v.L; a.Lp = v.Lp; a.c = v.c; a.nch = v.nch; a.chunked = v.chunked; a.skip_masked = v.skip_masked; a.split_r = v.split_r; a.split_keys = v.split_keys;
+  a.direct = v.direct; a.d_out = v.d_out; a.dk_out = (T*)v.dk_out; a.dv_out = (T*)v.dv_out; a.dsrc_out = (T*)v.dsrc_out;
+  a.ddest_out = (T*)v.ddest_out; a.src_in = (const T*)v.src_in; a.dest_in = (const T*)v.dest_in;
   return a;
 }
 

@@ -15,6 +15,9 @@ struct BwdArgsV {
   void *dS_st, *dG_st;
   const void* Bt;
   int R, L, Lp, c, nch, chunked, skip_masked, split_r, split_keys;
+  int direct, d_out;
+  void *dk_out, *dv_out, *dsrc_out, *ddest_out;
+  const void *src_in, *dest_in;
 };
 
 // Every launcher returns hipGetLastError() after enqueuing.  dtype: 0 fp32, 1 bf16.  D in {64,128}.
