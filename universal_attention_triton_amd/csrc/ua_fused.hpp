@@ -313,7 +313,7 @@ __global__ void __launch_bounds__(256) k_chunk_masked_denom(T* __restrict__ deno
 // product, no affinity chain, no scan).  The two waves that share a 32-query block copy its four key tiles (two each)
 // into one LDS region per step.
 template <class T, int D, int NST, int NW, bool CHUNKED, bool BI = false>
-__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW >= 8 ? NW / 4 : (BI ? 3 : 2), NW >= 8 ? NW / 4 : (BI ? 3 : 2)))) k_fwd_fused2(const T* __restrict__ Qp, const T* __restrict__ Kp,
+__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW >= 8 ? (BI && NST == 1 ? 4 : NW / 4) : (BI ? 3 : 2), NW >= 8 ? (BI && NST == 1 ? 4 : NW / 4) : (BI ? 3 : 2)))) k_fwd_fused2(const T* __restrict__ Qp, const T* __restrict__ Kp,
                                                     const T* __restrict__ VT, const float* __restrict__ lsrc,
                                                     const float* __restrict__ ldest, const float* __restrict__ C,
                                                     T* __restrict__ O, float* __restrict__ lse, float* __restrict__ lse2,

@@ -42,7 +42,7 @@ hipError_t launch_carry(int dtype, int D, const void* Kp, const float* lsrc, con
                                                                const float*, T*, float*, float*, const int*, const int*, \
                                                                int, int, int, int, ChunkOut<T>, const _Float16*);
 #define UA_INST(T, D, NST, NW, CH) UA_INST2(T, D, NST, NW, CH, false)
-UA_INST2(bf16, 64, 1, 4, false, true) UA_INST2(bf16, 128, 1, 4, false, true)
+UA_INST2(bf16, 64, 1, 8, false, true) UA_INST2(bf16, 128, 1, 8, false, true)
 UA_INST(bf16, 64, 1, 8, false) UA_INST(bf16, 64, 2, 8, false) UA_INST(bf16, 64, 2, 12, false) UA_INST(bf16, 64, 2, 16, false)
 UA_INST(bf16, 128, 2, 4, false) UA_INST(bf16, 64, 2, 4, false) UA_INST(bf16, 128, 1, 8, false) UA_INST(bf16, 128, 2, 8, false) UA_INST(bf16, 128, 2, 12, false) UA_INST(bf16, 128, 2, 16, false)
 UA_INST(float, 64, 1, 8, false) UA_INST(float, 128, 1, 8, false)
@@ -65,9 +65,11 @@ static hipError_t fused_bi(const void* Qp, const void* Kp, const void* VT, const
                            const float* C, void* O, float* lse, float* lse2, const int* reach, const int* minkey, int R, int L,
                            int Lp, int d, int Zq, hipStream_t s, const void* Bt) {
   using T = bf16;
-  // 4-wave workgroups with a single LDS stage: three of them share a CU and cover each other's waits (measured
-  // against 8 waves with two stages: 1.20 vs 1.32 ms at b=1 h=32 L=8192 d=128)
-  hipLaunchKernelGGL((k_fwd_fused2<T, D, 1, 4, false, true>), dim3(Lp / 64, Zq), dim3(256), 0, s, (const T*)Qp, (const T*)Kp,
+  // 8-wave workgroups (128 queries) with a single LDS stage, two per CU, which cover each other's waits.  The kernel
+  // is bound by the key / value tiles it pulls from L2 (without those loads it runs 28 % faster), so queries per
+  // workgroup count: same box, b=1 h=32 L=8192 d=128: 1.07 ms, against 1.15 ms for three 4-wave workgroups per CU and
+  // 1.25 ms for one 8-wave workgroup with two stages
+  hipLaunchKernelGGL((k_fwd_fused2<T, D, 1, 8, false, true>), dim3(Lp / 128, Zq), dim3(512), 0, s, (const T*)Qp, (const T*)Kp,
                      (const T*)VT, lsrc, ldest, C, (T*)O, lse, lse2, reach, minkey, R, L, Lp, d, ChunkOut<T>{}, (const _Float16*)Bt);
   return hipGetLastError();
 }
