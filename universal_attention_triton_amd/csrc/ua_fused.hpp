@@ -1174,21 +1174,25 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
 // ---------------------------------------------------------------------------------------------
 // Query side of the backward from the tiles k_bwd_keys2 left (16-bit dtypes, fused mode): pure matrix work.
 //   dQ[t,:] = sum_s dS[s,t] k_s        dkcol[u,:] = sum_s dG[s,u] k_s
-// grid (Lp/128, Zq); 8 waves; wave w owns queries 16*(8*jt+w)..+15 and streams its own row of 1 KB tiles (two
-// 32-key halves of dS and of dG per step of 64 keys) straight into LDS, where they are read transposed as A
+// grid (Lp/128, Zq); 8 waves; wave w owns queries 16*(8*jt+w)..+15 and streams its own row of 1 KB tiles (HV
+// 32-key halves of dS and of dG per step of 32 HV keys) straight into LDS, where they are read transposed as A
 // operands; the transposed key tiles are shared by the workgroup.  dG belongs to the kv head: with r query groups
 // per head, group r accumulates the feature tiles n = r, r + R, ... of dkcol (its slice of dKdacc holds zeros
 // elsewhere; k_bwd_finish adds the slices).  With a.split_keys every query head has a dG of its own (the part of
 // its group) and accumulates all feature tiles.
 // ---------------------------------------------------------------------------------------------
-template <class T, int D, int NST>
-__global__ void __launch_bounds__(512) k_bwd_queries3(BwdArgs<T> a, T* __restrict__ dq, int d) {
+// HV: 32-key halves per step.  With one half a stage is 25 KB and two workgroups share a CU (the kernel only moves
+// bytes: more of them in flight, and one workgroup's prologue and epilogue under the other's stream).
+template <class T, int D, int NST, int HV>
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(HV == 1 ? 4 : 2, HV == 1 ? 4 : 2)))
+k_bwd_queries3(BwdArgs<T> a, T* __restrict__ dq, int d) {
   static_assert(sizeof(T) == 2, "tiles are exchanged in 16-bit operand precision");
+  static_assert(HV == 1 || HV == 2, "one or two key halves per step");
   using TT = Tile<T, D, 32>;
   using ST = StageT<T>;
   constexpr int ND = D / 16;
-  // stage: [KT half 0][KT half 1][per wave: dS half 0, dS half 1, dG half 0, dG half 1][reach of the 4 key tiles]
-  constexpr int TILES = 2 * TT::BYTES, WAVE = 4 * ST::BYTES, SB = TILES + 8 * WAVE + 1024;
+  // stage: [KT half 0]([KT half 1])[per wave: dS half 0, (dS half 1,) dG half 0(, dG half 1)][reach of 4 key tiles]
+  constexpr int TILES = HV * TT::BYTES, WAVE = 2 * HV * ST::BYTES, SB = TILES + 8 * WAVE + 1024;
   UA_STAGES(SB);
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
   int bx, zq;
@@ -1203,8 +1207,8 @@ __global__ void __launch_bounds__(512) k_bwd_queries3(BwdArgs<T> a, T* __restric
 #pragma unroll
   for (int n = 0; n < ND; ++n) { dQ[n] = (f32x4){0, 0, 0, 0}; dKc[n] = (f32x4){0, 0, 0, 0}; }
   const T* KTz = a.KT + (long)zk * D * Lp;
-  const int n_kt = 2 * jt + 2;
-  const int kt_min = (a.minkey[zk * (nT16 >> 1) + 4 * jt] >> 2) & ~1;
+  const int n_kt = (4 * jt + 4) / HV;                  // steps of 32 HV keys
+  const int kt_min = (a.minkey[zk * (nT16 >> 1) + 4 * jt] >> (HV == 2 ? 2 : 1)) & ~1;
   // this lane's 16 bytes of the wave's tiles of key half h: base + h * 1024
   const long st_head = tri_tiles(Lp >> 5) << 10;
   const char* pS = reinterpret_cast<const char*>(a.dS_st) + (long)zq * st_head + (tri_grad_row(tq) << 10) + 16 * lane;
@@ -1214,28 +1218,28 @@ __global__ void __launch_bounds__(512) k_bwd_queries3(BwdArgs<T> a, T* __restric
 
 #define UA_ISSUE(s, base)                                                                   \
   {                                                                                         \
-    const int k0_ = 64 * (s);                                                               \
+    const int k0_ = 32 * HV * (s);                                                          \
     stT.issue((base), KTz + (long)k0_ * D, w);                                              \
-    stT.issue((base) + TT::BYTES, KTz + (long)(k0_ + 32) * D, w);                           \
+    if (HV == 2) stT.issue((base) + TT::BYTES, KTz + (long)(k0_ + 32) * D, w);              \
     char* mine_ = (base) + TILES + w * WAVE;                                                \
-    const long h_ = (long)(2 * (s)) << 10;                                                  \
+    const long h_ = (long)(HV * (s)) << 10;                                                 \
     __builtin_amdgcn_global_load_lds(pS + h_, (lds_ptr_t)mine_, 16, 0, 0);                  \
-    __builtin_amdgcn_global_load_lds(pS + h_ + 1024, (lds_ptr_t)(mine_ + ST::BYTES), 16, 0, 0);     \
-    __builtin_amdgcn_global_load_lds(pG + h_, (lds_ptr_t)(mine_ + 2 * ST::BYTES), 16, 0, 0);        \
-    __builtin_amdgcn_global_load_lds(pG + h_ + 1024, (lds_ptr_t)(mine_ + 3 * ST::BYTES), 16, 0, 0); \
-    if (w == 0) issue_row((base) + TILES + 8 * WAVE, reach_z + 4 * (s));                    \
+    if (HV == 2) __builtin_amdgcn_global_load_lds(pS + h_ + 1024, (lds_ptr_t)(mine_ + ST::BYTES), 16, 0, 0);     \
+    __builtin_amdgcn_global_load_lds(pG + h_, (lds_ptr_t)(mine_ + HV * ST::BYTES), 16, 0, 0);                    \
+    if (HV == 2) __builtin_amdgcn_global_load_lds(pG + h_ + 1024, (lds_ptr_t)(mine_ + 3 * ST::BYTES), 16, 0, 0); \
+    if (w == 0) issue_row((base) + TILES + 8 * WAVE, reach_z + 4 * (HV == 2 ? (s) : (s) >> 1));                  \
   }
 #define UA_COMPUTE(s, base) bq_step((s), (base))
   auto bq_step = [&] __device__ (int kti, char* base) {
     char* mine = base + TILES + w * WAVE;
     const int* rch = reinterpret_cast<const int*>(base + TILES + 8 * WAVE);
 #pragma unroll
-    for (int kq = 0; kq < 2; ++kq) {
+    for (int kq = 0; kq < HV; ++kq) {
       // the half's two 16-key tiles: visited by k_bwd_keys2 (hence written) iff not after the queries and in reach
-      const int sbk = 4 * kti + 2 * kq;
-      const bool live0 = sbk <= tq && rch[2 * kq] >= tbq, live1 = sbk + 1 <= tq && rch[2 * kq + 1] >= tbq;
+      const int sbk = 2 * (HV * kti + kq), ri = HV == 2 ? 2 * kq : 2 * (kti & 1);
+      const bool live0 = sbk <= tq && rch[ri] >= tbq, live1 = sbk + 1 <= tq && rch[ri + 1] >= tbq;
       if (!live0 && !live1) continue;
-      Frag<T> as = ST::get(mine + kq * ST::BYTES, lane), ag = ST::get(mine + (2 + kq) * ST::BYTES, lane);
+      Frag<T> as = ST::get(mine + kq * ST::BYTES, lane), ag = ST::get(mine + (HV + kq) * ST::BYTES, lane);
       // elements 0-3 of an operand are keys of the first tile, 4-7 of the second (perm32)
       if (!live0) { reinterpret_cast<uint2*>(&as)[0] = make_uint2(0, 0); reinterpret_cast<uint2*>(&ag)[0] = make_uint2(0, 0); }
       if (!live1) { reinterpret_cast<uint2*>(&as)[1] = make_uint2(0, 0); reinterpret_cast<uint2*>(&ag)[1] = make_uint2(0, 0); }

@@ -97,13 +97,13 @@ hipError_t launch_bwd_queries(int dtype, int D, const BwdArgsV& a, void* dq, int
   return D == 64 ? bwdq_t<float, 64, 1>(a, dq, d, Zk, s) : bwdq_t<float, 128, 1>(a, dq, d, Zk, s);
 }
 
-template __global__ void k_bwd_queries3<bf16, 64, 2>(BwdArgs<bf16>, bf16*, int);
-template __global__ void k_bwd_queries3<bf16, 128, 2>(BwdArgs<bf16>, bf16*, int);
+template __global__ void k_bwd_queries3<bf16, 64, 2, 1>(BwdArgs<bf16>, bf16*, int);
+template __global__ void k_bwd_queries3<bf16, 128, 2, 1>(BwdArgs<bf16>, bf16*, int);
 hipError_t launch_bwd_queries_from_tiles(int D, const BwdArgsV& v, void* dq, int d, int Zq, hipStream_t s) {
   const BwdArgs<bf16> a = typed<bf16>(v);
   const dim3 grid(v.Lp / 128, Zq);
-  if (D == 64) hipLaunchKernelGGL((k_bwd_queries3<bf16, 64, 2>), grid, dim3(512), 0, s, a, (bf16*)dq, d);
-  else hipLaunchKernelGGL((k_bwd_queries3<bf16, 128, 2>), grid, dim3(512), 0, s, a, (bf16*)dq, d);
+  if (D == 64) hipLaunchKernelGGL((k_bwd_queries3<bf16, 64, 2, 1>), grid, dim3(512), 0, s, a, (bf16*)dq, d);
+  else hipLaunchKernelGGL((k_bwd_queries3<bf16, 128, 2, 1>), grid, dim3(512), 0, s, a, (bf16*)dq, d);
   return hipGetLastError();
 }
 
