@@ -135,6 +135,7 @@ FAST_CHUNK_SHAPES = [  # chunk a multiple of 64: key-/query-stationary kernels; 
     (1, 2, 2, 512, 64, 64),      # query groups, two chunks per 128-key workgroup
     (1, 1, 1, 768, 128, 192),    # chunk boundaries that are not multiples of 128
     (1, 1, 2, 512, 32, 256),     # one chunk spans two workgroups
+    (2, 2, 3, 320, 16, 64),      # L a multiple of 64 but not of 128: a padded 64-key tile beyond the last chunk
 ]
 
 

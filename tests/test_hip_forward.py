@@ -14,6 +14,8 @@ SHAPES = [  # b, h, r, L, d, c
     (1, 2, 1, 384, 128, 128),
     (1, 1, 2, 320, 80, 32),      # L not a multiple of 128, d padded to 128
     (1, 2, 1, 512, 64, 256),
+    (2, 2, 3, 320, 16, 64),      # chunk of 64, L = 5 chunks: the padding up to 384 holds a 64-key tile that belongs to no chunk
+    (1, 1, 1, 192, 32, 192),     # likewise with a single chunk
 ]
 
 

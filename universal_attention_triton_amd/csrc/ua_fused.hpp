@@ -400,7 +400,9 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW
 #define UA_COMPUTE_SLOW(s, base) fwd_tile(n_kt - 1 - (s), (base), TrueC())
   // chunked operator: chunk i is complete, write its normalised result and restart the softmax
   auto flush_chunk = [&] __device__ (int i) __attribute__((always_inline)) {
-    if (live && i <= (16 * tq) / co.c) {     // chunks after this wave's queries are written by k_chunk_masked_*
+    // chunks after this wave's queries are written by k_chunk_masked_*; a key tile of padding beyond the last chunk
+    // (L a multiple of 64 but not of 128) belongs to no chunk
+    if (live && i < co.nch && i <= (16 * tq) / co.c) {
       const bool via_lds = sizeof(T) == 2 && co.vec && co.out;
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
