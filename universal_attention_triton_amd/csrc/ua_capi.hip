@@ -70,7 +70,7 @@ Layout make_layout(const ua_desc& d, bool chunked) {
   auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
   const size_t kbytes = (size_t)l.Zk * l.Lp * l.D * l.esz, qbytes = (size_t)l.Zq * l.Lp * l.D * l.esz;
   l.Kp = take(kbytes); l.KT = take(kbytes); l.Vp = take(kbytes); l.VT = take(kbytes);
-  l.Qp = take(qbytes); l.QT = take(qbytes);
+  l.Qp = take(qbytes);
   l.lsrc = take((size_t)l.Zk * l.Lp * 4); l.ldest = take((size_t)l.Zk * l.Lp * 4);
   const size_t carries = (size_t)l.Zk * l.nT * l.Lp * 4;     // one float per (16-query tile, key)
   l.lse2 = take((size_t)l.Zq * l.nch * l.Lp * 4);
@@ -83,9 +83,12 @@ Layout make_layout(const ua_desc& d, bool chunked) {
   const size_t sq = (size_t)ua::tri_tiles(l.Lp / 32) * 1024;     // the causal triangle of 1 KB tiles, per head
   l.Bt = l.tiles ? take((size_t)l.Zk * sq) : 0;
   l.C = l.tiles ? 0 : take(carries);      // the bias tiles replace the forward carries
+  // transposed queries (and upstream gradient below): read by the key-stationary backward only, which takes its
+  // transposed operands out of the natural tiles when it exchanges tiles
+  l.QT = l.tiles ? 0 : take(qbytes);
   l.fwd_end = off;
   const size_t gbytes = (size_t)l.Zq * l.nch * l.Lp * l.D * l.esz;
-  l.dOp = take(gbytes); l.dOT = take(gbytes);
+  l.dOp = take(gbytes); l.dOT = l.tiles ? 0 : take(gbytes);
   l.delta = take((size_t)l.Zq * l.nch * l.Lp * 4);
   // the key-chunk-stationary backward (chunk not a multiple of 64) adds up dQ through atomics; the other paths keep
   // suffix carries instead
@@ -219,7 +222,8 @@ int pack_inputs(const ua_desc& d, const Layout& l, bool rowmajor, const ua_rows*
   const bool prune = !chunked && (d.flags & UA_FLAG_PRUNE);
   UA_HIP(pack(d.dtype, l.D, K, ws + l.Kp, ws + l.KT, d.d, d.L, l.Lp, l.Zk, mode, s, prune ? (float*)(ws + l.knorm2) : nullptr));
   UA_HIP(pack(d.dtype, l.D, V, ws + l.Vp, ws + l.VT, d.d, d.L, l.Lp, l.Zk, chunked ? TR_PERM16 : TR_NATURAL, s));
-  UA_HIP(pack(d.dtype, l.D, Q, ws + l.Qp, ws + l.QT, d.d, d.L, l.Lp, l.Zq, mode, s, prune ? (float*)(ws + l.qnorm2) : nullptr));
+  UA_HIP(pack(d.dtype, l.D, Q, ws + l.Qp, l.tiles ? nullptr : ws + l.QT, d.d, d.L, l.Lp, l.Zq, mode, s,
+              prune ? (float*)(ws + l.qnorm2) : nullptr));
   const dim3 grid((l.Lp + 255) / 256, l.Zk);
   if (d.dtype == UA_BF16)
     hipLaunchKernelGGL((ua::k_gates<ua::bf16>), grid, dim3(256), 0, s, (const ua::bf16*)src, (const ua::bf16*)dest,
@@ -299,8 +303,8 @@ int run_bwd_common(const ua_desc& d, const Layout& l, char* ws, bool chunked, co
     UA_HIP(zero_fill(ws + l.dKdacc, (size_t)l.Zk * l.Lp * l.D * 4, s));
   }
   ua::BwdArgsV a{};
-  a.Kp = ws + l.Kp; a.Vp = ws + l.Vp; a.KT = ws + l.KT; a.Qp = ws + l.Qp; a.QT = ws + l.QT; a.dOp = ws + l.dOp;
-  a.dOT = ws + l.dOT; a.lsrc = (const float*)(ws + l.lsrc); a.ldest = (const float*)(ws + l.ldest);
+  a.Kp = ws + l.Kp; a.Vp = ws + l.Vp; a.KT = ws + l.KT; a.Qp = ws + l.Qp; a.QT = l.tiles ? nullptr : ws + l.QT; a.dOp = ws + l.dOp;
+  a.dOT = l.tiles ? nullptr : ws + l.dOT; a.lsrc = (const float*)(ws + l.lsrc); a.ldest = (const float*)(ws + l.ldest);
   a.lse2 = (const float*)(ws + l.lse2); a.delta = (const float*)(ws + l.delta); a.C = (const float*)(ws + l.C);
   a.reach = (const int*)(ws + l.reach); a.minkey = (const int*)(ws + l.minkey);
   a.dQacc = (float*)(ws + l.dQacc); a.dKdacc = (float*)(ws + l.dKdacc); a.Dsuf = (float*)(ws + l.Dsuf);
@@ -382,7 +386,7 @@ int ua_fused_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, cons
   const ua::RowsView lsev = contiguous_view(lse, d.L, 1), none = null_view();
   {
     UA_PROF("pack_dO+delta", s);
-    UA_HIP(pack(d.dtype, l.D, dOv, w + l.dOp, w + l.dOT, d.d, d.L, l.Lp, l.Zq, TR_PERM32, s));
+    UA_HIP(pack(d.dtype, l.D, dOv, w + l.dOp, l.tiles ? nullptr : w + l.dOT, d.d, d.L, l.Lp, l.Zq, TR_PERM32, s));
     if (d.dtype == UA_BF16) UA_HIP(delta_t<ua::bf16>(Ov, dOv, none, lsev, (float*)(w + l.delta), (float*)(w + l.lse2), d.d, d.L, l.Lp, l.Zq, s));
     else UA_HIP(delta_t<float>(Ov, dOv, none, lsev, (float*)(w + l.delta), (float*)(w + l.lse2), d.d, d.L, l.Lp, l.Zq, s));
   }

@@ -571,6 +571,23 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW
   }
 }
 
+// The A operand [16 features 16n.. x 32 positions] of a "transposed" product out of the NATURAL tile [32 positions][D]
+// (k-group-major, see Tile): two transposing reads, each turning a block of 4 positions x 16 features (8 bytes per lane:
+// lane i of a 16-lane group supplies position i/4 of the block and features 4(i%4)..+3) into 4 positions of feature i
+// per lane.  The k index follows as_operand16: elements 0-3 are positions 4G..4G+3, elements 4-7 positions 16+4G..+3
+// (G = lane / 16).  The 64 lanes of one read touch 2 x 256 contiguous bytes, i.e. every bank twice, which is what 512
+// bytes cost anyway.
+template <class T>
+__device__ __forceinline__ Frag<T> ld8_tr(const T* tile, int n, int lane) {
+  static_assert(sizeof(T) == 2, "transposing LDS reads are 16-bit");
+  const int i = lane & 15, G = lane >> 4;
+  const char* p = reinterpret_cast<const char*>(tile) + (((2 * n + ((i & 3) >> 1)) * 32 + 4 * G + (i >> 2)) << 4) + 8 * (i & 1);
+  Frag<T> f;
+  reinterpret_cast<v4s16*>(&f)[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s16_t)p);
+  reinterpret_cast<v4s16*>(&f)[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s16_t)(p + 256));
+  return f;
+}
+
 // ---------------------------------------------------------------------------------------------
 // Key-stationary backward (fused mode).  grid (Lp/128, Zk); 8 waves; wave w owns keys 128g+16w..+15 and
 // sweeps the 32-query blocks from the last one down to its own; one (query block, query group) per step.
@@ -588,8 +605,12 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   // merged operator with tile exchange: the bias comes from the fp16 tiles of k_carry2<BO> (a.Bt), one 1 KB tile per wave
   // and step after the stats row (the chunked operator keeps the carries C, and Dsuf for the recomputing query side)
   constexpr bool BI = TO && !CH;
-  constexpr int TILES = (CH ? 4 : 3) * (TN::BYTES + TT::BYTES), SB = TILES + (CH ? 2048 : 1024) + (BI ? 8 * 1024 : 0);
-  // tiles of a stage: Kt, Q, dO | KT, QT, dOT | (CH) dO, dOT of the workgroup's second chunk
+  // ... and the operands of the three products that contract over the block's positions are read out of the natural
+  // tiles with transposing LDS reads (ld8_tr), so the transposed copies are neither staged nor fetched
+  constexpr bool TR = BI;
+  constexpr int TILES = TR ? 3 * TN::BYTES : (CH ? 4 : 3) * (TN::BYTES + TT::BYTES);
+  constexpr int SB = TILES + (CH ? 2048 : 1024) + (BI ? 8 * 1024 : 0);
+  // tiles of a stage: Kt, Q, dO | (!TR) KT, QT, dOT | (CH) dO, dOT of the workgroup's second chunk
   // stats row of a stage: [lse2: 32f][delta: 32f][ldest: 32f][unused: 32f][forward carries of the 128 keys: 128f]
   // (CH) followed by [lse2: 32f][delta: 32f] of the second chunk
   UA_STAGES(SB);
@@ -667,9 +688,11 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
     stN.issue((base), Kz + (long)(32 * tb_) * D, w);                                        \
     stN.issue((base) + TN::BYTES, a.Qp + qo_, w);                                           \
     stN.issue((base) + 2 * TN::BYTES, a.dOp + go_, w);                                      \
-    stT.issue((base) + 3 * TN::BYTES, KTz + (long)(32 * tb_) * D, w);                       \
-    stT.issue((base) + 3 * TN::BYTES + TT::BYTES, a.QT + qo_, w);                           \
-    stT.issue((base) + 3 * TN::BYTES + 2 * TT::BYTES, a.dOT + go_, w);                      \
+    if (!TR) {                                                                              \
+      stT.issue((base) + 3 * TN::BYTES, KTz + (long)(32 * tb_) * D, w);                     \
+      stT.issue((base) + 3 * TN::BYTES + TT::BYTES, a.QT + qo_, w);                         \
+      stT.issue((base) + 3 * TN::BYTES + 2 * TT::BYTES, a.dOT + go_, w);                    \
+    }                                                                                       \
     if (w == 0) {                                                                           \
       const float* src_;                                                                    \
       if (lane < 8) src_ = a.lse2 + zg_ * Lp + 32 * tb_ + 4 * lane;                         \
@@ -803,9 +826,15 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
         __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&bs)[1], reinterpret_cast<u32x2*>(p + ((long)(tb + 1) << 10)));
       }
 #pragma unroll
-      for (int n = 0; n < ND; ++n) mma16(dVt[n], ld8(sdOT + TT::at(n, col, 0, g)), bp);
+      for (int n = 0; n < ND; ++n) {
+        if constexpr (TR) mma16(dVt[n], ld8_tr<T>(sdO, n, lane), bp);
+        else mma16(dVt[n], ld8(sdOT + TT::at(n, col, 0, g)), bp);
+      }
 #pragma unroll
-      for (int n = 0; n < ND; ++n) mma16(dKt[n], ld8(sQT + TT::at(n, col, 0, g)), bs);
+      for (int n = 0; n < ND; ++n) {
+        if constexpr (TR) mma16(dKt[n], ld8_tr<T>(sQ, n, lane), bs);
+        else mma16(dKt[n], ld8(sQT + TT::at(n, col, 0, g)), bs);
+      }
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -836,7 +865,10 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
         __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&b)[1], reinterpret_cast<u32x2*>(p + ((long)(tb + 1) << 10)));
       }
 #pragma unroll
-      for (int n = 0; n < ND; ++n) mma16(dKt[n], ld8(sKT + TT::at(n, col, 0, g)), b);
+      for (int n = 0; n < ND; ++n) {
+        if constexpr (TR) mma16(dKt[n], ld8_tr<T>(sKt, n, lane), b);
+        else mma16(dKt[n], ld8(sKT + TT::at(n, col, 0, g)), b);
+      }
     }
   };
   {
