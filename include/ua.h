@@ -52,8 +52,8 @@ enum {
   UA_FLAG_SHARE_GROUPS = 8, /* bf16 fused ops with r > 1 (and ua_workspace_bytes): the key side of the backward sweeps the r
                               query groups of a kv head inside one workgroup, sharing the key-key part of every step.
                               Without the flag it does so only when there are enough kv heads to fill the device and
-                              otherwise gives every query group a sweep of its own (more workspace: the key-side
-                              partial sums are then kept per query head).  Same results up to summation order. */
+                              otherwise divides the groups into parts with a sweep each (more workspace: the key-side
+                              partial sums are then kept per part).  Same results up to summation order. */
   UA_FLAG_PRUNE = 2        /* fused ops: skip (key, query) pairs whose softmax weight is provably below 2^-48 because
                               of the accumulated decay (no counterpart in the reference, which visits every pair).
                               The bound uses the largest key and query norms of the head; results change by less

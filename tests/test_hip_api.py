@@ -172,12 +172,14 @@ def test_recomputing_and_tile_exchanging_bf16_kernels_agree(shape, prune):
         assert rel_err(y, x) <= 6e-3, (name, rel_err(y, x))
 
 
-@pytest.mark.parametrize("shape", [(1, 2, 4, 512 + 32, 128, 32), (2, 1, 3, 640, 48, 64), (1, 3, 2, 300, 64, 4)])
+@pytest.mark.parametrize("shape", [(1, 2, 4, 512 + 32, 128, 32), (2, 1, 3, 640, 48, 64), (1, 3, 2, 300, 64, 4),
+                                   (4, 16, 4, 512, 32, 64)])      # the last one: two sweeps of two groups per kv head
 @pytest.mark.parametrize("prune", [False, True])
 def test_grouped_queries_shared_and_separate_key_sweeps_agree(shape, prune):
-    """bf16, r > 1: with few kv heads the key side of the backward gives every query group a sweep of its own and adds
-    the partial key gradients up afterwards; UA_FLAG_SHARE_GROUPS keeps one sweep per kv head.  Both must meet the
-    oracle and agree with each other up to bf16 rounding of the per-group decay gradients; the forward is the same."""
+    """bf16, r > 1: with few kv heads the key side of the backward divides the query groups of a kv head into parts
+    with a sweep each (down to one group per sweep) and adds the partial key gradients up afterwards;
+    UA_FLAG_SHARE_GROUPS keeps one sweep per kv head.  Both must meet the oracle and agree with each other up to
+    bf16 rounding of the per-part decay gradients; the forward is the same."""
     from universal_attention_triton_amd import ops
     b, h, r, L, d, c = shape
     dtype = torch.bfloat16

@@ -44,7 +44,7 @@ struct BwdArgs {
   const _Float16* Bt;           // with dS_st: fp16 bias tiles of k_carry2<BO>, [Zk][triangle, see tri_bias_row][1 KB]
   int R, L, Lp, c, nch, chunked, skip_masked;
   int split_r;                  // k_bwd_queries2: one workgroup per (kv head, query group); dKdacc is then [Zq][Lp][D]
-  int split_keys;               // k_bwd_keys2<!MR>: likewise; dKrow, dVrow, dsrc_raw and dG_st then hold one slice per query head
+  int key_parts;                // k_bwd_keys2: sweeps per kv head (1 .. R, a divisor of R); dKrow, dVrow, dsrc_raw and dG_st hold one slice per (kv head, part)
   // direct (tile exchange, r = 1): the two kernels write the caller's gradients themselves and k_bwd_finish is not run:
   // k_bwd_keys2 dv and dsrc, k_bwd_queries3 dk (row side from dKrow + its own column side) and ddest.
   // dk_out, dv_out [Z][L][d_out]; dsrc_out, ddest_out and the caller's gates src_in, dest_in [Z][L].

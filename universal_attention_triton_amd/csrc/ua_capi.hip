@@ -39,7 +39,7 @@ struct Layout {
   size_t dOp, dOT, delta, dQacc, dKdacc, Dsuf, dKrow, dVrow, dsrc_raw, masked_nz, dS_st, dG_st, total;
   bool tiles;       // bf16 merged operator: bias, dS and dG tiles are exchanged through the workspace
   bool grad_tiles;  // ... dS and dG tiles (also the chunked operator with a chunk that is a multiple of 64)
-  bool split_keys;  // key side of the backward: one sweep per query head instead of per kv head (see make_layout)
+  int key_parts;    // key side of the backward: sweeps per kv head, each over r / key_parts query groups (see make_layout)
 };
 
 int check_desc(const ua_desc* d, bool chunked) {
@@ -99,13 +99,25 @@ Layout make_layout(const ua_desc& d, bool chunked) {
   l.masked_nz = take(256);
   // score and decay gradients of every (32 keys, 16 queries) tile
   l.grad_tiles = l.tiles || (chunked && d.chunk % 64 == 0 && d.dtype == UA_BF16 && !(d.flags & UA_FLAG_RECOMPUTE));
-  // Grouped queries with few kv heads: the key-stationary kernel's longest workgroup sweeps Lp/32 * r steps while the
-  // device-wide average is Zk * (Lp/128) / CUs times half of that, so with fewer than about 1.5 workgroups per CU (256
-  // CUs) the launch waits for that one workgroup.  Each query group then gets a sweep of its own (r times the
-  // workgroups, a longest one r times shorter, the key-key part of a step repeated per group) and the key-side sums are
-  // kept per query head.  UA_FLAG_SHARE_GROUPS keeps the shared sweep.
-  l.split_keys = l.tiles && d.r > 1 && !(d.flags & UA_FLAG_SHARE_GROUPS) && (long)l.Zk * (l.Lp / 128) <= 384;
-  const size_t Zs = l.split_keys ? l.Zq : l.Zk;
+  // Grouped queries: the key-stationary kernel sweeps the r query groups of a kv head in one workgroup, sharing the
+  // key-key part of every step (a step of a further group costs about 0.7 of a full one).  Its longest workgroup then
+  // runs Lp/32 * r steps, and with few kv heads the launch waits for it.  The groups can instead be divided into p parts
+  // with a sweep each (p times the workgroups, a longest one p times shorter, the key-key part repeated per part; the
+  // key-side sums are then kept per (kv head, part)).  p = the divisor of r with the smallest estimate
+  // max(longest workgroup, 1.1 x average load of the 256 CUs).  UA_FLAG_SHARE_GROUPS forces p = 1.
+  l.key_parts = 1;
+  if (l.tiles && d.r > 1 && !(d.flags & UA_FLAG_SHARE_GROUPS)) {
+    const double blocks = l.Lp / 32, wgs = (double)l.Zk * (l.Lp / 128);
+    double best = 0;
+    for (int p = 1; p <= d.r; ++p) {
+      if (d.r % p) continue;
+      const double w = 1.0 + 0.7 * (d.r / p - 1);                 // cost of one query block for the groups of a part
+      const double longest = blocks * w, average = 1.1 * wgs * p * (blocks / 2) * w / 256.0;
+      const double cost = longest > average ? longest : average;
+      if (p == 1 || cost < best) { best = cost; l.key_parts = p; }
+    }
+  }
+  const size_t Zs = (size_t)l.Zk * l.key_parts;
   l.dS_st = l.grad_tiles ? take((size_t)l.Zq * sq) : 0;
   l.dG_st = l.grad_tiles ? take(Zs * sq) : 0;
   l.dKrow = take(Zs * l.Lp * l.D * 4);
@@ -279,7 +291,7 @@ hipError_t finish_t(const Layout& l, const ua_desc& d, char* ws, bool chunked, c
                      (const float*)(ws + l.dVrow), (const float*)(ws + l.dKdacc), chunked ? (const float*)(ws + l.dQacc) : nullptr,
                      (const float*)(ws + l.dsrc_raw), (const T*)(ws + l.Kp), (const T*)src, (const T*)dest, (T*)dk, (T*)dv,
                      (T*)dq, (T*)dsrc, (T*)ddest, l.Zk, l.Zq, d.L, l.Lp, l.D, d.d, chunked ? 0 : 1, chunked ? 1 : d.r,
-                     l.split_keys ? d.r : 1);
+                     l.key_parts);
   return hipGetLastError();
 }
 
@@ -315,7 +327,7 @@ int run_bwd_common(const ua_desc& d, const Layout& l, char* ws, bool chunked, co
   a.R = d.r; a.L = d.L; a.Lp = l.Lp; a.c = is_chunked ? d.chunk : 128; a.nch = l.nch; a.chunked = is_chunked ? 1 : 0;
   a.skip_masked = (d.flags & UA_FLAG_SKIP_MASKED) ? 1 : 0;
   a.split_r = (!chunked && d.r > 1) ? 1 : 0;
-  a.split_keys = l.split_keys ? 1 : 0;
+  a.key_parts = l.key_parts;
   // merged bf16 operator with one query group: the two kernels write the caller's gradients themselves
   const bool direct = l.tiles && d.r == 1;
   a.direct = direct ? 1 : 0; a.d_out = d.d; a.dk_out = dkc; a.dv_out = dvc; a.dsrc_out = dsrc; a.ddest_out = ddest;

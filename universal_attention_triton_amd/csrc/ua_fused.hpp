@@ -615,15 +615,16 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   // (CH) followed by [lse2: 32f][delta: 32f] of the second chunk
   UA_STAGES(SB);
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
-  // grid y: kv heads (MR: the query groups of a head are swept one after the other, sharing the key-key part of a
-  // step), or, with a.split_keys, query heads: one workgroup per (kv head, query group), each a sweep of its own whose
-  // key-side sums land in slice zo of dKrow / dVrow / dsrc_raw / dG_st (k_bwd_finish and k_bwd_queries3 add them up).
-  // That repeats the key-key part per group but cuts the longest workgroup of the launch by the factor r, which is
-  // what bounds the launch when there are few kv heads.
+  // grid y: (kv head, part).  The r query groups of a kv head are divided into a.key_parts parts; a workgroup sweeps
+  // the groups of its part one after the other (MR: more than one, sharing the key-key part of a step) and its
+  // key-side sums land in slice zo of dKrow / dVrow / dsrc_raw / dG_st (k_bwd_finish and k_bwd_queries3 add the parts
+  // up).  More parts repeat the key-key part of a step but shorten the longest workgroup of the launch, which is
+  // what bounds it when there are few kv heads.
   int bx, zo;
   xcd_map(bx, zo);
-  const int zk = (!MR && a.split_keys) ? zo / a.R : zo;
-  const int Lp = a.Lp, L = a.L, nT16 = Lp / 16, R = MR ? a.R : 1;
+  const int zk = zo / a.key_parts;
+  const int Lp = a.Lp, L = a.L, nT16 = Lp / 16, R = MR ? a.R / a.key_parts : 1;
+  const long zq0 = (long)zk * a.R + (zo % a.key_parts) * (a.R / a.key_parts);      // first query head of the part
   const int kg = bx, sb16 = 8 * kg + w, spos = 16 * sb16 + col;      // key group 0 sweeps the most query blocks: first
   const int nTr = (L + 31) / 32, first = 4 * kg;
   if (first >= nTr) return;                      // every key of this workgroup is padding
@@ -681,7 +682,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
 #define UA_ISSUE(s, base)                                                                   \
   {                                                                                         \
     const int tb_ = top - (s) / R;                                                          \
-    const long zq_ = MR ? (long)zk * R + (s) % R : (long)zo;                                \
+    const long zq_ = zq0 + (MR ? (s) % R : 0);                                              \
     const long qo_ = (zq_ * Lp + 32 * tb_) * D;   /* tile base, natural and transposed */      \
     const long zg_ = zq_ * nch + ch0;             /* z index of dO, delta, lse2 */             \
     const long go_ = (zg_ * Lp + 32 * tb_) * D;                                             \
@@ -821,7 +822,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
       const Frag<T> bp = as_operand16<T>(P[0], P[1]), bs = as_operand16<T>(dS[0], dS[1]);
       if constexpr (TO) {     // the two halves of the operand are the two query tiles of the block
         // query tiles 2 tb and 2 tb + 1: their rows start tb + 1 tiles apart
-        char* p = reinterpret_cast<char*>(a.dS_st) + (MR ? (long)zk * R + r : (long)zo) * st_head + (tri_grad_row(2 * tb) << 10) + st_lane;
+        char* p = reinterpret_cast<char*>(a.dS_st) + (zq0 + r) * st_head + (tri_grad_row(2 * tb) << 10) + st_lane;
         __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&bs)[0], reinterpret_cast<u32x2*>(p));
         __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&bs)[1], reinterpret_cast<u32x2*>(p + ((long)(tb + 1) << 10)));
       }
@@ -1211,9 +1212,8 @@ __global__ void __launch_bounds__(512) k_bwd_queries2(BwdArgs<T> a, T* __restric
 // grid (Lp/128, Zq); 8 waves; wave w owns queries 16*(8*jt+w)..+15 and streams its own row of 1 KB tiles (HV
 // 32-key halves of dS and of dG per step of 32 HV keys) straight into LDS, where they are read transposed as A
 // operands; the transposed key tiles are shared by the workgroup.  dG belongs to the kv head: with r query groups
-// per head, group r accumulates the feature tiles n = r, r + R, ... of dkcol (its slice of dKdacc holds zeros
-// elsewhere; k_bwd_finish adds the slices).  With a.split_keys every query head has a dG of its own (the part of
-// its group) and accumulates all feature tiles.
+// per head swept together (a part, see k_bwd_keys2: Rl groups share one dG), group r accumulates the feature tiles
+// n = r % Rl, r % Rl + Rl, ... of dkcol (its slice of dKdacc holds zeros elsewhere; k_bwd_finish adds the slices).
 // ---------------------------------------------------------------------------------------------
 // HV: 32-key halves per step.  With one half a stage is 25 KB and two workgroups share a CU (the kernel only moves
 // bytes: more of them in flight, and one workgroup's prologue and epilogue under the other's stream).
@@ -1246,8 +1246,9 @@ k_bwd_queries3(BwdArgs<T> a, T* __restrict__ dq, int d) {
   // this lane's 16 bytes of the wave's tiles of key half h: base + h * 1024
   const long st_head = tri_tiles(Lp >> 5) << 10;
   const char* pS = reinterpret_cast<const char*>(a.dS_st) + (long)zq * st_head + (tri_grad_row(tq) << 10) + 16 * lane;
-  const bool own_dg = a.split_keys != 0;
-  const char* pG = reinterpret_cast<const char*>(a.dG_st) + (long)(own_dg ? zq : zk) * st_head + (tri_grad_row(tq) << 10) + 16 * lane;
+  // dG belongs to the part of the kv head's query groups that was swept together (see k_bwd_keys2): Rl groups
+  const int Rl = R / a.key_parts;
+  const char* pG = reinterpret_cast<const char*>(a.dG_st) + ((long)zk * a.key_parts + r / Rl) * st_head + (tri_grad_row(tq) << 10) + 16 * lane;
   const int* reach_z = a.reach + zk * nT16;
 
 #define UA_ISSUE(s, base)                                                                   \
@@ -1282,7 +1283,7 @@ k_bwd_queries3(BwdArgs<T> a, T* __restrict__ dq, int d) {
       for (int n = 0; n < ND; ++n) {
         const Frag<T> kb = ld8(sKT + TT::at(n, col, 0, g));
         mma16(dQ[n], as, kb);
-        if (own_dg || n % R == r) mma16(dKc[n], ag, kb);
+        if (n % Rl == r % Rl) mma16(dKc[n], ag, kb);
       }
     }
   };

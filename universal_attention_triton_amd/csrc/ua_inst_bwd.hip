@@ -14,7 +14,7 @@ static BwdArgs<T> typed(const BwdArgsV& v) {
   a.C = v.C;
   a.dS_st = (T*)v.dS_st; a.dG_st = (T*)v.dG_st; a.Bt = (const _Float16*)v.Bt;
   a.dQacc = v.dQacc; a.dKdacc = v.dKdacc; a.Dsuf = v.Dsuf; a.dKrow = v.dKrow; a.dVrow = v.dVrow; a.dsrc_raw = v.dsrc_raw;
-  a.R = v.R; a.L = v.L; a.Lp = v.Lp; a.c = v.c; a.nch = v.nch; a.chunked = v.chunked; a.skip_masked = v.skip_masked; a.split_r = v.split_r; a.split_keys = v.split_keys;
+  a.R = v.R; a.L = v.L; a.Lp = v.Lp; a.c = v.c; a.nch = v.nch; a.chunked = v.chunked; a.skip_masked = v.skip_masked; a.split_r = v.split_r; a.key_parts = v.key_parts > 0 ? v.key_parts : 1;
   a.direct = v.direct; a.d_out = v.d_out; a.dk_out = (T*)v.dk_out; a.dv_out = (T*)v.dv_out; a.dsrc_out = (T*)v.dsrc_out;
   a.ddest_out = (T*)v.ddest_out; a.src_in = (const T*)v.src_in; a.dest_in = (const T*)v.dest_in;
   return a;
@@ -56,9 +56,9 @@ template <class T, int D, int NST>
 static hipError_t bwd2_t(const BwdArgsV& v, int Zk, hipStream_t s) {
   const BwdArgs<T> a = typed<T>(v);
   if constexpr (sizeof(T) == 2) {
-    if (v.dS_st && !v.chunked && v.split_keys) return bwd2_mr<T, D, NST, false, false, true>(a, v.Lp, Zk * v.R, s);
     if (v.dS_st && !v.chunked)
-      return v.R > 1 ? bwd2_mr<T, D, NST, true, false, true>(a, v.Lp, Zk, s) : bwd2_mr<T, D, NST, false, false, true>(a, v.Lp, Zk, s);
+      return v.R / a.key_parts > 1 ? bwd2_mr<T, D, NST, true, false, true>(a, v.Lp, Zk * a.key_parts, s)
+                                   : bwd2_mr<T, D, NST, false, false, true>(a, v.Lp, Zk * a.key_parts, s);
     if (v.dS_st)
       return v.R > 1 ? bwd2_mr<T, D, NST, true, true, true>(a, v.Lp, Zk, s) : bwd2_mr<T, D, NST, false, true, true>(a, v.Lp, Zk, s);
   }

@@ -14,7 +14,7 @@ struct BwdArgsV {
   float *dQacc, *dKdacc, *Dsuf, *dKrow, *dVrow, *dsrc_raw;
   void *dS_st, *dG_st;
   const void* Bt;
-  int R, L, Lp, c, nch, chunked, skip_masked, split_r, split_keys;
+  int R, L, Lp, c, nch, chunked, skip_masked, split_r, key_parts;
   int direct, d_out;
   void *dk_out, *dv_out, *dsrc_out, *ddest_out;
   const void *src_in, *dest_in;
@@ -45,7 +45,7 @@ hipError_t launch_fwd_chunked2(int dtype, int D, const void* Qp, const void* Kp,
 // cols != 0: the kernel also produces dQ / dkcol through atomics (chunked mode, row-major working tensors);
 // cols == 0: it records the suffix carries and launch_bwd_queries finishes the query side (tiled working tensors;
 // with a.chunked set: the chunked operator for a chunk that is a multiple of 64).
-// With a.split_keys (bf16 tiles, merged operator) the grid covers the query heads: one sweep per (kv head, query group).
+// With a.key_parts > 1 (bf16 tiles, merged operator) the grid covers (kv head, part of its query groups) pairs.
 hipError_t launch_bwd_keys(int dtype, int D, const BwdArgsV& a, int Zk, int cols, hipStream_t s);
 hipError_t launch_bwd_queries(int dtype, int D, const BwdArgsV& a, void* dq, int d, int Zk, hipStream_t s);
 // bf16 only, a.dS_st / a.dG_st filled by launch_bwd_keys (cols == 0): the query side as pure matrix work over those tiles
