@@ -312,7 +312,10 @@ __global__ void __launch_bounds__(256) k_chunk_masked_denom(T* __restrict__ deno
 // BI (4 or 8 waves): the decay bias comes from the fp16 tiles k_carry2<BO> left in Bt instead of being recomputed (no key-key
 // product, no affinity chain, no scan).  The two waves that share a 32-query block copy its four key tiles (two each)
 // into one LDS region per step.
-template <class T, int D, int NST, int NW, bool CHUNKED, bool BI = false>
+// RB (bias tiles, 8 waves): query groups of one kv head per workgroup.  With grouped queries the RB groups' waves of a
+// 32-query block share the block's key, value and bias tiles: the workgroup then covers 4 / RB blocks of RB heads
+// (grid (Lp / (128 / RB), Zk * R / RB)) instead of 4 blocks of one head.
+template <class T, int D, int NST, int NW, bool CHUNKED, bool BI = false, int RB = 1>
 __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW >= 8 ? (BI && NST == 1 ? 4 : NW / 4) : (BI ? 3 : 2), NW >= 8 ? (BI && NST == 1 ? 4 : NW / 4) : (BI ? 3 : 2)))) k_fwd_fused2(const T* __restrict__ Qp, const T* __restrict__ Kp,
                                                     const T* __restrict__ VT, const float* __restrict__ lsrc,
                                                     const float* __restrict__ ldest, const float* __restrict__ C,
@@ -321,6 +324,7 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW
                                                     int R, int L, int Lp, int d, ChunkOut<T> co,
                                                     const _Float16* __restrict__ Bt = nullptr) {
   static_assert(!BI || ((NW == 8 || NW == 4) && !CHUNKED), "bias tiles: 4 or 8 waves, merged operator");
+  static_assert(RB == 1 || (BI && NW == 8 && (RB == 2 || RB == 4)), "shared blocks: bias tiles, 8 waves, 2 or 4 query groups");
   using TN = Tile<T, 32, D>;
   using TT = Tile<T, D, 32>;
   constexpr int NK = D / 32, ND = D / 16;
@@ -330,12 +334,16 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW
   UA_STAGES(SB);
   __shared__ __attribute__((aligned(256))) char sPbuf[NW * 2 * ST::BYTES];
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
-  int bx, zq;
-  xcd_map(bx, zq);
+  int bx, zy;
+  xcd_map(bx, zy);
+  constexpr int NB = NW / (2 * RB);                          // 32-query blocks per workgroup
+  // wave w: block w / (2 RB) of the workgroup, query group (w / 2) % RB of the workgroup's RB, half w % 2 of the block
+  const int zq = RB == 1 ? zy : (zy / (R / RB)) * R + (zy % (R / RB)) * RB + (w >> 1) % RB;
   const int zk = zq / R, nT16 = Lp / 16;
   const int jt = gridDim.x - 1 - bx;
-  const bool live = NW * jt + w < nT16;                      // the last workgroup may hold waves past the end
-  const int tq = live ? NW * jt + w : nT16 - 1;             // 16-query tile of this wave
+  const int blk = w / (2 * RB), wb = w % (2 * RB), tq_raw = 2 * (NB * jt + blk) + (w & 1);
+  const bool live = tq_raw < nT16;                           // the last workgroup may hold waves past the end
+  const int tq = live ? tq_raw : nT16 - 1;                   // 16-query tile of this wave
   char* sPw = sPbuf + w * 2 * ST::BYTES;     // P of the two 32-key halves of a step
   // chunked operator, 16-bit outputs: per-wave [16 queries][D + 8] tile through which a chunk's result is transposed
   __shared__ __attribute__((aligned(16))) T sObuf[(CHUNKED && sizeof(T) == 2) ? NW * 16 * (D + 8) : 8];
@@ -362,12 +370,12 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW
   f32x4 m = {-1.0e30f, -1.0e30f, -1.0e30f, -1.0e30f}, ls = {0, 0, 0, 0};
   const T* Kz = Kp + (long)zk * Lp * D;
   const T* Vz = VT + (long)zk * D * Lp;
-  const int tq_end = min(NW * (jt + 1), nT16);
+  const int tq_end = min(2 * NB * (jt + 1), nT16);
   const int n_kt = (tq_end + 3) / 4;   // key tiles of 64 covering s <= last query of the workgroup
   // key tiles that cannot reach this workgroup's first query block (see k_carry2) are not visited at all; inside
   // the visited range a tile that does not reach this wave's block gets a carry of -1e30 (its weights become 0)
   const int tbq = tq >> 1;
-  const int kt_min = minkey[zk * (nT16 >> 1) + ((NW * jt) >> 1)] >> 2;
+  const int kt_min = minkey[zk * (nT16 >> 1) + NB * jt] >> 2;
   const int n_steps = n_kt - kt_min;
   // per-wave stats row of a step: [C row: 64f][lsrc: 64f][reach of the 4 key tiles: 4 ints]; source of each lane's
   // 16 bytes as base + step * stride (in 4-byte units)
@@ -387,10 +395,15 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW
     stT.issue((base) + 2 * TN::BYTES, Vz + (long)(2 * kt_) * (32 * D), w);                  \
     stT.issue((base) + 2 * TN::BYTES + TT::BYTES, Vz + (long)(2 * kt_ + 1) * (32 * D), w);  \
     if (BI) {                                                                               \
-      const char* src_ = bt_src + ((long)(4 * kt_ + 2 * (w & 1)) << 10);                    \
-      char* dst_ = (base) + TILES + (w >> 1) * 4096 + (w & 1) * 2048;                       \
-      issue_row(dst_, src_);                                                                \
-      issue_row(dst_ + 1024, src_ + 1024);                                                  \
+      /* the 2 RB waves of a block fetch its four bias tiles: two each, or one each (the first four waves) */ \
+      if (RB == 1) {                                                                        \
+        const char* src_ = bt_src + ((long)(4 * kt_ + 2 * wb) << 10);                       \
+        char* dst_ = (base) + TILES + blk * 4096 + wb * 2048;                               \
+        issue_row(dst_, src_);                                                              \
+        issue_row(dst_ + 1024, src_ + 1024);                                                \
+      } else if (wb < 4) {                                                                  \
+        issue_row((base) + TILES + blk * 4096 + wb * 1024, bt_src + ((long)(4 * kt_ + wb) << 10)); \
+      }                                                                                     \
       if (w == 0) issue_row((base) + TILES + NW * 2048, reach + zk * nT16 + 4 * kt_);        \
     } else {                                                                                \
       issue_row((base) + TILES + w * 1024, row_base + (long)kt_ * row_step);                \
@@ -456,7 +469,7 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW
 #pragma unroll
           for (int q = 0; q < NK; ++q) mma16(sc, qf[q], ld8(sK + TN::at(j & 1, col, q, g)));
           typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
-          const f16x4 hb = *reinterpret_cast<const f16x4*>(base + TILES + (w >> 1) * 4096 + j * 1024 + 16 * lane + 8 * (w & 1));
+          const f16x4 hb = *reinterpret_cast<const f16x4*>(base + TILES + blk * 4096 + j * 1024 + 16 * lane + 8 * (w & 1));
           const bool in_reach = reinterpret_cast<const int*>(base + TILES + NW * 2048)[j] >= tbq;
           const bool diag = MASKED && (sbk == tq);
 #pragma unroll
@@ -541,7 +554,7 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW
   };
   {
     // the key tiles visited first hold the diagonal blocks of the waves
-    const int nslow = min(n_steps, (n_kt - (NW * jt) / 4 + 1) & ~1);
+    const int nslow = min(n_steps, (n_kt - (2 * NB * jt) / 4 + 1) & ~1);
     UA_PIPE_START(n_steps, UA_ISSUE);
     UA_PIPE_RANGE(0, nslow, n_steps, UA_ISSUE, UA_COMPUTE_SLOW);
     UA_PIPE_RANGE(nslow, n_steps, n_steps, UA_ISSUE, UA_COMPUTE_FAST);

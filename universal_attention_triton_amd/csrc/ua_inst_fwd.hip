@@ -37,11 +37,13 @@ hipError_t launch_carry(int dtype, int D, const void* Kp, const float* lsrc, con
 }
 
 // explicit instantiations (the implicit ones are not emitted on the host side for these kernels)
-#define UA_INST2(T, D, NST, NW, CH, BI)                                                                                  \
-  template __global__ void k_fwd_fused2<T, D, NST, NW, CH, BI>(const T*, const T*, const T*, const float*, const float*, \
+#define UA_INST3(T, D, NST, NW, CH, BI, RB)                                                                             \
+  template __global__ void k_fwd_fused2<T, D, NST, NW, CH, BI, RB>(const T*, const T*, const T*, const float*, const float*, \
                                                                const float*, T*, float*, float*, const int*, const int*, \
                                                                int, int, int, int, ChunkOut<T>, const _Float16*);
+#define UA_INST2(T, D, NST, NW, CH, BI) UA_INST3(T, D, NST, NW, CH, BI, 1)
 #define UA_INST(T, D, NST, NW, CH) UA_INST2(T, D, NST, NW, CH, false)
+UA_INST3(bf16, 64, 1, 8, false, true, 2) UA_INST3(bf16, 128, 1, 8, false, true, 2) UA_INST3(bf16, 64, 1, 8, false, true, 4) UA_INST3(bf16, 128, 1, 8, false, true, 4)
 UA_INST2(bf16, 64, 1, 8, false, true) UA_INST2(bf16, 128, 1, 8, false, true) UA_INST2(bf16, 64, 1, 4, false, true) UA_INST2(bf16, 128, 1, 4, false, true)
 UA_INST(bf16, 64, 1, 8, false) UA_INST(bf16, 64, 2, 8, false) UA_INST(bf16, 64, 2, 12, false) UA_INST(bf16, 64, 2, 16, false)
 UA_INST(bf16, 128, 2, 4, false) UA_INST(bf16, 64, 2, 4, false) UA_INST(bf16, 128, 1, 8, false) UA_INST(bf16, 128, 2, 8, false) UA_INST(bf16, 128, 2, 12, false) UA_INST(bf16, 128, 2, 16, false)
@@ -49,6 +51,7 @@ UA_INST(float, 64, 1, 8, false) UA_INST(float, 128, 1, 8, false)
 UA_INST(bf16, 64, 2, 8, true) UA_INST(bf16, 128, 2, 8, true) UA_INST(float, 64, 1, 8, true) UA_INST(float, 128, 1, 8, true)
 #undef UA_INST
 #undef UA_INST2
+#undef UA_INST3
 
 template <class T, int D, int NST, int NW>
 static hipError_t fused_t(const void* Qp, const void* Kp, const void* VT, const float* lsrc, const float* ldest,
@@ -71,12 +74,20 @@ static hipError_t fused_bi(const void* Qp, const void* Kp, const void* VT, const
   // 1.25 ms for one 8-wave workgroup with two stages
   // Small launches (under about six 128-query workgroups per CU) are bound by their longest workgroups instead and
   // run faster in 64-query pieces (config 3: 0.30 vs 0.33 ms; b=2 h=16 L=2048 d=64: 0.075 vs 0.085 ms).
-  if ((long)Zq * (Lp / 128) >= 1536)
+  // grouped queries: the groups of a kv head share the tiles of a 32-query block (see RB)
+#define UA_SHARED(RB_)                                                                                                     \
+  hipLaunchKernelGGL((k_fwd_fused2<T, D, 1, 8, false, true, RB_>), dim3(Lp / (128 / RB_), Zq / RB_), dim3(512), 0, s, (const T*)Qp, \
+                     (const T*)Kp, (const T*)VT, lsrc, ldest, C, (T*)O, lse, lse2, reach, minkey, R, L, Lp, d, ChunkOut<T>{},      \
+                     (const _Float16*)Bt)
+  if (R % 4 == 0) UA_SHARED(4);
+  else if (R % 2 == 0) UA_SHARED(2);
+  else if ((long)Zq * (Lp / 128) >= 1536)
     hipLaunchKernelGGL((k_fwd_fused2<T, D, 1, 8, false, true>), dim3(Lp / 128, Zq), dim3(512), 0, s, (const T*)Qp, (const T*)Kp,
                        (const T*)VT, lsrc, ldest, C, (T*)O, lse, lse2, reach, minkey, R, L, Lp, d, ChunkOut<T>{}, (const _Float16*)Bt);
   else
     hipLaunchKernelGGL((k_fwd_fused2<T, D, 1, 4, false, true>), dim3(Lp / 64, Zq), dim3(256), 0, s, (const T*)Qp, (const T*)Kp,
                        (const T*)VT, lsrc, ldest, C, (T*)O, lse, lse2, reach, minkey, R, L, Lp, d, ChunkOut<T>{}, (const _Float16*)Bt);
+#undef UA_SHARED
   return hipGetLastError();
 }
 // variants (bf16): 0 = 8 waves, double-buffered stages; 1 = 8 waves, single stage; 2 = 12 waves; 3 = 16 waves
