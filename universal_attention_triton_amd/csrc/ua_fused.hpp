@@ -94,8 +94,9 @@ struct FalseC { static constexpr bool value = false; };
 // 16-bit forward and backward kernels then read the bias instead of recomputing the affinity chain; fp16 resolves
 // the bias of every pair that carries weight (|bias| < 16: 2^-7 at worst) to better than the bf16 rounding of the
 // softmax weight itself.
-template <class T, int D, int NST, bool CM, bool BO>
-__global__ void __launch_bounds__(512) k_carry2(const T* __restrict__ Kp, const float* __restrict__ lsrc,
+// NW: waves per workgroup (8, or 4 for launches of few workgroups: twice as many, half as long in LDS and registers).
+template <class T, int D, int NST, bool CM, bool BO, int NW = 8>
+__global__ void __launch_bounds__(64 * NW) k_carry2(const T* __restrict__ Kp, const float* __restrict__ lsrc,
                                                 const float* __restrict__ ldest, float* __restrict__ C, int Lp,
                                                 const float* __restrict__ knorm2, const float* __restrict__ qnorm2, int R,
                                                 int* __restrict__ reach, _Float16* __restrict__ Bt) {
@@ -105,10 +106,10 @@ __global__ void __launch_bounds__(512) k_carry2(const T* __restrict__ Kp, const 
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
   int bx, z;
   xcd_map(bx, z);
-  const int nT = Lp / 32, nT16 = Lp / 16, sb16 = 8 * bx + w, first = 4 * bx;
+  const int nT = Lp / 32, nT16 = Lp / 16, sb16 = NW * bx + w, first = (NW / 2) * bx;
   const int spos = 16 * sb16 + col;
   const GroupMasks gm = group_masks(lane);
-  Stager<TN, 8> st;
+  Stager<TN, NW> st;
   st.init(w, lane, D * (long)sizeof(T), 32);
   Frag<T> ks[NK];
   {
@@ -123,19 +124,19 @@ __global__ void __launch_bounds__(512) k_carry2(const T* __restrict__ Kp, const 
   bool dead = false;
   int last = sb16 >> 1;
   __shared__ int n_dead;
-  __shared__ float red[2][8];
+  __shared__ float red[2][NW];
   float thr = -3.0e38f;
   if (tid == 0) n_dead = 0;
   if (knorm2) {
     float km = 0.f, qm = 0.f;
-    for (int i = tid; i < nT; i += 512) km = fmaxf(km, knorm2[(long)z * nT + i]);
-    for (int i = tid; i < R * nT; i += 512) qm = fmaxf(qm, qnorm2[(long)z * R * nT + i]);
+    for (int i = tid; i < nT; i += 64 * NW) km = fmaxf(km, knorm2[(long)z * nT + i]);
+    for (int i = tid; i < R * nT; i += 64 * NW) qm = fmaxf(qm, qnorm2[(long)z * R * nT + i]);
 #pragma unroll
     for (int m = 1; m <= 32; m <<= 1) { km = fmaxf(km, __shfl_xor(km, m, 64)); qm = fmaxf(qm, __shfl_xor(qm, m, 64)); }
     if (lane == 0) { red[0][w] = km; red[1][w] = qm; }
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < 8; ++i) { km = fmaxf(km, red[0][i]); qm = fmaxf(qm, red[1][i]); }
+    for (int i = 0; i < NW; ++i) { km = fmaxf(km, red[0][i]); qm = fmaxf(qm, red[1][i]); }
     thr = -(kPruneLog2 + 2.0f * kLog2e * sqrtf(km * qm));
   }
   __syncthreads();
@@ -202,14 +203,14 @@ __global__ void __launch_bounds__(512) k_carry2(const T* __restrict__ Kp, const 
       const int s1 = min(total, s0 + 16);
       UA_PIPE_START_AT(s0, s1, UA_ISSUE);
       if (s0 == 0) {
-        const int nslow = s1 < 4 ? s1 : 4;                         // the first four blocks hold the diagonals
+        const int nslow = s1 < NW / 2 ? s1 : NW / 2;               // the first NW / 2 blocks hold the diagonals
         UA_PIPE_RANGE(0, nslow, s1, UA_ISSUE, UA_COMPUTE_SLOW);
         UA_PIPE_RANGE(nslow, s1, s1, UA_ISSUE, UA_COMPUTE_FAST);
       } else {
         UA_PIPE_RANGE(s0, s1, s1, UA_ISSUE, UA_COMPUTE_FAST);
       }
       __syncthreads();
-      if (n_dead == 8) break;
+      if (n_dead == NW) break;
     }
   }
 #undef UA_ISSUE

@@ -17,7 +17,11 @@ static hipError_t carry_t(const void* Kp, const float* lsrc, const float* ldest,
                           const float* knorm2, const float* qnorm2, int R, int* reach, int* minkey, hipStream_t s, void* Bt) {
   constexpr int NST = 2;
   _Float16* none = nullptr;
-  if (tiled && Bt && sizeof(T) == 2) hipLaunchKernelGGL((k_carry2<T, D, NST, true, true>), dim3(Lp / 128, Zk), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, C, Lp, knorm2, qnorm2, R, reach, (_Float16*)Bt);
+  // bias tiles: launches of under two 8-wave workgroups per CU are bound by the latency of a workgroup's serial sweep
+  // and run faster as twice as many 4-wave workgroups
+  if (tiled && Bt && sizeof(T) == 2 && (long)Zk * (Lp / 128) < 512)
+    hipLaunchKernelGGL((k_carry2<T, D, NST, true, true, 4>), dim3(Lp / 64, Zk), dim3(256), 0, s, (const T*)Kp, lsrc, ldest, C, Lp, knorm2, qnorm2, R, reach, (_Float16*)Bt);
+  else if (tiled && Bt && sizeof(T) == 2) hipLaunchKernelGGL((k_carry2<T, D, NST, true, true>), dim3(Lp / 128, Zk), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, C, Lp, knorm2, qnorm2, R, reach, (_Float16*)Bt);
   else if (tiled) hipLaunchKernelGGL((k_carry2<T, D, NST, true, false>), dim3(Lp / 128, Zk), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, C, Lp, knorm2, qnorm2, R, reach, none);
   else hipLaunchKernelGGL((k_carry2<T, D, NST, false, false>), dim3(Lp / 128, Zk), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, C, Lp, knorm2, qnorm2, R, reach, none);
   hipError_t e = hipGetLastError();
