@@ -85,10 +85,12 @@ Layout make_layout(const ua_desc& d, bool chunked) {
   l.C = l.tiles ? 0 : take(carries);      // the bias tiles replace the forward carries
   // transposed queries (and upstream gradient below): read by the key-stationary backward only, which takes its
   // transposed operands out of the natural tiles when it exchanges tiles
-  l.QT = l.tiles ? 0 : take(qbytes);
+  // (so does the chunked backward with a chunk that is a multiple of 64)
+  l.grad_tiles = l.tiles || (chunked && d.chunk % 64 == 0 && d.dtype == UA_BF16 && !(d.flags & UA_FLAG_RECOMPUTE));
+  l.QT = l.grad_tiles ? 0 : take(qbytes);
   l.fwd_end = off;
   const size_t gbytes = (size_t)l.Zq * l.nch * l.Lp * l.D * l.esz;
-  l.dOp = take(gbytes); l.dOT = l.tiles ? 0 : take(gbytes);
+  l.dOp = take(gbytes); l.dOT = l.grad_tiles ? 0 : take(gbytes);
   l.delta = take((size_t)l.Zq * l.nch * l.Lp * 4);
   // the key-chunk-stationary backward (chunk not a multiple of 64) adds up dQ through atomics; the other paths keep
   // suffix carries instead
@@ -97,8 +99,7 @@ Layout make_layout(const ua_desc& d, bool chunked) {
   l.dKdacc = take((size_t)(atomics ? l.Zk : l.Zq) * l.Lp * l.D * 4);   // one slice per query group without atomics
   l.Dsuf = (atomics || l.tiles) ? 0 : take(carries);     // ... and the gradient tiles the suffix carries
   l.masked_nz = take(256);
-  // score and decay gradients of every (32 keys, 16 queries) tile
-  l.grad_tiles = l.tiles || (chunked && d.chunk % 64 == 0 && d.dtype == UA_BF16 && !(d.flags & UA_FLAG_RECOMPUTE));
+  // score and decay gradients of every (32 keys, 16 queries) tile (grad_tiles)
   // Grouped queries: the key-stationary kernel sweeps the r query groups of a kv head in one workgroup, sharing the
   // key-key part of every step (a step of a further group costs about 0.7 of a full one).  Its longest workgroup then
   // runs Lp/32 * r steps, and with few kv heads the launch waits for it.  The groups can instead be divided into p parts
@@ -234,7 +235,7 @@ int pack_inputs(const ua_desc& d, const Layout& l, bool rowmajor, const ua_rows*
   const bool prune = !chunked && (d.flags & UA_FLAG_PRUNE);
   UA_HIP(pack(d.dtype, l.D, K, ws + l.Kp, ws + l.KT, d.d, d.L, l.Lp, l.Zk, mode, s, prune ? (float*)(ws + l.knorm2) : nullptr));
   UA_HIP(pack(d.dtype, l.D, V, ws + l.Vp, ws + l.VT, d.d, d.L, l.Lp, l.Zk, chunked ? TR_PERM16 : TR_NATURAL, s));
-  UA_HIP(pack(d.dtype, l.D, Q, ws + l.Qp, l.tiles ? nullptr : ws + l.QT, d.d, d.L, l.Lp, l.Zq, mode, s,
+  UA_HIP(pack(d.dtype, l.D, Q, ws + l.Qp, l.grad_tiles ? nullptr : ws + l.QT, d.d, d.L, l.Lp, l.Zq, mode, s,
               prune ? (float*)(ws + l.qnorm2) : nullptr));
   const dim3 grid((l.Lp + 255) / 256, l.Zk);
   if (d.dtype == UA_BF16)
@@ -315,8 +316,8 @@ int run_bwd_common(const ua_desc& d, const Layout& l, char* ws, bool chunked, co
     UA_HIP(zero_fill(ws + l.dKdacc, (size_t)l.Zk * l.Lp * l.D * 4, s));
   }
   ua::BwdArgsV a{};
-  a.Kp = ws + l.Kp; a.Vp = ws + l.Vp; a.KT = ws + l.KT; a.Qp = ws + l.Qp; a.QT = l.tiles ? nullptr : ws + l.QT; a.dOp = ws + l.dOp;
-  a.dOT = l.tiles ? nullptr : ws + l.dOT; a.lsrc = (const float*)(ws + l.lsrc); a.ldest = (const float*)(ws + l.ldest);
+  a.Kp = ws + l.Kp; a.Vp = ws + l.Vp; a.KT = ws + l.KT; a.Qp = ws + l.Qp; a.QT = l.grad_tiles ? nullptr : ws + l.QT; a.dOp = ws + l.dOp;
+  a.dOT = l.grad_tiles ? nullptr : ws + l.dOT; a.lsrc = (const float*)(ws + l.lsrc); a.ldest = (const float*)(ws + l.ldest);
   a.lse2 = (const float*)(ws + l.lse2); a.delta = (const float*)(ws + l.delta); a.C = (const float*)(ws + l.C);
   a.reach = (const int*)(ws + l.reach); a.minkey = (const int*)(ws + l.minkey);
   a.dQacc = (float*)(ws + l.dQacc); a.dKdacc = (float*)(ws + l.dKdacc); a.Dsuf = (float*)(ws + l.Dsuf);
@@ -398,7 +399,7 @@ int ua_fused_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, cons
   const ua::RowsView lsev = contiguous_view(lse, d.L, 1), none = null_view();
   {
     UA_PROF("pack_dO+delta", s);
-    UA_HIP(pack(d.dtype, l.D, dOv, w + l.dOp, l.tiles ? nullptr : w + l.dOT, d.d, d.L, l.Lp, l.Zq, TR_PERM32, s));
+    UA_HIP(pack(d.dtype, l.D, dOv, w + l.dOp, l.grad_tiles ? nullptr : w + l.dOT, d.d, d.L, l.Lp, l.Zq, TR_PERM32, s));
     if (d.dtype == UA_BF16) UA_HIP(delta_t<ua::bf16>(Ov, dOv, none, lsev, (float*)(w + l.delta), (float*)(w + l.lse2), d.d, d.L, l.Lp, l.Zq, s));
     else UA_HIP(delta_t<float>(Ov, dOv, none, lsev, (float*)(w + l.delta), (float*)(w + l.lse2), d.d, d.L, l.Lp, l.Zq, s));
   }
@@ -473,7 +474,8 @@ int ua_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
       int* detect = (d.flags & UA_FLAG_SKIP_MASKED) ? nullptr : nz;
       if (d.dtype == UA_BF16) UA_HIP(delta_t<ua::bf16>(outv, gv, gdv, none, (float*)(w + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s, detect, d.chunk));
       else UA_HIP(delta_t<float>(outv, gv, gdv, none, (float*)(w + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s, detect, d.chunk));
-      UA_HIP(pack(d.dtype, l.D, gv, w + l.dOp, w + l.dOT, d.d, d.L, l.Lp, l.Zq * l.nch, TR_PERM32, s, nullptr, nz, d.chunk));
+      UA_HIP(pack(d.dtype, l.D, gv, w + l.dOp, l.grad_tiles ? nullptr : w + l.dOT, d.d, d.L, l.Lp, l.Zq * l.nch, TR_PERM32, s, nullptr, nz,
+                  d.chunk));
     }
     return run_bwd_common(d, l, w, true, static_src, static_dest, dkc, dvc, dxq, dsrc, ddest, s);
   }

@@ -619,10 +619,12 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   // merged operator with tile exchange: the bias comes from the fp16 tiles of k_carry2<BO> (a.Bt), one 1 KB tile per wave
   // and step after the stats row (the chunked operator keeps the carries C, and Dsuf for the recomputing query side)
   constexpr bool BI = TO && !CH;
-  // ... and the operands of the three products that contract over the block's positions are read out of the natural
-  // tiles with transposing LDS reads (ld8_tr), so the transposed copies are neither staged nor fetched
-  constexpr bool TR = BI;
-  constexpr int TILES = TR ? 3 * TN::BYTES : (CH ? 4 : 3) * (TN::BYTES + TT::BYTES);
+  // With the tile exchange the operands of the three products that contract over the block's positions are read out of
+  // the natural tiles with transposing LDS reads (ld8_tr), so the transposed copies are neither staged nor fetched
+  constexpr bool TR = TO;
+  constexpr int TILES = TR ? (CH ? 4 : 3) * TN::BYTES : (CH ? 4 : 3) * (TN::BYTES + TT::BYTES);
+  // offsets of the second chunk's upstream tile (CH), natural and transposed
+  constexpr int DO2 = TR ? 3 * TN::BYTES : 3 * TN::BYTES + 3 * TT::BYTES, DO2T = 4 * TN::BYTES + 3 * TT::BYTES;
   constexpr int SB = TILES + (CH ? 2048 : 1024) + (BI ? 8 * 1024 : 0);
   // tiles of a stage: Kt, Q, dO | (!TR) KT, QT, dOT | (CH) dO, dOT of the workgroup's second chunk
   // stats row of a stage: [lse2: 32f][delta: 32f][ldest: 32f][unused: 32f][forward carries of the 128 keys: 128f]
@@ -719,8 +721,8 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
     }                                                                                       \
     if (BI) issue_row((base) + TILES + 1024 + w * 1024, bt_src + (tri_bias_row(tb_) << 10)); \
     if (CH && two) {                                                                        \
-      stN.issue((base) + 3 * TN::BYTES + 3 * TT::BYTES, a.dOp + go_ + (long)Lp * D, w);     \
-      stT.issue((base) + 4 * TN::BYTES + 3 * TT::BYTES, a.dOT + go_ + (long)Lp * D, w);     \
+      stN.issue((base) + DO2, a.dOp + go_ + (long)Lp * D, w);                               \
+      if (!TR) stT.issue((base) + DO2T, a.dOT + go_ + (long)Lp * D, w);                     \
       if (w == 1) {                                                                         \
         const float* src_ = ((lane & 8) ? a.delta : a.lse2) + (zg_ + 1) * Lp + 32 * tb_ + 4 * (lane & 7); \
         issue_row((base) + TILES + 1024, src_);                                             \
@@ -745,9 +747,10 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   // (universal_attention_autograd.py:27-33) while the gradient still flows through the score:
   //   P = 1/c,  dS = (dP - delta) / c,  no decay part.
   auto uniform_step = [&] __device__ (int s, const char* base) __attribute__((always_inline)) {
-    const T* sdO = reinterpret_cast<const T*>(base + (csel ? 3 * TN::BYTES + 3 * TT::BYTES : 2 * TN::BYTES));
+    const T* sdO = reinterpret_cast<const T*>(base + (csel ? DO2 : 2 * TN::BYTES));
     const T* sQT = reinterpret_cast<const T*>(base + 3 * TN::BYTES + TT::BYTES);
-    const T* sdOT = reinterpret_cast<const T*>(base + (csel ? 4 * TN::BYTES + 3 * TT::BYTES : 3 * TN::BYTES + 2 * TT::BYTES));
+    const T* sdOT = reinterpret_cast<const T*>(base + (csel ? DO2T : 3 * TN::BYTES + 2 * TT::BYTES));
+    const T* sQ = reinterpret_cast<const T*>(base + TN::BYTES);
     const float* qstats = reinterpret_cast<const float*>(base + TILES) + (csel ? 256 : 0);
     f32x4 P[2], dS[2];
 #pragma unroll
@@ -761,9 +764,15 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
     }
     const Frag<T> bp = as_operand16<T>(P[0], P[1]), bs = as_operand16<T>(dS[0], dS[1]);
 #pragma unroll
-    for (int n = 0; n < ND; ++n) mma16(dVt[n], ld8(sdOT + TT::at(n, col, 0, g)), bp);
+    for (int n = 0; n < ND; ++n) {
+      if constexpr (TR) mma16(dVt[n], ld8_tr<T>(sdO, n, lane), bp);
+      else mma16(dVt[n], ld8(sdOT + TT::at(n, col, 0, g)), bp);
+    }
 #pragma unroll
-    for (int n = 0; n < ND; ++n) mma16(dKt[n], ld8(sQT + TT::at(n, col, 0, g)), bs);
+    for (int n = 0; n < ND; ++n) {
+      if constexpr (TR) mma16(dKt[n], ld8_tr<T>(sQ, n, lane), bs);
+      else mma16(dKt[n], ld8(sQT + TT::at(n, col, 0, g)), bs);
+    }
   };
   // MASKED: the step may be the query block that holds this wave's own keys (run-time flag diag)
   auto bwd_step = [&] __device__ (int s, const char* base, auto masked_c, const bool diag) {
@@ -771,10 +780,10 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
     const int tb = top - s / R, r = s % R;
     const T* sKt = reinterpret_cast<const T*>(base);
     const T* sQ = reinterpret_cast<const T*>(base + TN::BYTES);
-    const T* sdO = reinterpret_cast<const T*>(base + (csel ? 3 * TN::BYTES + 3 * TT::BYTES : 2 * TN::BYTES));
+    const T* sdO = reinterpret_cast<const T*>(base + (csel ? DO2 : 2 * TN::BYTES));
     const T* sKT = reinterpret_cast<const T*>(base + 3 * TN::BYTES);
     const T* sQT = reinterpret_cast<const T*>(base + 3 * TN::BYTES + TT::BYTES);
-    const T* sdOT = reinterpret_cast<const T*>(base + (csel ? 4 * TN::BYTES + 3 * TT::BYTES : 3 * TN::BYTES + 2 * TT::BYTES));
+    const T* sdOT = reinterpret_cast<const T*>(base + (csel ? DO2T : 3 * TN::BYTES + 2 * TT::BYTES));
     const float* stats = reinterpret_cast<const float*>(base + TILES);
     const float* qstats = stats + (csel ? 256 : 0);       // lse2 / delta of this wave's chunk
     f32x4 aff_l[2], bias_l[2], gk_l[2], dB_l[2];
