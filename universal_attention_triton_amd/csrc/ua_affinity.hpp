@@ -276,7 +276,7 @@ __global__ void __launch_bounds__(512) k_aff_bwd_keys(const T* __restrict__ Kp, 
     stN.issue(base, Kz + (long)(32 * tb) * D, w);
     stT.issue(base + TN::BYTES, KTz + (long)(32 * tb) * D, w);
     if (32 * tb + drow < L && dcol < L)          // L is a multiple of 8: the piece lies inside the row
-      issue_row(base + TN::BYTES + TT::BYTES + w * 1024, dz + (long)(32 * tb + drow) * L + dcol);
+      issue_row_nt(base + TN::BYTES + TT::BYTES + w * 1024, dz + (long)(32 * tb + drow) * L + dcol);
     if (w == 0) issue_row(base + TN::BYTES + TT::BYTES + DB, ldest + (long)z * Lp + 32 * tb + 4 * (lane & 7));
   };
   issue(0, stage[0]);
@@ -367,8 +367,8 @@ __global__ void __launch_bounds__(512) k_aff_bwd_cols(const T* __restrict__ KT, 
     stT.issue(base + TT::BYTES, KTz + (long)(64 * s + 32) * D, w);
     char* mine = base + TILES + w * WAVE;
     // halves 2 s and 2 s + 1 of this wave's row; a row has (tq >> 1) + 1 of them
-    if (2 * s <= (tq >> 1)) __builtin_amdgcn_global_load_lds(pW + ((long)(2 * s) << 10), (lds_ptr_t)mine, 16, 0, 0);
-    if (2 * s + 1 <= (tq >> 1)) __builtin_amdgcn_global_load_lds(pW + ((long)(2 * s + 1) << 10), (lds_ptr_t)(mine + ST::BYTES), 16, 0, 0);
+    if (2 * s <= (tq >> 1)) issue_row_nt(mine, pW + ((long)(2 * s) << 10));
+    if (2 * s + 1 <= (tq >> 1)) issue_row_nt(mine + ST::BYTES, pW + ((long)(2 * s + 1) << 10));
   };
   issue(0, stage[0]);
   for (int s = 0; s < n_kt; ++s) {

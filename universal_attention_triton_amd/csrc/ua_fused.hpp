@@ -19,6 +19,11 @@ namespace ua {
 __device__ __forceinline__ void issue_row(void* lds_base, const void* src_lane) {
   __builtin_amdgcn_global_load_lds(src_lane, (lds_ptr_t)lds_base, 16, 0, 0);
 }
+// The same for data that is read exactly once (the exchanged tiles): non-temporal, so that it does not displace the
+// operand tiles the workgroups of a head share in L2.
+__device__ __forceinline__ void issue_row_nt(void* lds_base, const void* src_lane) {
+  __builtin_amdgcn_global_load_lds(src_lane, (lds_ptr_t)lds_base, 16, 0, 2);
+}
 
 // Pipeline skeleton.  Every kernel declares two STATIC LDS arrays stage0 / stage1 (distinct objects, so the
 // compiler can prove that the asynchronous loads filling one stage do not alias the reads of the other and
@@ -400,10 +405,10 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW
       if (RB == 1) {                                                                        \
         const char* src_ = bt_src + ((long)(4 * kt_ + 2 * wb) << 10);                       \
         char* dst_ = (base) + TILES + blk * 4096 + wb * 2048;                               \
-        issue_row(dst_, src_);                                                              \
-        issue_row(dst_ + 1024, src_ + 1024);                                                \
+        issue_row_nt(dst_, src_);                                                           \
+        issue_row_nt(dst_ + 1024, src_ + 1024);                                             \
       } else if (wb < 4) {                                                                  \
-        issue_row((base) + TILES + blk * 4096 + wb * 1024, bt_src + ((long)(4 * kt_ + wb) << 10)); \
+        issue_row_nt((base) + TILES + blk * 4096 + wb * 1024, bt_src + ((long)(4 * kt_ + wb) << 10)); \
       }                                                                                     \
       if (w == 0) issue_row((base) + TILES + NW * 2048, reach + zk * nT16 + 4 * kt_);        \
     } else {                                                                                \
@@ -719,7 +724,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
                      : Cz + (long)(2 * tb_) * Lp + 4 * (lane - 32);                         \
       issue_row((base) + TILES, src_);                                                      \
     }                                                                                       \
-    if (BI) issue_row((base) + TILES + 1024 + w * 1024, bt_src + (tri_bias_row(tb_) << 10)); \
+    if (BI) issue_row_nt((base) + TILES + 1024 + w * 1024, bt_src + (tri_bias_row(tb_) << 10)); \
     if (CH && two) {                                                                        \
       stN.issue((base) + DO2, a.dOp + go_ + (long)Lp * D, w);                               \
       if (!TR) stT.issue((base) + DO2T, a.dOT + go_ + (long)Lp * D, w);                     \
@@ -1281,10 +1286,10 @@ k_bwd_queries3(BwdArgs<T> a, T* __restrict__ dq, int d) {
     if (HV == 2) stT.issue((base) + TT::BYTES, KTz + (long)(k0_ + 32) * D, w);              \
     char* mine_ = (base) + TILES + w * WAVE;                                                \
     const long h_ = (long)(HV * (s)) << 10;                                                 \
-    __builtin_amdgcn_global_load_lds(pS + h_, (lds_ptr_t)mine_, 16, 0, 0);                  \
-    if (HV == 2) __builtin_amdgcn_global_load_lds(pS + h_ + 1024, (lds_ptr_t)(mine_ + ST::BYTES), 16, 0, 0);     \
-    __builtin_amdgcn_global_load_lds(pG + h_, (lds_ptr_t)(mine_ + HV * ST::BYTES), 16, 0, 0);                    \
-    if (HV == 2) __builtin_amdgcn_global_load_lds(pG + h_ + 1024, (lds_ptr_t)(mine_ + 3 * ST::BYTES), 16, 0, 0); \
+    issue_row_nt(mine_, pS + h_);                                                                             \
+    if (HV == 2) issue_row_nt(mine_ + ST::BYTES, pS + h_ + 1024);                                        \
+    issue_row_nt(mine_ + HV * ST::BYTES, pG + h_);                                                               \
+    if (HV == 2) issue_row_nt(mine_ + 3 * ST::BYTES, pG + h_ + 1024);                                    \
     if (w == 0) issue_row((base) + TILES + 8 * WAVE, reach_z + 4 * (HV == 2 ? (s) : (s) >> 1));                  \
   }
 #define UA_COMPUTE(s, base) bq_step((s), (base))
