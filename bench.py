@@ -113,7 +113,7 @@ def cpu_baseline(cfg, index, budget_s=10.0):
 # runs of this script, each scaled by what the same counter reads for the plain 1 GiB copy of --calibrate-copy
 # (profiles/bench_cfg2_fused_fwd_bwd.md: 3.74 GB read + 4.58 GB written by k_bwd_keys2).  A measured constant, not
 # collected by a default run; configurations without such a measurement report null.
-MEASURED_TRAFFIC = {(2, "k_bwd_keys"): 7.46e9}
+MEASURED_TRAFFIC = {(2, "k_bwd_keys"): 7.17e9}
 
 
 def bench_affinity(args, cfg, inp):
