@@ -119,8 +119,9 @@ Layout make_layout(const ua_desc& d, bool chunked) {
     }
   }
   const size_t Zs = (size_t)l.Zk * l.key_parts;
-  l.dS_st = l.grad_tiles ? take((size_t)l.Zq * sq) : 0;
-  l.dG_st = l.grad_tiles ? take(Zs * sq) : 0;
+  const size_t sg = (size_t)ua::grp_tiles(l.Lp / 32) * 1024;    // grouped by the consuming workgroup, per head
+  l.dS_st = l.grad_tiles ? take((size_t)l.Zq * sg) : 0;
+  l.dG_st = l.grad_tiles ? take(Zs * sg) : 0;
   l.dKrow = take(Zs * l.Lp * l.D * 4);
   l.dVrow = take(Zs * l.Lp * l.D * 4);
   l.dsrc_raw = take(Zs * l.Lp * 4);

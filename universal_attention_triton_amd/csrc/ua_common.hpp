@@ -233,6 +233,12 @@ __device__ __forceinline__ void xcd_map(int& bx, int& by) {
 __host__ __device__ __forceinline__ constexpr long tri_bias_row(long tb) { return tb * (tb + 1); }
 __host__ __device__ __forceinline__ constexpr long tri_grad_row(long tq) { return (tq >> 1) * ((tq >> 1) + 1) + ((tq & 1) ? (tq >> 1) + 1 : 0); }
 __host__ __device__ __forceinline__ constexpr long tri_tiles(long nT32) { return nT32 * (nT32 + 1) + 8; }
+// The score / decay gradient tiles of the fused operator are grouped by the workgroup that consumes them (k_bwd_queries3:
+// 8 query tiles = 128 queries): group J = tq / 8 holds, for every 32-key half h = 0 .. 4 J + 3, the eight tiles of its
+// query tiles next to one another, so that the eight waves of the consumer read 8 KB contiguous per tensor and step.
+// (Halves beyond a query tile's own diagonal are never written nor used.)
+__host__ __device__ __forceinline__ constexpr long grp_tile(long tq, long h) { return 16 * (tq >> 3) * ((tq >> 3) + 1) + 8 * h + (tq & 7); }
+__host__ __device__ __forceinline__ constexpr long grp_tiles(long nT32) { return 16 * (nT32 >> 2) * ((nT32 >> 2) + 1) + 8; }
 
 __device__ __forceinline__ void wait_async_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 

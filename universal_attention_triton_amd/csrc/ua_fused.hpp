@@ -697,8 +697,8 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   static_assert(!TO || sizeof(T) == 2, "tiles are exchanged in 16-bit operand precision");
   // this lane's 16 bytes of the wave's bias tile of query block 0
   const char* bt_src = reinterpret_cast<const char*>(a.Bt) + (((long)zk * tri_tiles(Lp >> 5) + sb16) << 10) + 16 * lane;
-  const long st_head = tri_tiles(Lp >> 5) << 10;                   // bytes of gradient tiles per head
-  const long st_lane = ((long)(sb16 >> 1) << 10) + StageT<bf16>::addr(perm32(16 * (sb16 & 1) + col), 8 * g);
+  const long st_head = grp_tiles(Lp >> 5) << 10;                   // bytes of gradient tiles per head
+  const long st_lane = StageT<bf16>::addr(perm32(16 * (sb16 & 1) + col), 8 * g);
 
 #define UA_ISSUE(s, base)                                                                   \
   {                                                                                         \
@@ -850,9 +850,9 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
       const Frag<T> bp = as_operand16<T>(P[0], P[1]), bs = as_operand16<T>(dS[0], dS[1]);
       if constexpr (TO) {     // the two halves of the operand are the two query tiles of the block
         // query tiles 2 tb and 2 tb + 1: their rows start tb + 1 tiles apart
-        char* p = reinterpret_cast<char*>(a.dS_st) + (zq0 + r) * st_head + (tri_grad_row(2 * tb) << 10) + st_lane;
+        char* p = reinterpret_cast<char*>(a.dS_st) + (zq0 + r) * st_head + (grp_tile(2 * tb, sb16 >> 1) << 10) + st_lane;
         __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&bs)[0], reinterpret_cast<u32x2*>(p));
-        __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&bs)[1], reinterpret_cast<u32x2*>(p + ((long)(tb + 1) << 10)));
+        __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&bs)[1], reinterpret_cast<u32x2*>(p + 1024));
       }
 #pragma unroll
       for (int n = 0; n < ND; ++n) {
@@ -889,9 +889,9 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
       dcar += tot;
       const Frag<T> b = as_operand16<T>(dB[0], dB[1]);
       if constexpr (TO) {
-        char* p = reinterpret_cast<char*>(a.dG_st) + (long)zo * st_head + (tri_grad_row(2 * tb) << 10) + st_lane;
+        char* p = reinterpret_cast<char*>(a.dG_st) + (long)zo * st_head + (grp_tile(2 * tb, sb16 >> 1) << 10) + st_lane;
         __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&b)[0], reinterpret_cast<u32x2*>(p));
-        __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&b)[1], reinterpret_cast<u32x2*>(p + ((long)(tb + 1) << 10)));
+        __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&b)[1], reinterpret_cast<u32x2*>(p + 1024));
       }
 #pragma unroll
       for (int n = 0; n < ND; ++n) {
@@ -1272,11 +1272,11 @@ k_bwd_queries3(BwdArgs<T> a, T* __restrict__ dq, int d) {
   const int n_kt = (4 * jt + 4) / HV;                  // steps of 32 HV keys
   const int kt_min = (a.minkey[zk * (nT16 >> 1) + 4 * jt] >> (HV == 2 ? 2 : 1)) & ~1;
   // this lane's 16 bytes of the wave's tiles of key half h: base + h * 1024
-  const long st_head = tri_tiles(Lp >> 5) << 10;
-  const char* pS = reinterpret_cast<const char*>(a.dS_st) + (long)zq * st_head + (tri_grad_row(tq) << 10) + 16 * lane;
+  const long st_head = grp_tiles(Lp >> 5) << 10;
+  const char* pS = reinterpret_cast<const char*>(a.dS_st) + (long)zq * st_head + (grp_tile(tq, 0) << 10) + 16 * lane;
   // dG belongs to the part of the kv head's query groups that was swept together (see k_bwd_keys2): Rl groups
   const int Rl = R / a.key_parts;
-  const char* pG = reinterpret_cast<const char*>(a.dG_st) + ((long)zk * a.key_parts + r / Rl) * st_head + (tri_grad_row(tq) << 10) + 16 * lane;
+  const char* pG = reinterpret_cast<const char*>(a.dG_st) + ((long)zk * a.key_parts + r / Rl) * st_head + (grp_tile(tq, 0) << 10) + 16 * lane;
   const int* reach_z = a.reach + zk * nT16;
 
 #define UA_ISSUE(s, base)                                                                   \
@@ -1285,11 +1285,11 @@ k_bwd_queries3(BwdArgs<T> a, T* __restrict__ dq, int d) {
     stT.issue((base), KTz + (long)k0_ * D, w);                                              \
     if (HV == 2) stT.issue((base) + TT::BYTES, KTz + (long)(k0_ + 32) * D, w);              \
     char* mine_ = (base) + TILES + w * WAVE;                                                \
-    const long h_ = (long)(HV * (s)) << 10;                                                 \
+    const long h_ = (long)(HV * (s)) << 13;      /* half h of the group: 8 tiles on */         \
     issue_row_nt(mine_, pS + h_);                                                                             \
-    if (HV == 2) issue_row_nt(mine_ + ST::BYTES, pS + h_ + 1024);                                        \
+    if (HV == 2) issue_row_nt(mine_ + ST::BYTES, pS + h_ + 8192);                                        \
     issue_row_nt(mine_ + HV * ST::BYTES, pG + h_);                                                               \
-    if (HV == 2) issue_row_nt(mine_ + 3 * ST::BYTES, pG + h_ + 1024);                                    \
+    if (HV == 2) issue_row_nt(mine_ + 3 * ST::BYTES, pG + h_ + 8192);                                    \
     if (w == 0) issue_row((base) + TILES + 8 * WAVE, reach_z + 4 * (HV == 2 ? (s) : (s) >> 1));                  \
   }
 #define UA_COMPUTE(s, base) bq_step((s), (base))
