@@ -230,7 +230,7 @@ __global__ void __launch_bounds__(512) k_aff_bwd_side(const T* __restrict__ Kp, 
 // k_aff_bwd_keys is key-stationary like k_aff_bwd_side<false> but sweeps the query blocks from the last one down to
 // its own, carrying the reverse running sum per key (dcar), and reads the (32 queries, 128 keys) block of daff of a step
 // through LDS (rows of 256 bytes, 16 bytes per lane).  It leaves W = dl F as bf16 tiles of 1 KB — (32 keys, 16
-// queries) in the LDS image of StageT, rows of the causal triangle as in BwdArgs::dG_st — and k_aff_bwd_cols, one
+// queries) in the LDS image of StageT, row after row of the causal triangle (tri_grad_row) — and k_aff_bwd_cols, one
 // wave per 16 positions u, turns its row of tiles into the column side sum_s W[s,u] k_s with nothing but matrix products.
 //   grid (Lp/128, Z), 8 waves each.
 // ---------------------------------------------------------------------------------------------

@@ -39,7 +39,7 @@ struct BwdArgs {
   float* dsrc_raw;              // [Zk][Lp]
   // optional (16-bit dtypes, fused mode): k_bwd_keys2 leaves the score gradient dS [Zq] and the decay gradient dG [Zk]
   // of every visited (16 keys, 32 queries) tile, in operand precision, as [z][causal triangle of (16-query tile, 32-key half)
-  // pairs, see tri_grad_row] tiles of 1 KB laid out like StageT (32 keys x 16 queries); k_bwd_queries3 turns them into dQ and the column side of dK
+  // pairs, grouped by eight query tiles, see grp_tile] tiles of 1 KB laid out like StageT (32 keys x 16 queries); k_bwd_queries3 turns them into dQ and the column side of dK
   T *dS_st, *dG_st;
   const _Float16* Bt;           // with dS_st: fp16 bias tiles of k_carry2<BO>, [Zk][triangle, see tri_bias_row][1 KB]
   int R, L, Lp, c, nch, chunked, skip_masked;

@@ -228,6 +228,7 @@ __device__ __forceinline__ void xcd_map(int& bx, int& by) {
 // The tensors of 1 KB tiles the 16-bit kernels exchange only hold the causal triangle, row after row:
 //   bias tiles:      row = 32-query block tb, key tiles j = 0 .. 2 tb + 1          -> the row starts at tile tb (tb + 1)
 //   gradient tiles:  row = 16-query tile tq,  32-key halves h = 0 .. tq / 2        -> the row starts at tile tri_grad_row(tq)
+//                    (stand-alone bias op; the fused operator groups its gradient tiles, see grp_tile)
 // Both triangles have nT32 (nT32 + 1) tiles per head (nT32 = Lp / 32); consumers read whole steps and may run a few tiles
 // past the end of a row (into the next rows; past the last row of a head into the slack).
 __host__ __device__ __forceinline__ constexpr long tri_bias_row(long tb) { return tb * (tb + 1); }
