@@ -39,6 +39,33 @@ def test_descriptor_validation_and_workspace_sizes():
     assert lib.ua_workspace_bytes(ctypes.byref(ok), 9) == 0
 
 
+def test_workspace_follows_the_flags_and_the_group_layout():
+    """Sizing rules of the bf16 fused operator (host logic only): recomputation needs less than the tile exchange; with
+    grouped queries the key-side partial sums are kept per part of a kv head's groups, so the shared sweep
+    (UA_FLAG_SHARE_GROUPS) never needs more, needs less where few kv heads call for several parts (config 3: two), and
+    the same where the kv heads fill the device by themselves; fp32 ignores both flags."""
+    lib = _lib.load()
+
+    def size(b, h, r, L, d, dtype, flags, op=_lib.UA_OP_FUSED_BWD):
+        desc = _lib.UaDesc(b, h, r, L, d, 128, dtype, flags)
+        n = lib.ua_workspace_bytes(ctypes.byref(desc), op)
+        assert n > 0, lib.ua_last_error()
+        return n
+
+    bf, f32 = _lib.UA_BF16, _lib.UA_F32
+    assert size(1, 32, 1, 8192, 128, bf, _lib.UA_FLAG_RECOMPUTE) < size(1, 32, 1, 8192, 128, bf, 0) < 8 << 30
+    few, many = (1, 8, 4, 4096, 128), (1, 64, 4, 4096, 128)
+    assert size(*few, bf, _lib.UA_FLAG_SHARE_GROUPS) < size(*few, bf, 0)
+    assert size(*many, bf, _lib.UA_FLAG_SHARE_GROUPS) == size(*many, bf, 0)
+    # one more slice of the three key-side partial sums and of the decay-gradient tiles per extra part: config 3 has two parts
+    Lp, D, tiles = 4096, 128, 16 * 32 * 33 + 8
+    extra = 8 * (2 * Lp * D * 4 + Lp * 4 + tiles * 1024)
+    assert abs(size(*few, bf, 0) - size(*few, bf, _lib.UA_FLAG_SHARE_GROUPS) - extra) <= 4 * 256
+    for flags in (_lib.UA_FLAG_SHARE_GROUPS, _lib.UA_FLAG_RECOMPUTE):
+        assert size(*few, f32, flags) == size(*few, f32, 0)
+    assert size(*few, bf, 0, _lib.UA_OP_FUSED_FWD) == size(*few, bf, _lib.UA_FLAG_SHARE_GROUPS, _lib.UA_OP_FUSED_FWD)
+
+
 def test_null_and_small_workspace_are_rejected_before_any_launch():
     lib = _lib.load()
     d = _lib.UaDesc(1, 1, 1, 128, 64, 32, _lib.UA_F32, 0)
