@@ -352,3 +352,39 @@ def test_decoder_front_end_takes_sequence_major_projections_without_copies(dtype
     gs = gs.view(b, s, 2, n_kv).permute(2, 0, 3, 1)
     assert rel_err(gs[0].reshape(g_ref[3].shape), g_ref[3]) <= TOL[dtype]
     assert rel_err(gs[1].reshape(g_ref[4].shape), g_ref[4]) <= TOL[dtype]
+
+
+def test_entry_points_can_be_captured_in_a_hip_graph():
+    """The entry points enqueue kernels on the given stream and neither allocate, synchronise nor memset, so a forward +
+    backward step can be captured once and replayed: three replays on fresh inputs, with eager work and
+    synchronisations in between, each compared with the eager result on the same inputs."""
+    from universal_attention_triton_amd import ops
+    b, h, r, L, d, c = 1, 2, 2, 320, 64, 64
+    dtype = torch.bfloat16
+    static = {k: v.cuda() for k, v in orc.make_inputs(b, h, r, L, d, c, dtype=dtype, seed=60).items()}
+    a = [static[k] for k in NAMES]
+
+    def step():
+        O, lse, ws = ops.fused_forward(*a, for_backward=True)
+        return (O, lse) + tuple(ops.fused_backward(*a, O, lse, static["dO"], ws=ws))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                                          # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = step()
+    for seed in (61, 62, 63):
+        fresh = orc.make_inputs(b, h, r, L, d, c, dtype=dtype, seed=seed)
+        for k in list(NAMES) + ["dO"]:
+            static[k].copy_(fresh[k])
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in captured]
+        want = step()                                   # eager, same inputs
+        torch.cuda.synchronize()
+        for x, y in zip(got, want):
+            assert torch.equal(x, y)
