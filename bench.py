@@ -176,6 +176,9 @@ def main():
                  "second device). Re-run with --gpus 1.")
     from oracle import ua_oracle as orc
     from universal_attention_triton_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):            # only a tree without a built library builds it first
+        from universal_attention_triton_amd import build as _build
+        _build.build()
     from universal_attention_triton_amd.universal_attention import universal_attention
 
     cfg = CONFIGS[args.config]

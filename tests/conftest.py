@@ -10,6 +10,11 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+    # the tests load the library that is built in-tree; only a tree without one builds it first
+    from universal_attention_triton_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        from universal_attention_triton_amd import build
+        build.build()
 
 
 @pytest.fixture(scope="session")
