@@ -116,6 +116,18 @@ int ua_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
 int ua_fused_fwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
                  const void* static_dest, void* O, float* lse, void* ws, size_t ws_bytes, ua_stream_t stream);
 
+/* The fused forward for callers that cannot allocate or supply device scratch (code under HIP graph capture, serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as ua_fused_fwd
+ * minus the workspace: the scratch is a device array inside the library, UA_NOALLOC_SCRATCH_BYTES per GPU, held from
+ * the library's load until the process ends.  Problems whose ua_workspace_bytes(desc, UA_OP_FUSED_FWD) exceeds it are
+ * refused with UA_EWORKSPACE.  Calls no hipMalloc / hipFree.  All calls on one GPU share the array: two calls that
+ * overlap on one GPU (different streams or threads) race, and the forward state a later ua_fused_bwd could reuse is not
+ * kept (call ua_fused_bwd with ws_has_fwd = 0). */
+#define UA_NOALLOC_SCRATCH_BYTES (64u << 20)
+size_t ua_noalloc_scratch_bytes(void);
+int ua_fused_fwd_noalloc(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
+                         const void* static_dest, void* O, float* lse, ua_stream_t stream);
+
 /* Fused backward: replaces SMVecMatMul.backward + UniversalAttention.backward
  * (universal_attention_autograd.py:291-297, :47-99) / _attention.backward (universal_attention_kernel_opt.py:504-581).
  * O, lse: as produced by ua_fused_fwd; dO contiguous [b,h,r,L,d]. */

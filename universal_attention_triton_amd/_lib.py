@@ -42,6 +42,8 @@ SIGNATURES = {
     "ua_bwd": (c_int, [P(UaDesc), P(UaRows), P(UaRows), P(UaRows), c_void_p, c_void_p, P(UaChunked), P(UaChunked), c_void_p,
                        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
     "ua_fused_fwd": (c_int, [P(UaDesc), P(UaRows), P(UaRows), P(UaRows), c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "ua_noalloc_scratch_bytes": (c_size_t, []),
+    "ua_fused_fwd_noalloc": (c_int, [P(UaDesc), P(UaRows), P(UaRows), P(UaRows), c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "ua_fused_bwd": (c_int, [P(UaDesc), P(UaRows), P(UaRows), P(UaRows), c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                              c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
     "ua_merge_fwd": (c_int, [c_int, c_int64, c_int32, c_int32, c_int32, P(UaChunked), c_void_p, c_void_p, c_void_p]),

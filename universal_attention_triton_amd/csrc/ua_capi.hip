@@ -378,6 +378,46 @@ int ua_fused_fwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, cons
   return run_fused_fwd_kernels(*desc, l, w, O, lse, tuned_variant(*desc, UA_OP_FUSED_FWD), s);
 }
 
+// ---- forward for callers that cannot allocate: scratch in a device array of the library itself ----------------
+// One copy of the array exists per GPU, at its own address; the name below is only a host-side handle, the address
+// comes from hipGetSymbolAddress with that GPU current and is what the kernels receive.
+static __device__ __align__(256) unsigned char scratch[UA_NOALLOC_SCRATCH_BYTES];
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices] = {};
+int scratch_of_current_device(void** out) {
+  int dev = -1;
+  UA_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return fail(UA_EINVAL, "device index %d out of range", dev);
+  std::lock_guard<std::mutex> g(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    UA_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return fail(UA_ELAUNCH, "hipGetSymbolAddress returned a null address");
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return UA_OK;
+}
+}  // namespace
+
+size_t ua_noalloc_scratch_bytes(void) { return UA_NOALLOC_SCRATCH_BYTES; }
+
+int ua_fused_fwd_noalloc(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
+                         const void* static_dest, void* O, float* lse, ua_stream_t stream) {
+  if (int e = check_desc(desc, false)) return e;
+  const Layout l = make_layout(*desc, false);
+  if (l.fwd_end > (size_t)UA_NOALLOC_SCRATCH_BYTES)
+    return fail(UA_EWORKSPACE, "problem needs %zu bytes of scratch, the built-in array holds %zu: use ua_fused_fwd with a workspace",
+                l.fwd_end, (size_t)UA_NOALLOC_SCRATCH_BYTES);
+  void* ws = nullptr;
+  if (int e = scratch_of_current_device(&ws)) return e;
+  // every region of the forward state is written before it is read (padding included), so nothing of the previous
+  // call's contents has to be cleared
+  return ua_fused_fwd(desc, kc, vc, xq, static_src, static_dest, O, lse, ws, UA_NOALLOC_SCRATCH_BYTES, stream);
+}
+
 int ua_fused_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
                  const void* static_dest, const void* O, const float* lse, const void* dO, void* dkc, void* dvc, void* dxq,
                  void* dsrc, void* ddest, void* ws, size_t ws_bytes, int ws_has_fwd, ua_stream_t stream) {

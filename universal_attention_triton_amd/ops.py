@@ -290,3 +290,25 @@ def affinity_backward(k, src, dest, daff):
                                    dk.data_ptr(), dsrc.data_ptr(), ddest.data_ptr(), ws.data_ptr(), ws.numel(), _stream()),
                "ua_affinity_bwd")
     return dk, dsrc, ddest
+
+
+def fused_forward_noalloc(kc, vc, xq, static_src, static_dest, O, lse):
+    """ua_fused_fwd_noalloc: the fused forward into caller-provided O [b,h,r,l,d] (xq.dtype) and lse [b,h,r,l]
+    (float32), with the library's built-in scratch instead of a workspace.  Nothing is allocated, so nothing is copied
+    either: every tensor must already be laid out as the C ABI wants it (unit feature stride, contiguous gates and
+    outputs); problems beyond ua_noalloc_scratch_bytes() raise UaError."""
+    _require_gpu(kc, vc, xq, static_src, static_dest, O, lse)
+    if not (kc.dtype == vc.dtype == xq.dtype == static_src.dtype == static_dest.dtype == O.dtype) or lse.dtype != torch.float32:
+        raise TypeError("inputs and O share one dtype, lse is float32")
+    for t in (kc, vc, xq):
+        if t.stride(-1) != 1:
+            raise ValueError("unit feature stride required (no copies are made)")
+    for t in (static_src, static_dest, O, lse):
+        if not t.is_contiguous():
+            raise ValueError("gates and outputs must be contiguous (no copies are made)")
+    lib = _lib.load()
+    desc = _desc(kc, xq, False, 0)
+    _lib.check(lib.ua_fused_fwd_noalloc(ctypes.byref(desc), ctypes.byref(_rows_k(kc)), ctypes.byref(_rows_k(vc)),
+                                        ctypes.byref(_rows_q(xq)), static_src.data_ptr(), static_dest.data_ptr(), O.data_ptr(),
+                                        lse.data_ptr(), _stream()), "ua_fused_fwd_noalloc")
+    return O, lse
