@@ -158,15 +158,37 @@ int ua_affinity_bwd(const ua_desc* desc, const ua_rows* k, const void* src, cons
                     void* dsrc, void* ddest, void* ws, size_t ws_bytes, ua_stream_t stream);
 
 /* On-device autotune table: replaces the @triton.autotune wrappers
- * (universal_attention_kernel.py:10-25, universal_attention_kernel_opt.py:8-36).  Times the kernel variants
- * available for (op, desc) on `stream` using `ws` and records the fastest in the process-wide table that
- * the ops consult.  Synchronises.  Returns the chosen variant id (>= 0) or a negative error. */
+ * (universal_attention_kernel.py:10-25, universal_attention_kernel_opt.py:8-36,115-118,309-312, affinity_kernel_opt.py:6-27).
+ * The table is process-wide and thread-safe, keyed by (kernel slot, dtype, padded head dim, r, log2 bucket of L, log2
+ * bucket of b*h).  Every launch of a slot's kernel consults it: an entry set by ua_tune_set / ua_autotune wins, then the
+ * built-in entries shipped for the reference's benchmark shapes, then a size heuristic.
+ * Kernel slots (the `slot` argument of ua_tune_get / set / variants): */
+enum {
+  UA_TUNE_FWD_RECOMPUTE = 2, /* == UA_OP_FUSED_FWD.  Forward without bias tiles (fp32, UA_FLAG_RECOMPUTE): bf16 0 = 8 waves
+                                two LDS stages, 1 = 8 waves one stage, 2 = 12 waves, 3 = 16 waves, 4 = 4 waves; fp32: one */
+  UA_TUNE_CARRY = 16,        /* bias pre-pass of the bf16 operator: 0 = 8 waves x 16 keys per workgroup, 1 = 4 waves */
+  UA_TUNE_FWD_TILES = 17,    /* bf16 forward over bias tiles: 0 = one 32-query block per wave (256-query workgroups, two
+                                LDS stages), 1 = 16 queries per wave (128-query workgroups, one stage, two per CU),
+                                2 = 16 queries per wave, 64-query workgroups (r = 1 only) */
+  UA_TUNE_BWD_PARTS = 18,    /* key side of the bf16 backward with r > 1: variant i divides the query groups of a kv
+                                head into the i-th smallest divisor of r parts with a sweep each (0 = one shared sweep).
+                                Changes ua_workspace_bytes: set it before sizing the workspace. */
+  UA_TUNE_BWD_QUERIES = 19   /* query side of the bf16 backward over gradient tiles: 0 = steps of 32 keys, two workgroups
+                                per CU; 1 = steps of 64 keys, one workgroup per CU */
+};
+/* ua_autotune(desc, op, ...) with op = UA_OP_FUSED_FWD or UA_OP_FUSED_BWD times every variant of every kernel slot on
+ * that op's path for desc (hipEvents on `stream`, synchronises) and records the fastest of each.  `ws` must hold what
+ * the op itself left there for desc: call ua_fused_fwd (resp. ua_fused_fwd + ua_fused_bwd with ws_has_fwd) on the same
+ * workspace first; the tuning runs re-launch the kernels on that state.  UA_OP_FUSED_BWD clobbers the backward part of
+ * the workspace (the forward state stays valid).  Returns 0 or a negative error. */
 int ua_autotune(const ua_desc* desc, int op, void* ws, size_t ws_bytes, ua_stream_t stream);
-/* Table access for persistence: get / force the variant of (op, desc). -1 = no entry / built-in default. */
-int ua_tune_get(const ua_desc* desc, int op);
-int ua_tune_set(const ua_desc* desc, int op, int variant);
-/* Number of variants an op has for this description (>= 1), or a negative error. */
-int ua_tune_variants(const ua_desc* desc, int op);
+/* Table access for persistence: entry of (slot, desc) set by ua_tune_set / ua_autotune, -1 if none. */
+int ua_tune_get(const ua_desc* desc, int slot);
+int ua_tune_set(const ua_desc* desc, int slot, int variant);   /* variant -1 removes the entry */
+/* What a launch of the slot's kernel would use for desc right now (entry, else built-in, else heuristic). */
+int ua_tune_choice(const ua_desc* desc, int slot);
+/* Number of variants a slot has for this description (>= 1), or a negative error. */
+int ua_tune_variants(const ua_desc* desc, int slot);
 
 /* Per-kernel timing, no counterpart in the reference (its harness times whole calls with CUDA events,
  * Universal_Attention/triton/_debug.py:413-446).  While enabled every kernel group the ops enqueue is bracketed

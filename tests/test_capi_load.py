@@ -89,12 +89,58 @@ def test_ops_refuse_cpu_tensors():
         ops.fused_forward(k, k, torch.zeros(1, 1, 1, 32, 16), torch.ones(1, 1, 1, 32), torch.ones(1, 1, 32))
 
 
-def test_tune_table_roundtrip():
+def test_tune_table_roundtrip_and_choice_order():
+    """An entry wins over the built-in table and the heuristic; -1 removes it; out-of-range variants and unknown slots
+    are refused; the slots report their variant counts (host logic only)."""
     lib = _lib.load()
     d = _lib.UaDesc(1, 2, 1, 1024, 128, 0, _lib.UA_BF16, 0)
-    n = lib.ua_tune_variants(ctypes.byref(d), _lib.UA_OP_FUSED_FWD)
-    assert n >= 1
-    assert lib.ua_tune_set(ctypes.byref(d), _lib.UA_OP_FUSED_FWD, n - 1) == 0
-    assert lib.ua_tune_get(ctypes.byref(d), _lib.UA_OP_FUSED_FWD) == n - 1
-    assert lib.ua_tune_set(ctypes.byref(d), _lib.UA_OP_FUSED_FWD, n) < 0
-    assert lib.ua_tune_set(ctypes.byref(d), _lib.UA_OP_FUSED_FWD, 0) == 0
+    for slot, n_min in ((_lib.UA_TUNE_FWD_RECOMPUTE, 5), (_lib.UA_TUNE_CARRY, 2), (_lib.UA_TUNE_FWD_TILES, 3),
+                        (_lib.UA_TUNE_BWD_PARTS, 1), (_lib.UA_TUNE_BWD_QUERIES, 2)):
+        n = lib.ua_tune_variants(ctypes.byref(d), slot)
+        assert n >= n_min, (slot, n)
+        base = lib.ua_tune_choice(ctypes.byref(d), slot)
+        assert 0 <= base < n and lib.ua_tune_get(ctypes.byref(d), slot) == -1
+        assert lib.ua_tune_set(ctypes.byref(d), slot, n - 1) == 0
+        assert lib.ua_tune_get(ctypes.byref(d), slot) == n - 1 == lib.ua_tune_choice(ctypes.byref(d), slot)
+        assert lib.ua_tune_set(ctypes.byref(d), slot, n) < 0
+        assert lib.ua_tune_set(ctypes.byref(d), slot, -1) == 0
+        assert lib.ua_tune_get(ctypes.byref(d), slot) == -1 and lib.ua_tune_choice(ctypes.byref(d), slot) == base
+    assert lib.ua_tune_variants(ctypes.byref(d), 7) < 0
+    # grouped queries: one variant per divisor of r; fp32 has a single variant everywhere but the recomputing forward
+    g = _lib.UaDesc(1, 8, 4, 4096, 128, 0, _lib.UA_BF16, 0)
+    assert lib.ua_tune_variants(ctypes.byref(g), _lib.UA_TUNE_BWD_PARTS) == 3
+    assert lib.ua_tune_variants(ctypes.byref(g), _lib.UA_TUNE_FWD_TILES) == 2
+    f = _lib.UaDesc(1, 8, 4, 4096, 128, 0, _lib.UA_F32, 0)
+    assert [lib.ua_tune_variants(ctypes.byref(f), s) for s in (16, 17, 18, 19)] == [1, 1, 1, 1]
+
+
+def test_number_of_key_side_parts_follows_the_table_and_sizes_the_workspace():
+    lib = _lib.load()
+    g = _lib.UaDesc(1, 8, 4, 4096, 128, 0, _lib.UA_BF16, 0)
+    sizes = []
+    for v in range(3):
+        assert lib.ua_tune_set(ctypes.byref(g), _lib.UA_TUNE_BWD_PARTS, v) == 0
+        sizes.append(lib.ua_workspace_bytes(ctypes.byref(g), _lib.UA_OP_FUSED_BWD))
+    lib.ua_tune_set(ctypes.byref(g), _lib.UA_TUNE_BWD_PARTS, -1)
+    assert sizes[0] < sizes[1] < sizes[2]
+    shared = _lib.UaDesc(1, 8, 4, 4096, 128, 0, _lib.UA_BF16, _lib.UA_FLAG_SHARE_GROUPS)
+    assert lib.ua_workspace_bytes(ctypes.byref(shared), _lib.UA_OP_FUSED_BWD) == sizes[0]
+
+
+def test_tune_table_persists_through_json(tmp_path):
+    from universal_attention_triton_amd import tune
+    lib = _lib.load()
+    tune.set_entry(2, 16, 1, 2048, 64, "bf16", "fwd_tiles", 2)
+    tune.set_entry(1, 8, 4, 4096, 128, "bf16", "bwd_queries", 1)
+    path = str(tmp_path / "ua_tune.json")
+    tune.save(path)
+    d1 = _lib.UaDesc(2, 16, 1, 2048, 64, 0, _lib.UA_BF16, 0)
+    d2 = _lib.UaDesc(1, 8, 4, 4096, 128, 0, _lib.UA_BF16, 0)
+    lib.ua_tune_set(ctypes.byref(d1), _lib.UA_TUNE_FWD_TILES, -1)
+    lib.ua_tune_set(ctypes.byref(d2), _lib.UA_TUNE_BWD_QUERIES, -1)
+    assert lib.ua_tune_get(ctypes.byref(d1), _lib.UA_TUNE_FWD_TILES) == -1
+    assert tune.load(path) >= 2
+    assert lib.ua_tune_get(ctypes.byref(d1), _lib.UA_TUNE_FWD_TILES) == 2
+    assert lib.ua_tune_get(ctypes.byref(d2), _lib.UA_TUNE_BWD_QUERIES) == 1
+    lib.ua_tune_set(ctypes.byref(d1), _lib.UA_TUNE_FWD_TILES, -1)
+    lib.ua_tune_set(ctypes.byref(d2), _lib.UA_TUNE_BWD_QUERIES, -1)

@@ -113,31 +113,6 @@ def test_second_generation_calling_convention(dtype):
         attention(q, k, v, False, 1.0, inp["static_src"].reshape(B, Hkv, L).cuda(), inp["static_dest"].cuda())
 
 
-def test_every_forward_variant_gives_the_same_result_and_autotune_records_one():
-    from universal_attention_triton_amd import ops
-    inp = orc.make_inputs(1, 2, 2, 1024 + 64, 128, 32, dtype=torch.bfloat16, seed=51)    # L not a multiple of 128/192/256
-    a = [inp[k].cuda() for k in NAMES]
-    O_ref, lse_ref, _ = dense_reference(inp)
-    n = ops.tune_variants(a[0], a[2])
-    assert n >= 2
-    results = []
-    for v in range(n):
-        ops.tune_set(a[0], a[2], v)
-        assert ops.tune_get(a[0], a[2]) == v
-        O, lse, _ = ops.fused_forward(*a, recompute=True)      # the variants belong to the recomputing forward
-        torch.cuda.synchronize()
-        assert rel_err(O, O_ref) <= TOL[torch.bfloat16], (v, rel_err(O, O_ref))
-        assert float((lse.cpu().double() - lse_ref).abs().max()) <= 2e-2
-        results.append(O.float().cpu())
-    for v in range(1, n):
-        assert rel_err(results[v], results[0]) <= 2e-3, v            # same arithmetic, different summation order
-    best = ops.autotune(*a)
-    assert 0 <= best < n and ops.tune_get(a[0], a[2]) == best
-    O, _, _ = ops.fused_forward(*a, recompute=True)
-    assert rel_err(O, O_ref) <= TOL[torch.bfloat16]
-    ops.tune_set(a[0], a[2], 0)
-
-
 @pytest.mark.parametrize("shape", [(1, 2, 1, 1024 + 64, 128, 32), (2, 1, 3, 640, 48, 64)])
 @pytest.mark.parametrize("prune", [False, True])
 def test_recomputing_and_tile_exchanging_bf16_kernels_agree(shape, prune):

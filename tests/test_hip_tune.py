@@ -1,0 +1,103 @@
+"""The autotune table on the GPU (reference: the @triton.autotune wrappers around every launch,
+Universal_Attention/triton/universal_attention_kernel.py:10-25, universal_attention_kernel_opt.py:8-36): every variant of
+every kernel slot on the default bf16 path meets the oracle; ua_autotune records a choice per slot; the entries shipped
+for the benchmark shapes are as fast as what ua_autotune finds on this device (within 3 %)."""
+import statistics
+
+import pytest
+import torch
+
+from oracle import ua_oracle as orc
+from universal_attention_triton_amd import ops
+from .util import NAMES, TOL, dense_reference, rel_err
+
+pytestmark = pytest.mark.gpu
+BF = torch.bfloat16
+
+
+def _step(a, dO):
+    O, lse, ws = ops.fused_forward(*a, for_backward=True)
+    g = ops.fused_backward(*a, O, lse, dO, ws=ws)
+    return O, lse, g
+
+
+@pytest.mark.parametrize("shape", [(1, 2, 1, 1024 + 64, 128), (1, 2, 4, 512 + 32, 64), (2, 1, 2, 768, 128)])
+def test_every_variant_of_every_slot_on_the_default_path_meets_the_oracle(shape):
+    b, h, r, L, d = shape
+    inp = orc.make_inputs(b, h, r, L, d, 32, dtype=BF, seed=61 + r)
+    a = [inp[k].cuda() for k in NAMES]
+    dO = inp["dO"].cuda()
+    O_ref, lse_ref, g_ref = dense_reference(inp)
+    for slot in ("carry", "fwd_tiles", "bwd_parts", "bwd_queries"):
+        n = ops.tune_variants(a[0], a[2], slot)
+        assert n >= (1 if slot == "bwd_parts" and r == 1 else 2), (slot, n)
+        for v in range(n):
+            ops.tune_set(a[0], a[2], v, slot)
+            try:
+                O, lse, g = _step(a, dO)
+                torch.cuda.synchronize()
+            finally:
+                ops.tune_set(a[0], a[2], -1, slot)
+            assert rel_err(O, O_ref) <= TOL[BF], (slot, v, rel_err(O, O_ref))
+            assert float((lse.cpu().double() - lse_ref).abs().max()) <= 2e-2, (slot, v)
+            for name, x, ref in zip(NAMES, g, g_ref):
+                assert rel_err(x.reshape(ref.shape), ref) <= TOL[BF], (slot, v, name, rel_err(x.reshape(ref.shape), ref))
+
+
+def test_recomputing_forward_variants_agree_and_autotune_records_a_choice_per_slot():
+    inp = orc.make_inputs(1, 2, 2, 1024 + 64, 128, 32, dtype=BF, seed=51)    # L not a multiple of 128/192/256
+    a = [inp[k].cuda() for k in NAMES]
+    O_ref, lse_ref, _ = dense_reference(inp)
+    n = ops.tune_variants(a[0], a[2], "fwd_recompute")
+    assert n >= 2
+    results = []
+    for v in range(n):
+        ops.tune_set(a[0], a[2], v, "fwd_recompute")
+        O, lse, _ = ops.fused_forward(*a, recompute=True)
+        torch.cuda.synchronize()
+        assert rel_err(O, O_ref) <= TOL[BF], (v, rel_err(O, O_ref))
+        results.append(O.float().cpu())
+    ops.tune_set(a[0], a[2], -1, "fwd_recompute")
+    for v in range(1, n):
+        assert rel_err(results[v], results[0]) <= 2e-3, v            # same arithmetic, different summation order
+    chosen = ops.autotune(*a)
+    assert set(chosen) == {"carry", "fwd_tiles", "bwd_parts", "bwd_queries"}, chosen
+    for slot, v in chosen.items():
+        assert 0 <= v < ops.tune_variants(a[0], a[2], slot) and ops.tune_choice(a[0], a[2], slot) == v
+    O, _, _ = ops.fused_forward(*a)
+    assert rel_err(O, O_ref) <= TOL[BF]
+    for slot in chosen:
+        ops.tune_set(a[0], a[2], -1, slot)
+
+
+def _median_ms(a, dO, reps=7):
+    for _ in range(2):
+        _step(a, dO)
+    times = []
+    for _ in range(reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        _step(a, dO)
+        e1.record()
+        e1.synchronize()
+        times.append(e0.elapsed_time(e1))
+    return statistics.median(times)
+
+
+@pytest.mark.parametrize("cfg", [(1, 32, 1, 8192, 128, 1002), (1, 8, 4, 4096, 128, 1003)], ids=["config2", "config3"])
+def test_shipped_table_is_within_3_percent_of_autotune_on_this_device(cfg):
+    b, h, r, L, d, seed = cfg
+    inp = orc.make_inputs(b, h, r, L, d, 128, dtype=BF, seed=seed)
+    a = [inp[k].cuda() for k in NAMES]
+    dO = inp["dO"].cuda()
+    slots = [s for s in ("carry", "fwd_tiles", "bwd_parts", "bwd_queries") if ops.tune_variants(a[0], a[2], s) > 1]
+    shipped = {s: ops.tune_choice(a[0], a[2], s) for s in slots}
+    t_shipped = _median_ms(a, dO)
+    tuned = ops.autotune(*a, dO=dO)
+    try:
+        if {s: tuned[s] for s in slots} != shipped:
+            t_tuned = _median_ms(a, dO)
+            assert t_shipped <= 1.03 * t_tuned, (shipped, tuned, t_shipped, t_tuned)
+    finally:
+        for s in slots:
+            ops.tune_set(a[0], a[2], -1, s)

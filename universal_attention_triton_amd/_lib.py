@@ -12,6 +12,8 @@ LIB_PATH = os.path.join(HERE, "libua_hip.so")
 
 UA_F32, UA_BF16 = 0, 1
 UA_OP_FWD, UA_OP_BWD, UA_OP_FUSED_FWD, UA_OP_FUSED_BWD = 0, 1, 2, 3
+UA_TUNE_FWD_RECOMPUTE, UA_TUNE_CARRY, UA_TUNE_FWD_TILES, UA_TUNE_BWD_PARTS, UA_TUNE_BWD_QUERIES = 2, 16, 17, 18, 19
+TUNE_SLOTS = {"fwd_recompute": 2, "carry": 16, "fwd_tiles": 17, "bwd_parts": 18, "bwd_queries": 19}
 UA_FLAG_SKIP_MASKED = 1
 UA_FLAG_RECOMPUTE = 4
 UA_FLAG_PRUNE = 2
@@ -56,6 +58,7 @@ SIGNATURES = {
     "ua_tune_get": (c_int, [P(UaDesc), c_int]),
     "ua_tune_set": (c_int, [P(UaDesc), c_int, c_int]),
     "ua_tune_variants": (c_int, [P(UaDesc), c_int]),
+    "ua_tune_choice": (c_int, [P(UaDesc), c_int]),
     "ua_prof_enable": (None, [c_int]),
     "ua_prof_collect": (c_int, [ctypes.c_char_p, c_size_t]),
 }
@@ -71,6 +74,7 @@ class UaError(RuntimeError):
 def load():
     """Returns the loaded library; raises if it has not been built (python -m universal_attention_triton_amd.build)."""
     global _lib
+    env_file = None
     with _lock:
         if _lib is None:
             if not os.path.exists(LIB_PATH):
@@ -81,6 +85,11 @@ def load():
                 fn = getattr(lib, name)
                 fn.restype, fn.argtypes = res, args
             _lib = lib
+            env_file = os.environ.get("UA_TUNE_FILE")
+    if env_file and os.path.exists(env_file) and not getattr(load, "_env_done", False):
+        load._env_done = True
+        from . import tune
+        tune.load(env_file)
     return _lib
 
 

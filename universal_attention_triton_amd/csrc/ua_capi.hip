@@ -3,6 +3,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -57,7 +58,91 @@ int check_desc(const ua_desc* d, bool chunked) {
   return UA_OK;
 }
 
-Layout make_layout(const ua_desc& d, bool chunked) {
+// ---- autotune table ------------------------------------------------------------------------
+// key: kernel slot, dtype, padded head dim, r, log2 bucket of L, log2 bucket of b*h
+using TuneKey = std::tuple<int, int, int, int, int, int>;
+std::mutex g_tune_mu;
+std::map<TuneKey, int> g_tune;
+
+int l_bucket(int L) { int b = 0; while ((128 << b) < L) ++b; return b; }
+int z_bucket(long z) { int b = 0; while ((1L << b) < z) ++b; return b; }
+TuneKey tune_key(const ua_desc& d, int slot) {
+  return TuneKey(slot, d.dtype, d.d <= 64 ? 64 : 128, d.r, l_bucket(d.L), z_bucket((long)d.b * d.h));
+}
+bool known_slot(int slot) {
+  return slot == UA_TUNE_FWD_RECOMPUTE || slot == UA_TUNE_CARRY || slot == UA_TUNE_FWD_TILES || slot == UA_TUNE_BWD_PARTS ||
+         slot == UA_TUNE_BWD_QUERIES;
+}
+int n_divisors(int r) { int n = 0; for (int p = 1; p <= r; ++p) n += r % p == 0; return n; }
+int nth_divisor(int r, int i) { for (int p = 1; p <= r; ++p) if (r % p == 0 && i-- == 0) return p; return 1; }
+int divisor_index(int r, int p) { int i = 0; for (int q = 1; q < p; ++q) i += r % q == 0; return i; }
+int n_variants(const ua_desc& d, int slot) {
+  const bool bf = d.dtype == UA_BF16;
+  switch (slot) {
+    case UA_TUNE_FWD_RECOMPUTE: return ua::fwd_fused_variants(d.dtype, d.d <= 64 ? 64 : 128);
+    case UA_TUNE_CARRY: return bf ? 2 : 1;
+    case UA_TUNE_FWD_TILES: return bf ? (d.r % 2 == 0 ? 2 : 3) : 1;
+    case UA_TUNE_BWD_PARTS: return bf ? n_divisors(d.r) : 1;
+    case UA_TUNE_BWD_QUERIES: return bf ? 2 : 1;
+  }
+  return 1;
+}
+// Entries shipped with the library: measured with ua_autotune on one MI355X for the shapes the reference's benchmark
+// recipes name (bf16; b, h, r, L, d).  {slot, D, r, L bucket, b*h bucket, variant}
+struct BuiltIn { int slot, D, r, lb, zb, variant; };
+const BuiltIn kBuiltIn[] = {
+#include "ua_tune_defaults.inc"
+};
+// size heuristics for everything else
+int heuristic_variant(const ua_desc& d, int slot) {
+  const long Zk = (long)d.b * d.h, Zq = Zk * d.r;
+  const int Lp = (int)align_up((size_t)d.L, 128);
+  switch (slot) {
+    case UA_TUNE_CARRY:      // under two 8-wave workgroups per CU the sweep latency of a workgroup bounds the launch
+      return Zk * (Lp / 128) < 512 ? 1 : 0;
+    case UA_TUNE_FWD_TILES:  // 256-query workgroups need about four per CU to balance; small launches run 64-query pieces
+      if (Zq * (Lp / 256) >= 1024) return 0;
+      return (d.r % 2 == 0 || Zq * (Lp / 128) >= 1536) ? 1 : 2;
+    case UA_TUNE_BWD_PARTS: {
+      // Grouped queries: the key-stationary kernel sweeps the r query groups of a kv head in one workgroup, sharing the
+      // key-key part of every step (a step of a further group costs about 0.7 of a full one).  Its longest workgroup then
+      // runs Lp/32 * r steps, and with few kv heads the launch waits for it.  The groups can instead be divided into p
+      // parts with a sweep each (p times the workgroups, a longest one p times shorter, the key-key part repeated per
+      // part).  p = the divisor of r with the smallest estimate max(longest workgroup, 1.1 x average load of the 256 CUs).
+      int best_p = 1;
+      const double blocks = Lp / 32, wgs = (double)Zk * (Lp / 128);
+      double best = 0;
+      for (int p = 1; p <= d.r; ++p) {
+        if (d.r % p) continue;
+        const double w = 1.0 + 0.7 * (d.r / p - 1);                 // cost of one query block for the groups of a part
+        const double longest = blocks * w, average = 1.1 * wgs * p * (blocks / 2) * w / 256.0;
+        const double cost = longest > average ? longest : average;
+        if (p == 1 || cost < best) { best = cost; best_p = p; }
+      }
+      return divisor_index(d.r, best_p);
+    }
+  }
+  return 0;
+}
+int tune_entry(const ua_desc& d, int slot) {
+  std::lock_guard<std::mutex> g(g_tune_mu);
+  auto it = g_tune.find(tune_key(d, slot));
+  return it == g_tune.end() ? -1 : it->second;
+}
+int tuned_variant(const ua_desc& d, int slot) {
+  const int n = n_variants(d, slot);
+  int v = tune_entry(d, slot);
+  if (v >= 0 && v < n) return v;
+  const TuneKey k = tune_key(d, slot);
+  if (d.dtype == UA_BF16)
+    for (const BuiltIn& e : kBuiltIn)
+      if (e.slot == slot && e.D == std::get<2>(k) && e.r == d.r && e.lb == std::get<4>(k) && e.zb == std::get<5>(k) && e.variant < n)
+        return e.variant;
+  v = heuristic_variant(d, slot);
+  return v < n ? v : 0;
+}
+
+Layout make_layout(const ua_desc& d, bool chunked, int force_parts = 0) {
   Layout l{};
   l.D = d.d <= 64 ? 64 : 128;
   l.Lp = (int)align_up((size_t)d.L, 128);
@@ -100,24 +185,11 @@ Layout make_layout(const ua_desc& d, bool chunked) {
   l.Dsuf = (atomics || l.tiles) ? 0 : take(carries);     // ... and the gradient tiles the suffix carries
   l.masked_nz = take(256);
   // score and decay gradients of every (32 keys, 16 queries) tile (grad_tiles)
-  // Grouped queries: the key-stationary kernel sweeps the r query groups of a kv head in one workgroup, sharing the
-  // key-key part of every step (a step of a further group costs about 0.7 of a full one).  Its longest workgroup then
-  // runs Lp/32 * r steps, and with few kv heads the launch waits for it.  The groups can instead be divided into p parts
-  // with a sweep each (p times the workgroups, a longest one p times shorter, the key-key part repeated per part; the
-  // key-side sums are then kept per (kv head, part)).  p = the divisor of r with the smallest estimate
-  // max(longest workgroup, 1.1 x average load of the 256 CUs).  UA_FLAG_SHARE_GROUPS forces p = 1.
+  // Grouped queries: the key side sweeps the query groups of a kv head in key_parts parts (UA_TUNE_BWD_PARTS; the key-side
+  // sums are then kept per (kv head, part)).  UA_FLAG_SHARE_GROUPS forces one shared sweep.
   l.key_parts = 1;
-  if (l.tiles && d.r > 1 && !(d.flags & UA_FLAG_SHARE_GROUPS)) {
-    const double blocks = l.Lp / 32, wgs = (double)l.Zk * (l.Lp / 128);
-    double best = 0;
-    for (int p = 1; p <= d.r; ++p) {
-      if (d.r % p) continue;
-      const double w = 1.0 + 0.7 * (d.r / p - 1);                 // cost of one query block for the groups of a part
-      const double longest = blocks * w, average = 1.1 * wgs * p * (blocks / 2) * w / 256.0;
-      const double cost = longest > average ? longest : average;
-      if (p == 1 || cost < best) { best = cost; l.key_parts = p; }
-    }
-  }
+  if (l.tiles && d.r > 1 && !(d.flags & UA_FLAG_SHARE_GROUPS)) l.key_parts = nth_divisor(d.r, tuned_variant(d, UA_TUNE_BWD_PARTS));
+  if (force_parts > 0) l.key_parts = force_parts;
   const size_t Zs = (size_t)l.Zk * l.key_parts;
   const size_t sg = (size_t)ua::grp_tiles(l.Lp / 32) * 1024;    // grouped by the consuming workgroup, per head
   l.dS_st = l.grad_tiles ? take((size_t)l.Zq * sg) : 0;
@@ -249,40 +321,27 @@ int pack_inputs(const ua_desc& d, const Layout& l, bool rowmajor, const ua_rows*
   return UA_OK;
 }
 
-// ---- autotune table ------------------------------------------------------------------------
-using TuneKey = std::tuple<int, int, int, int, int, int>;  // op, dtype, D, r, chunk, L bucket
-std::mutex g_tune_mu;
-std::map<TuneKey, int> g_tune;
-
-int l_bucket(int L) { int b = 0; while ((128 << b) < L) ++b; return b; }
-TuneKey tune_key(const ua_desc& d, int op) {
-  const bool chunked = (op == UA_OP_FWD || op == UA_OP_BWD);
-  return TuneKey(op, d.dtype, d.d <= 64 ? 64 : 128, d.r, chunked ? d.chunk : 0, l_bucket(d.L));
+int launch_carry_for(const ua_desc& d, const Layout& l, char* ws, int variant, hipStream_t s) {
+  UA_HIP(ua::launch_carry(d.dtype, l.D, ws + l.Kp, (const float*)(ws + l.lsrc), (const float*)(ws + l.ldest),
+                          (float*)(ws + l.C), l.Lp, l.Zk, 1, (d.flags & UA_FLAG_PRUNE) ? (const float*)(ws + l.knorm2) : nullptr,
+                          (const float*)(ws + l.qnorm2), d.r, (int*)(ws + l.reach), (int*)(ws + l.minkey), s,
+                          l.tiles ? ws + l.Bt : nullptr, variant));
+  return UA_OK;
 }
-int n_variants(const ua_desc& d, int op) {
-  if (op == UA_OP_FUSED_FWD) return ua::fwd_fused_variants(d.dtype, d.d <= 64 ? 64 : 128);
-  return 1;
-}
-int tuned_variant(const ua_desc& d, int op) {
-  std::lock_guard<std::mutex> g(g_tune_mu);
-  auto it = g_tune.find(tune_key(d, op));
-  return it == g_tune.end() ? 0 : it->second;
-}
-
-int run_fused_fwd_kernels(const ua_desc& d, const Layout& l, char* ws, void* O, float* lse, int variant, hipStream_t s) {
-  {
-    UA_PROF("k_carry", s);
-    UA_HIP(ua::launch_carry(d.dtype, l.D, ws + l.Kp, (const float*)(ws + l.lsrc), (const float*)(ws + l.ldest),
-                            (float*)(ws + l.C), l.Lp, l.Zk, 1, (d.flags & UA_FLAG_PRUNE) ? (const float*)(ws + l.knorm2) : nullptr,
-                            (const float*)(ws + l.qnorm2), d.r, (int*)(ws + l.reach), (int*)(ws + l.minkey), s,
-                            l.tiles ? ws + l.Bt : nullptr));
-  }
-  UA_PROF("k_fwd_fused", s);
+int launch_fwd_for(const ua_desc& d, const Layout& l, char* ws, void* O, float* lse, int variant, hipStream_t s) {
   UA_HIP(ua::launch_fwd_fused(d.dtype, l.D, variant, ws + l.Qp, ws + l.Kp, ws + l.VT, (const float*)(ws + l.lsrc),
                               (const float*)(ws + l.ldest), (const float*)(ws + l.C), O, lse, (float*)(ws + l.lse2),
                               (const int*)(ws + l.reach), (const int*)(ws + l.minkey), d.r, d.L, l.Lp, d.d, l.Zq, s,
                               l.tiles ? ws + l.Bt : nullptr));
   return UA_OK;
+}
+int run_fused_fwd_kernels(const ua_desc& d, const Layout& l, char* ws, void* O, float* lse, hipStream_t s) {
+  {
+    UA_PROF("k_carry", s);
+    if (int e = launch_carry_for(d, l, ws, l.tiles ? tuned_variant(d, UA_TUNE_CARRY) : 0, s)) return e;
+  }
+  UA_PROF("k_fwd_fused", s);
+  return launch_fwd_for(d, l, ws, O, lse, tuned_variant(d, l.tiles ? UA_TUNE_FWD_TILES : UA_TUNE_FWD_RECOMPUTE), s);
 }
 
 template <class T>
@@ -341,7 +400,7 @@ int run_bwd_common(const ua_desc& d, const Layout& l, char* ws, bool chunked, co
   if (!chunked) {
     UA_PROF("k_bwd_queries", s);
     // chunked operator with tiles: both are enqueued, the flag k_delta left on the device decides which one works
-    if (l.grad_tiles) UA_HIP(ua::launch_bwd_queries_from_tiles(l.D, a, dxq, d.d, l.Zq, s));
+    if (l.grad_tiles) UA_HIP(ua::launch_bwd_queries_from_tiles(l.D, a, dxq, d.d, l.Zq, s, tuned_variant(d, UA_TUNE_BWD_QUERIES)));
     if (!l.tiles) UA_HIP(ua::launch_bwd_queries(d.dtype, l.D, a, dxq, d.d, l.Zk, s));
   }
   if (direct) return UA_OK;
@@ -351,6 +410,45 @@ int run_bwd_common(const ua_desc& d, const Layout& l, char* ws, bool chunked, co
   return UA_OK;
 }
 
+}  // namespace
+
+namespace {
+// times launch(variant) for every variant of the slot (one warm-up, the fastest of six timed launches each) and
+// records the fastest; the events are destroyed on every path
+template <class F>
+int tune_slot(const ua_desc& d, int slot, hipStream_t s, F launch) {
+  const int n = n_variants(d, slot);
+  if (n <= 1) return UA_OK;
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
+    if (e0) (void)hipEventDestroy(e0);
+    return fail(UA_ELAUNCH, "hipEventCreate failed");
+  }
+  int best = -1, rc = UA_OK;
+  float best_ms = 1e30f;
+  for (int v = 0; v < n && rc == UA_OK; ++v) {
+    for (int rep = 0; rep < 7 && rc == UA_OK; ++rep) {
+      if (hipEventRecord(e0, s) != hipSuccess) { rc = fail(UA_ELAUNCH, "hipEventRecord failed"); break; }
+      const int e = launch(v);
+      if (e == 1) break;                     // variant not applicable to this problem
+      if (e != UA_OK) { rc = e; break; }
+      float ms = 0.f;
+      if (hipEventRecord(e1, s) != hipSuccess || hipEventSynchronize(e1) != hipSuccess || hipEventElapsedTime(&ms, e0, e1) != hipSuccess) {
+        rc = fail(UA_ELAUNCH, "timing variant %d of slot %d failed", v, slot);
+        break;
+      }
+      if (rep > 0 && ms < best_ms) { best_ms = ms; best = v; }
+    }
+  }
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  if (rc != UA_OK) return rc;
+  if (best >= 0) {
+    std::lock_guard<std::mutex> g(g_tune_mu);
+    g_tune[tune_key(d, slot)] = best;
+  }
+  return UA_OK;
+}
 }  // namespace
 
 extern "C" {
@@ -375,7 +473,7 @@ int ua_fused_fwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, cons
   char* w = (char*)ws;
   hipStream_t s = (hipStream_t)stream;
   if (int e = pack_inputs(*desc, l, false, kc, vc, xq, static_src, static_dest, w, s)) return e;
-  return run_fused_fwd_kernels(*desc, l, w, O, lse, tuned_variant(*desc, UA_OP_FUSED_FWD), s);
+  return run_fused_fwd_kernels(*desc, l, w, O, lse, s);
 }
 
 // ---- forward for callers that cannot allocate: scratch in a device array of the library itself ----------------
@@ -430,10 +528,7 @@ int ua_fused_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, cons
   const ua_desc& d = *desc;
   if (!ws_has_fwd) {
     if (int e = pack_inputs(d, l, false, kc, vc, xq, static_src, static_dest, w, s)) return e;
-    UA_HIP(ua::launch_carry(d.dtype, l.D, w + l.Kp, (const float*)(w + l.lsrc), (const float*)(w + l.ldest),
-                            (float*)(w + l.C), l.Lp, l.Zk, 1, (d.flags & UA_FLAG_PRUNE) ? (const float*)(w + l.knorm2) : nullptr,
-                            (const float*)(w + l.qnorm2), d.r, (int*)(w + l.reach), (int*)(w + l.minkey), s,
-                            l.tiles ? w + l.Bt : nullptr));
+    if (int e = launch_carry_for(d, l, w, l.tiles ? tuned_variant(d, UA_TUNE_CARRY) : 0, s)) return e;
   }
   const long rowsz = (long)d.L * d.d;
   const ua::RowsView Ov = contiguous_view(O, rowsz, d.d), dOv = contiguous_view(dO, rowsz, d.d);
@@ -685,59 +780,88 @@ int ua_prof_collect(char* buf, size_t cap) {
   return (int)out.size();
 }
 
-int ua_tune_variants(const ua_desc* desc, int op) {
-  if (op < UA_OP_FWD || op > UA_OP_FUSED_BWD) return fail(UA_EINVAL, "unknown op %d", op);
-  if (int e = check_desc(desc, op == UA_OP_FWD || op == UA_OP_BWD)) return e;
-  return n_variants(*desc, op);
+int ua_tune_variants(const ua_desc* desc, int slot) {
+  if (!known_slot(slot)) return fail(UA_EINVAL, "unknown kernel slot %d", slot);
+  if (int e = check_desc(desc, false)) return e;
+  return n_variants(*desc, slot);
 }
-int ua_tune_get(const ua_desc* desc, int op) {
+int ua_tune_get(const ua_desc* desc, int slot) {
   if (!desc) return -1;
-  std::lock_guard<std::mutex> g(g_tune_mu);
-  auto it = g_tune.find(tune_key(*desc, op));
-  return it == g_tune.end() ? -1 : it->second;
+  return tune_entry(*desc, slot);
 }
-int ua_tune_set(const ua_desc* desc, int op, int variant) {
-  const int n = ua_tune_variants(desc, op);
+int ua_tune_choice(const ua_desc* desc, int slot) {
+  const int n = ua_tune_variants(desc, slot);
   if (n < 0) return n;
-  if (variant < 0 || variant >= n) return fail(UA_EINVAL, "variant %d out of range [0,%d)", variant, n);
+  return tuned_variant(*desc, slot);
+}
+int ua_tune_set(const ua_desc* desc, int slot, int variant) {
+  const int n = ua_tune_variants(desc, slot);
+  if (n < 0) return n;
+  if (variant < -1 || variant >= n) return fail(UA_EINVAL, "variant %d out of range [-1,%d)", variant, n);
   std::lock_guard<std::mutex> g(g_tune_mu);
-  g_tune[tune_key(*desc, op)] = variant;
+  if (variant < 0) g_tune.erase(tune_key(*desc, slot));
+  else g_tune[tune_key(*desc, slot)] = variant;
   return UA_OK;
 }
 
 int ua_autotune(const ua_desc* desc, int op, void* ws, size_t ws_bytes, ua_stream_t stream) {
-  const int n = ua_tune_variants(desc, op);
-  if (n < 0) return n;
-  if (n == 1) { ua_tune_set(desc, op, 0); return 0; }
-  // only the fused forward has more than one variant: time the main kernel on whatever the workspace holds
-  const Layout l = make_layout(*desc, false);
-  if (!ws || ws_bytes < l.total) return fail(UA_EWORKSPACE, "autotune needs the backward-sized workspace (%zu bytes)", l.total);
+  if (op != UA_OP_FUSED_FWD && op != UA_OP_FUSED_BWD) return fail(UA_EINVAL, "ua_autotune tunes UA_OP_FUSED_FWD or UA_OP_FUSED_BWD (got %d)", op);
+  if (int e = check_desc(desc, false)) return e;
+  const ua_desc& d = *desc;
+  Layout l = make_layout(d, false);
+  if (!ws || (uintptr_t)ws % 256 != 0) return fail(UA_EWORKSPACE, "autotune needs the 256-byte aligned workspace the op ran on");
+  if (ws_bytes < l.total) return fail(UA_EWORKSPACE, "autotune needs the backward-sized workspace (%zu bytes)", l.total);
   char* w = (char*)ws;
   hipStream_t s = (hipStream_t)stream;
-  // deterministic, finite operands: zero the packed inputs; throw-away outputs go to backward scratch
-  UA_HIP(zero_fill(w, l.fwd_end, s));
-  void* Otmp = w + l.dOp;
-  float* lsetmp = (float*)(w + l.delta);
-  hipEvent_t e0, e1;
-  UA_HIP(hipEventCreate(&e0)); UA_HIP(hipEventCreate(&e1));
-  int best = 0; float best_ms = 1e30f;
-  for (int v = 0; v < n; ++v) {
-    for (int rep = 0; rep < 2; ++rep) {   // first pass warms up
-      UA_HIP(hipEventRecord(e0, s));
-      hipError_t e = ua::launch_fwd_fused(desc->dtype, l.D, v, w + l.Qp, w + l.Kp, w + l.VT, (const float*)(w + l.lsrc),
-                                          (const float*)(w + l.ldest), (const float*)(w + l.C), Otmp, lsetmp, (float*)(w + l.lse2),
-                                          (const int*)(w + l.reach), (const int*)(w + l.minkey), desc->r, desc->L, l.Lp, desc->d, l.Zq, s);
-      if (e != hipSuccess) return fail(UA_ELAUNCH, "autotune launch: %s", hipGetErrorString(e));
-      UA_HIP(hipEventRecord(e1, s));
-      UA_HIP(hipEventSynchronize(e1));
-      float ms = 0.f;
-      UA_HIP(hipEventElapsedTime(&ms, e0, e1));
-      if (rep == 1 && ms < best_ms) { best_ms = ms; best = v; }
+  // throw-away outputs live in the backward part of the workspace
+  if (op == UA_OP_FUSED_FWD) {
+    void* Otmp = w + l.dOp;                  // [Zq][L][d] fits in [Zq][Lp][D]
+    float* lsetmp = (float*)(w + l.delta);
+    if (l.tiles) {
+      if (int e = tune_slot(d, UA_TUNE_FWD_TILES, s, [&](int v) { return launch_fwd_for(d, l, w, Otmp, lsetmp, v, s); })) return e;
+      // the pre-pass rewrites the bias tiles, the reach table and the first-key table with the same values
+      if (int e = tune_slot(d, UA_TUNE_CARRY, s, [&](int v) { return launch_carry_for(d, l, w, v, s); })) return e;
+    } else {
+      if (int e = tune_slot(d, UA_TUNE_FWD_RECOMPUTE, s, [&](int v) { return launch_fwd_for(d, l, w, Otmp, lsetmp, v, s); })) return e;
     }
+    return UA_OK;
   }
-  hipEventDestroy(e0); hipEventDestroy(e1);
-  ua_tune_set(desc, op, best);
-  return best;
+  if (!l.tiles) return UA_OK;                // the recomputing backward has one variant per kernel
+  // key side first (it reads the packed upstream gradient, which the query side's throw-away dQ then overwrites)
+  auto bwd_args = [&](const Layout& ll) {
+    ua::BwdArgsV a{};
+    a.Kp = w + ll.Kp; a.Vp = w + ll.Vp; a.KT = w + ll.KT; a.Qp = w + ll.Qp; a.dOp = w + ll.dOp;
+    a.lsrc = (const float*)(w + ll.lsrc); a.ldest = (const float*)(w + ll.ldest); a.lse2 = (const float*)(w + ll.lse2);
+    a.delta = (const float*)(w + ll.delta); a.C = (const float*)(w + ll.C);
+    a.reach = (const int*)(w + ll.reach); a.minkey = (const int*)(w + ll.minkey);
+    a.dKdacc = (float*)(w + ll.dKdacc); a.dKrow = (float*)(w + ll.dKrow); a.dVrow = (float*)(w + ll.dVrow);
+    a.dsrc_raw = (float*)(w + ll.dsrc_raw); a.masked_nz = (const int*)(w + ll.masked_nz);
+    a.dS_st = w + ll.dS_st; a.dG_st = w + ll.dG_st; a.Bt = w + ll.Bt;
+    a.R = d.r; a.L = d.L; a.Lp = ll.Lp; a.c = 128; a.nch = 1; a.key_parts = ll.key_parts;
+    return a;
+  };
+  if (d.r > 1 && !(d.flags & UA_FLAG_SHARE_GROUPS)) {
+    if (int e = tune_slot(d, UA_TUNE_BWD_PARTS, s, [&](int v) {
+          const Layout ll = make_layout(d, false, nth_divisor(d.r, v));
+          if (ll.total > ws_bytes) return 1;               // this many parts need a larger workspace: not timed
+          const ua::BwdArgsV a = bwd_args(ll);
+          UA_HIP(ua::launch_bwd_keys(d.dtype, ll.D, a, ll.Zk, 0, s));
+          return (int)UA_OK;
+        })) return e;
+    l = make_layout(d, false);
+    if (ws_bytes < l.total) return fail(UA_EWORKSPACE, "the chosen number of parts needs %zu bytes of workspace", l.total);
+    // leave tiles that match the chosen layout for the query side
+    { const ua::BwdArgsV a = bwd_args(l); UA_HIP(ua::launch_bwd_keys(d.dtype, l.D, a, l.Zk, 0, s)); }
+  }
+  {
+    const ua::BwdArgsV a = bwd_args(l);
+    void* dqtmp = w + l.dOp;
+    if (int e = tune_slot(d, UA_TUNE_BWD_QUERIES, s, [&](int v) {
+          UA_HIP(ua::launch_bwd_queries_from_tiles(l.D, a, dqtmp, d.d, l.Zq, s, v));
+          return (int)UA_OK;
+        })) return e;
+  }
+  return UA_OK;
 }
 
 }  // extern "C"

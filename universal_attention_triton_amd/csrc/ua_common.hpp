@@ -406,6 +406,36 @@ __device__ __forceinline__ float suffix32(f32x4& x0, f32x4& x1, const GroupMasks
   for (int v = 0; v < 4; ++v) { x0[v] += a0; x1[v] += a1; }
   return t0 + t1;
 }
+// ---- the same scans on the matrix core (16-bit operands) --------------------------------------------------------
+// A running sum over the 32 queries of a block is a product with a triangular 0/1 matrix: with the block's values as
+// the B operand of as_operand16 (k index = query, column = key) and the matrix as the A operand (row = query u inside
+// tile i), the result tile has the layout of the input tiles and the carry enters as the accumulator.  Three matrix
+// instructions (two tiles and the block total through a matrix of ones) replace about 40 vector instructions of the
+// in-lane adds and lane exchanges above; the summands are rounded to the operand precision, the sums are float32.
+// query position of element e of lane group g in an as_operand16 fragment
+__device__ __forceinline__ constexpr int operand16_query(int g, int e) { return e < 4 ? 4 * g + e : 16 + 4 * g + (e - 4); }
+struct ScanOps { Frag<bf16> tri[2], ones; };
+// SUFFIX = false: row u of tile i sums the queries <= 16 i + u (inclusive prefix); true: the queries >= 16 i + u
+template <bool SUFFIX> __device__ __forceinline__ ScanOps scan_operands(int lane) {
+  const int u = lane & 15, g = lane >> 4;
+  ScanOps o;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const int q = operand16_query(g, e);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) o.tri[i].v[e] = (bf16)((SUFFIX ? q >= 16 * i + u : q <= 16 * i + u) ? 1.0f : 0.0f);
+    o.ones.v[e] = (bf16)1.0f;
+  }
+  return o;
+}
+// y[i] = carry + running sums of the block (values in xb), carry += block total; every register of carry holds the same value
+__device__ __forceinline__ void scan32_mma(const ScanOps& o, const Frag<bf16>& xb, f32x4& carry, f32x4 (&y)[2]) {
+  y[0] = carry; y[1] = carry;
+  mma16(y[0], o.tri[0], xb);
+  mma16(y[1], o.tri[1], xb);
+  mma16(carry, o.ones, xb);
+}
+
 // the 4 per-query values of lane group g inside a 16-query tile, from a float array indexed by query
 __device__ __forceinline__ f32x4 load_t4(const float* __restrict__ p16, int g) {
   const float4 x = *reinterpret_cast<const float4*>(p16 + 4 * g);

@@ -124,6 +124,10 @@ __global__ void __launch_bounds__(64 * NW) k_carry2(const T* __restrict__ Kp, co
   }
   const float la = lsrc[(long)z * Lp + spos];
   float carry = 0.f;
+  // bias tiles: the running sum over the block's queries runs on the matrix core (see scan32_mma); carry4 replaces carry
+  ScanOps sc_ops;
+  f32x4 carry4 = {0, 0, 0, 0};
+  if constexpr (BO) sc_ops = scan_operands<false>(lane);
   float* Cz = C + (long)z * nT16 * Lp + spos;
   const T* Kz = Kp + (long)z * Lp * D;
   bool dead = false;
@@ -159,7 +163,7 @@ __global__ void __launch_bounds__(64 * NW) k_carry2(const T* __restrict__ Kp, co
     constexpr bool MASKED = decltype(masked_c)::value;
     const int tb = first + s;
     if (dead) return;
-    if (__builtin_amdgcn_ballot_w64(carry > thr) == 0) {        // every key of this wave is out of reach from here on
+    if (__builtin_amdgcn_ballot_w64((BO ? carry4[0] : carry) > thr) == 0) {        // every key of this wave is out of reach from here on
       dead = true;
       if (lane == 0) atomicAdd(&n_dead, 1);
       return;
@@ -182,14 +186,14 @@ __global__ void __launch_bounds__(64 * NW) k_carry2(const T* __restrict__ Kp, co
       }
     }
     if constexpr (BO) {
-      const float tot = prefix32(x[0], x[1], gm);
+      f32x4 y[2];
+      scan32_mma(sc_ops, as_operand16<bf16>(x[0], x[1]), carry4, y);
       typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
       f16x8 hb;
 #pragma unroll
-      for (int v = 0; v < 4; ++v) { hb[v] = (_Float16)(x[0][v] + carry); hb[4 + v] = (_Float16)(x[1][v] + carry); }
+      for (int v = 0; v < 4; ++v) { hb[v] = (_Float16)y[0][v]; hb[4 + v] = (_Float16)y[1][v]; }
       char* dst = reinterpret_cast<char*>(Bt) + (((long)z * tri_tiles(nT) + tri_bias_row(tb) + sb16) << 10) + 16 * lane;
       __builtin_nontemporal_store(hb, reinterpret_cast<f16x8*>(dst));
-      carry += tot;
     } else {
       float b0, a0, t0, b1, a1, t1;
       group_scan((x[0][0] + x[0][1]) + (x[0][2] + x[0][3]), gm, b0, a0, t0);
@@ -590,6 +594,205 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Fused forward of the 16-bit operator with bias tiles, one 32-query block per wave.
+// grid (ceil(Lp/32 / NB), Zk * R / RB), 8 waves, NB = 8 / RB blocks per workgroup; wave w owns block NB jt + w / RB of
+// query group w % RB of the workgroup's RB groups (grouped queries share the key and value tiles of a step).
+// Against k_fwd_fused2<BI> (16 queries per wave): every key / value operand read from LDS feeds two matrix
+// instructions (the two 16-query tiles of the block), the staged tiles serve 256 queries instead of 128, and a bias
+// tile of k_carry2<BO> -- (16 keys, 32 queries), lane l owning bytes 16 l .. 16 l + 15 -- is exactly what a lane of
+// this kernel needs for a key tile, so it is loaded straight into registers one step ahead and never touches LDS.
+// 64 keys per step, key tiles visited from the diagonal backwards, two LDS stages.
+// ---------------------------------------------------------------------------------------------
+template <int D, int RB>
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+k_fwd_fused3(const bf16* __restrict__ Qp, const bf16* __restrict__ Kp, const bf16* __restrict__ VT, bf16* __restrict__ O,
+             float* __restrict__ lse, float* __restrict__ lse2, const int* __restrict__ reach, const int* __restrict__ minkey,
+             int R, int L, int Lp, int d, const _Float16* __restrict__ Bt) {
+  using T = bf16;
+  using TN = Tile<T, 32, D>;
+  using TT = Tile<T, D, 32>;
+  using ST = StageT<T>;
+  static_assert(RB == 1 || RB == 2 || RB == 4, "1, 2 or 4 query groups per workgroup");
+  constexpr int NK = D / 32, ND = D / 16, NST = 2, NB = 8 / RB;
+  constexpr int TILES = 2 * TN::BYTES + 2 * TT::BYTES, SB = TILES + 1024;     // + reach of the step's four key tiles
+  UA_STAGES(SB);
+  __shared__ __attribute__((aligned(256))) char sPbuf[8 * 4 * ST::BYTES];     // per wave: P of (query tile, 32-key half)
+  typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
+  int bx, zy;
+  xcd_map(bx, zy);
+  const int zq = RB == 1 ? zy : (zy / (R / RB)) * R + (zy % (R / RB)) * RB + w % RB;
+  const int zk = zq / R, nT16 = Lp / 16, nT32 = Lp / 32;
+  const int jt = gridDim.x - 1 - bx;                          // heaviest workgroups first
+  const int qb_raw = NB * jt + w / RB;
+  const bool live = qb_raw < nT32;                            // the last workgroup may hold waves past the end
+  const int qb = live ? qb_raw : nT32 - 1;                    // 32-query block of this wave
+  char* sPw = sPbuf + w * 4 * ST::BYTES;
+  Stager<TN, 8> stN;
+  Stager<TT, 8> stT;
+  stN.init(w, lane, D * (long)sizeof(T), 32);
+  stT.init(w, lane, Lp * (long)sizeof(T), D);
+
+  Frag<T> qf[2][NK];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int q = 0; q < NK; ++q) qf[i][q] = ld8(Qp + nat_off<D>(zq, Lp, 32 * qb + 16 * i + col, 32 * q + 8 * g));
+  f32x4 o[2][ND], m[2], ls[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+#pragma unroll
+    for (int n = 0; n < ND; ++n) o[i][n] = (f32x4){0, 0, 0, 0};
+    m[i] = (f32x4){-1.0e30f, -1.0e30f, -1.0e30f, -1.0e30f};
+    ls[i] = (f32x4){0, 0, 0, 0};
+  }
+  const T* Kz = Kp + (long)zk * Lp * D;
+  const T* Vz = VT + (long)zk * D * Lp;
+  const int qb_end = min(NB * (jt + 1), nT32);
+  const int n_kt = (qb_end + 1) / 2;                          // key tiles of 64 covering s <= last query of the workgroup
+  // key tiles that cannot reach this workgroup's first query block (see k_carry2) are not visited
+  const int kt_min = minkey[zk * nT32 + NB * jt] >> 2;
+  const int n_steps = n_kt - kt_min;
+  // this lane's 16 bytes of key tile 0 of the wave's query block
+  const char* bt_src = reinterpret_cast<const char*>(Bt) + (((long)zk * tri_tiles(nT32) + tri_bias_row(qb)) << 10) + 16 * lane;
+  f16x8 hb_next[4];
+  auto load_bias = [&] __device__ (int kt) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      hb_next[j] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(bt_src + ((long)(4 * kt + j) << 10)));
+  };
+
+#define UA_ISSUE(s, base)                                                                   \
+  {                                                                                         \
+    const int kt_ = n_kt - 1 - (s);                                                         \
+    stN.issue((base), Kz + (long)(64 * kt_) * D, w);                                        \
+    stN.issue((base) + TN::BYTES, Kz + (long)(64 * kt_ + 32) * D, w);                       \
+    stT.issue((base) + 2 * TN::BYTES, Vz + (long)(2 * kt_) * (32 * D), w);                  \
+    stT.issue((base) + 2 * TN::BYTES + TT::BYTES, Vz + (long)(2 * kt_ + 1) * (32 * D), w);  \
+    if (w == 0) issue_row((base) + TILES, reach + zk * nT16 + 4 * kt_);                      \
+  }
+#define UA_COMPUTE_FAST(s, base) fwd_tile(n_kt - 1 - (s), (base), FalseC())
+#define UA_COMPUTE_SLOW(s, base) fwd_tile(n_kt - 1 - (s), (base), TrueC())
+  auto fwd_tile = [&] __device__ (int kt, const char* base, auto masked_c) {
+    constexpr bool MASKED = decltype(masked_c)::value;
+    // the bias tiles of this step arrived during the previous one; fetch the next step's (a tile row is followed by
+    // the next rows and the tensor by slack, so the loads of the last step stay inside the tensor)
+    f16x8 hb[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) hb[j] = hb_next[j];
+    if (kt > 0) load_bias(kt - 1);
+    if (MASKED && 4 * kt > 2 * qb + 1) return;         // the whole step lies after this wave's queries
+    const int* rch = reinterpret_cast<const int*>(base + TILES);
+    f32x4 s2[2][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int sbk = 4 * kt + j;                      // 16-key tile
+      const T* sK = reinterpret_cast<const T*>(base + (j >> 1) * TN::BYTES);
+      if (!MASKED || sbk <= 2 * qb + 1) {
+        f32x4 sc[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+#pragma unroll
+        for (int q = 0; q < NK; ++q) {
+          const Frag<T> kb = ld8(sK + TN::at(j & 1, col, q, g));
+          mma16(sc[0], qf[0][q], kb);
+          mma16(sc[1], qf[1][q], kb);
+        }
+        const bool in_reach = rch[j] >= qb;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const int tq = 2 * qb + i;
+          const bool diag = MASKED && sbk == tq, after = MASKED && sbk > tq;
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            const float x = in_reach ? __builtin_fmaf(sc[i][v], kLog2e, (float)hb[j][4 * i + v]) : -1.0e30f;
+            s2[i][j][v] = (MASKED && (after || (diag && 4 * g + v < col))) ? -1.0e30f : x;
+          }
+        }
+      } else {
+        s2[0][j] = (f32x4){-1.0e30f, -1.0e30f, -1.0e30f, -1.0e30f};
+        s2[1][j] = s2[0][j];
+      }
+    }
+    // online softmax: rescale only when some query of this wave raises its maximum
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      f32x4 mx;
+      bool grow = false;
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        mx[v] = allmax16(fmaxf(fmaxf(s2[i][0][v], s2[i][1][v]), fmaxf(s2[i][2][v], s2[i][3][v])));
+        grow |= (mx[v] > m[i][v]);
+      }
+      if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const float mn = fmaxf(m[i][v], mx[v]);
+          const float alpha = __builtin_amdgcn_exp2f(m[i][v] - mn);
+          m[i][v] = mn;
+          ls[i][v] *= alpha;
+#pragma unroll
+          for (int n = 0; n < ND; ++n) o[i][n][v] *= alpha;
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        f32x4 p;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          p[v] = __builtin_amdgcn_exp2f(s2[i][j][v] - m[i][v]);
+          ls[i][v] += p[v];
+        }
+        ST::put(sPw + (2 * i + (j >> 1)) * ST::BYTES, 16 * (j & 1) + col, g, p);
+      }
+    }
+#pragma unroll
+    for (int kq = 0; kq < 2; ++kq) {                   // 32 keys per k-step
+      if (!MASKED || 4 * kt + 2 * kq <= 2 * qb + 1) {
+        const T* sV = reinterpret_cast<const T*>(base + 2 * TN::BYTES + kq * TT::BYTES);
+        const Frag<T> pa0 = ST::get(sPw + kq * ST::BYTES, lane), pa1 = ST::get(sPw + (2 + kq) * ST::BYTES, lane);
+#pragma unroll
+        for (int n = 0; n < ND; ++n) {
+          const Frag<T> vb = ld8(sV + TT::at(n, col, 0, g));
+          mma16(o[0][n], pa0, vb);
+          mma16(o[1][n], pa1, vb);
+        }
+      }
+    }
+  };
+  {
+    // the key tiles visited first hold the diagonal blocks of the waves: those with keys of the workgroup's own blocks
+    const int nslow = min(n_steps, (n_kt - (NB * jt) / 2 + 1) & ~1);
+    if (n_steps > 0) load_bias(n_kt - 1);
+    UA_PIPE_START(n_steps, UA_ISSUE);
+    UA_PIPE_RANGE(0, nslow, n_steps, UA_ISSUE, UA_COMPUTE_SLOW);
+    UA_PIPE_RANGE(nslow, n_steps, n_steps, UA_ISSUE, UA_COMPUTE_FAST);
+  }
+#undef UA_ISSUE
+#undef UA_COMPUTE_FAST
+#undef UA_COMPUTE_SLOW
+  if (!live) return;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const float tot = allsum16(ls[i][v]);
+      const float inv = 1.0f / tot;
+      const int t = 32 * qb + 16 * i + 4 * g + v;
+      if (t < L) {
+#pragma unroll
+        for (int n = 0; n < ND; ++n) {
+          const int dd = 16 * n + col;
+          if (dd < d) O[((long)zq * L + t) * d + dd] = cvt<T>(o[i][n][v] * inv);
+        }
+      }
+      if (col == 0) {
+        const float l2v = m[i][v] + __builtin_amdgcn_logf(tot);
+        lse2[(long)zq * Lp + t] = (t < L) ? l2v : 0.f;
+        if (t < L) lse[(long)zq * L + t] = l2v * kLn2;
+      }
+    }
+}
+
 // The A operand [16 features 16n.. x 32 positions] of a "transposed" product out of the NATURAL tile [32 positions][D]
 // (k-group-major, see Tile): two transposing reads, each turning a block of 4 positions x 16 features (8 bytes per lane:
 // lane i of a 16-lane group supplies position i/4 of the block and features 4(i%4)..+3) into 4 positions of feature i
@@ -687,6 +890,12 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
 #pragma unroll
   for (int n = 0; n < ND; ++n) { dVt[n] = (f32x4){0, 0, 0, 0}; dKt[n] = (f32x4){0, 0, 0, 0}; }
   float dsrc_acc = 0.f, dcar = 0.f;
+  // 16-bit operands: the reverse running sum of dS over the block's queries runs on the matrix core (scan32_mma); dcar4
+  // replaces dcar, and with several query groups (MR) the groups' sums accumulate in dB through the same products
+  constexpr bool MS = sizeof(T) == 2;
+  ScanOps sc_ops;
+  f32x4 dcar4 = {0, 0, 0, 0}, dtot4 = {0, 0, 0, 0};
+  if constexpr (MS) sc_ops = scan_operands<true>(lane);
   f32x4 aff_s[2], bias_s[2], gk_s[2], dB_s[2];     // state of the current query block (used when MR); gk = relu(G)
   const T* Kz = a.Kp + (long)zk * Lp * D;
   const T* KTz = a.KT + (long)zk * D * Lp;
@@ -868,30 +1077,49 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
         if constexpr (TR) mma16(dKt[n], ld8_tr<T>(sQ, n, lane), bs);
         else mma16(dKt[n], ld8(sQT + TT::at(n, col, 0, g)), bs);
       }
+      if constexpr (MS) {
+        // dB (+)= reverse running sums of this group's dS; the block totals of the groups add up in dtot4
+        if (!MR || r == 0) { dB[0] = dcar4; dB[1] = dcar4; if (MR) dtot4 = dcar4; }
+        mma16(dB[0], sc_ops.tri[0], bs);
+        mma16(dB[1], sc_ops.tri[1], bs);
+        mma16(MR ? dtot4 : dcar4, sc_ops.ones, bs);
+      }
       __builtin_amdgcn_s_setprio(0);
+      if constexpr (!MS) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) dB[i][v] = MR ? dB[i][v] + dS[i][v] : dS[i][v];
+          for (int v = 0; v < 4; ++v) dB[i][v] = MR ? dB[i][v] + dS[i][v] : dS[i][v];
+      }
     }
     if (!MR || r == R - 1) {
-      float t1;
-      const float tot = suffix32(dB[0], dB[1], gm, t1);
-      if (!BI && g == 0) {
-        Dz[(long)(2 * tb + 1) * Lp] = dcar;
-        Dz[(long)(2 * tb) * Lp] = dcar + t1;
+      float t1 = 0.f, tot = 0.f;
+      if constexpr (MS) {
+        // suffix carries for the recomputing query side: before the block's second tile, before its first
+        if (!BI && g == 0) {
+          Dz[(long)(2 * tb + 1) * Lp] = dcar;
+          Dz[(long)(2 * tb) * Lp] = dB[1][0];
+        }
+        if (MR) dcar4 = dtot4;
+      } else {
+        tot = suffix32(dB[0], dB[1], gm, t1);
+        if (!BI && g == 0) {
+          Dz[(long)(2 * tb + 1) * Lp] = dcar;
+          Dz[(long)(2 * tb) * Lp] = dcar + t1;
+        }
       }
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
-          float dl = dB[i][v] + dcar;
+          float dl = MS ? dB[i][v] : dB[i][v] + dcar;
           if (MASKED) dl = (diag && tl0 + 16 * i + v <= 0) ? 0.f : dl;
           dB[i][v] = decay_grad(dl, aff[i][v], gk[i][v]);
           dsrc_acc = __builtin_fmaf(dB[i][v], gk[i][v], dsrc_acc);
         }
       }
-      dcar += tot;
+      if constexpr (MS) dcar = dcar4[0];
+      else dcar += tot;
       const Frag<T> b = as_operand16<T>(dB[0], dB[1]);
       if constexpr (TO) {
         char* p = reinterpret_cast<char*>(a.dG_st) + (long)zo * st_head + (grp_tile(2 * tb, sb16 >> 1) << 10) + st_lane;

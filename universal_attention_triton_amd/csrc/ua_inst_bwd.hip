@@ -99,11 +99,15 @@ hipError_t launch_bwd_queries(int dtype, int D, const BwdArgsV& a, void* dq, int
 
 template __global__ void k_bwd_queries3<bf16, 64, 2, 1>(BwdArgs<bf16>, bf16*, int);
 template __global__ void k_bwd_queries3<bf16, 128, 2, 1>(BwdArgs<bf16>, bf16*, int);
-hipError_t launch_bwd_queries_from_tiles(int D, const BwdArgsV& v, void* dq, int d, int Zq, hipStream_t s) {
+template __global__ void k_bwd_queries3<bf16, 64, 2, 2>(BwdArgs<bf16>, bf16*, int);
+template __global__ void k_bwd_queries3<bf16, 128, 2, 2>(BwdArgs<bf16>, bf16*, int);
+hipError_t launch_bwd_queries_from_tiles(int D, const BwdArgsV& v, void* dq, int d, int Zq, hipStream_t s, int variant) {
   const BwdArgs<bf16> a = typed<bf16>(v);
   const dim3 grid(v.Lp / 128, Zq);
-  if (D == 64) hipLaunchKernelGGL((k_bwd_queries3<bf16, 64, 2, 1>), grid, dim3(512), 0, s, a, (bf16*)dq, d);
-  else hipLaunchKernelGGL((k_bwd_queries3<bf16, 128, 2, 1>), grid, dim3(512), 0, s, a, (bf16*)dq, d);
+#define UA_Q3(D_, HV_) hipLaunchKernelGGL((k_bwd_queries3<bf16, D_, 2, HV_>), grid, dim3(512), 0, s, a, (bf16*)dq, d)
+  if (variant == 1) { if (D == 64) UA_Q3(64, 2); else UA_Q3(128, 2); }
+  else { if (D == 64) UA_Q3(64, 1); else UA_Q3(128, 1); }
+#undef UA_Q3
   return hipGetLastError();
 }
 

@@ -1,6 +1,7 @@
 // Instantiations and launchers of the forward kernels.
 #include <algorithm>
 #include <cstdint>
+#include <cstdlib>
 #include "ua_fused.hpp"
 #include "ua_fwd.hpp"
 #include "ua_internal.hpp"
@@ -14,12 +15,13 @@ static void allow_lds(K kernel, size_t bytes) {
 
 template <class T, int D>
 static hipError_t carry_t(const void* Kp, const float* lsrc, const float* ldest, float* C, int Lp, int Zk, int tiled,
-                          const float* knorm2, const float* qnorm2, int R, int* reach, int* minkey, hipStream_t s, void* Bt) {
+                          const float* knorm2, const float* qnorm2, int R, int* reach, int* minkey, hipStream_t s, void* Bt,
+                          int variant) {
   constexpr int NST = 2;
   _Float16* none = nullptr;
-  // bias tiles: launches of under two 8-wave workgroups per CU are bound by the latency of a workgroup's serial sweep
-  // and run faster as twice as many 4-wave workgroups
-  if (tiled && Bt && sizeof(T) == 2 && (long)Zk * (Lp / 128) < 512)
+  // bias tiles, variant 1: 4-wave workgroups (launches of under two 8-wave workgroups per CU are bound by the latency
+  // of a workgroup's serial sweep and run faster as twice as many 4-wave workgroups)
+  if (tiled && Bt && sizeof(T) == 2 && variant == 1)
     hipLaunchKernelGGL((k_carry2<T, D, NST, true, true, 4>), dim3(Lp / 64, Zk), dim3(256), 0, s, (const T*)Kp, lsrc, ldest, C, Lp, knorm2, qnorm2, R, reach, (_Float16*)Bt);
   else if (tiled && Bt && sizeof(T) == 2) hipLaunchKernelGGL((k_carry2<T, D, NST, true, true>), dim3(Lp / 128, Zk), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, C, Lp, knorm2, qnorm2, R, reach, (_Float16*)Bt);
   else if (tiled) hipLaunchKernelGGL((k_carry2<T, D, NST, true, false>), dim3(Lp / 128, Zk), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, C, Lp, knorm2, qnorm2, R, reach, none);
@@ -33,8 +35,8 @@ static hipError_t carry_t(const void* Kp, const float* lsrc, const float* ldest,
 }
 hipError_t launch_carry(int dtype, int D, const void* Kp, const float* lsrc, const float* ldest, float* C, int Lp, int Zk,
                         int tiled, const float* knorm2, const float* qnorm2, int R, int* reach, int* minkey, hipStream_t s,
-                        void* Bt) {
-#define UA_ARGS Kp, lsrc, ldest, C, Lp, Zk, tiled, knorm2, qnorm2, R, reach, minkey, s, Bt
+                        void* Bt, int variant) {
+#define UA_ARGS Kp, lsrc, ldest, C, Lp, Zk, tiled, knorm2, qnorm2, R, reach, minkey, s, Bt, variant
   if (dtype == 1) return D == 64 ? carry_t<bf16, 64>(UA_ARGS) : carry_t<bf16, 128>(UA_ARGS);
   return D == 64 ? carry_t<float, 64>(UA_ARGS) : carry_t<float, 128>(UA_ARGS);
 #undef UA_ARGS
@@ -49,6 +51,12 @@ hipError_t launch_carry(int dtype, int D, const void* Kp, const float* lsrc, con
 #define UA_INST(T, D, NST, NW, CH) UA_INST2(T, D, NST, NW, CH, false)
 UA_INST3(bf16, 64, 1, 8, false, true, 2) UA_INST3(bf16, 128, 1, 8, false, true, 2) UA_INST3(bf16, 64, 1, 8, false, true, 4) UA_INST3(bf16, 128, 1, 8, false, true, 4)
 UA_INST2(bf16, 64, 1, 8, false, true) UA_INST2(bf16, 128, 1, 8, false, true) UA_INST2(bf16, 64, 1, 4, false, true) UA_INST2(bf16, 128, 1, 4, false, true)
+template __global__ void k_fwd_fused3<64, 1>(const bf16*, const bf16*, const bf16*, bf16*, float*, float*, const int*, const int*, int, int, int, int, const _Float16*);
+template __global__ void k_fwd_fused3<64, 2>(const bf16*, const bf16*, const bf16*, bf16*, float*, float*, const int*, const int*, int, int, int, int, const _Float16*);
+template __global__ void k_fwd_fused3<64, 4>(const bf16*, const bf16*, const bf16*, bf16*, float*, float*, const int*, const int*, int, int, int, int, const _Float16*);
+template __global__ void k_fwd_fused3<128, 1>(const bf16*, const bf16*, const bf16*, bf16*, float*, float*, const int*, const int*, int, int, int, int, const _Float16*);
+template __global__ void k_fwd_fused3<128, 2>(const bf16*, const bf16*, const bf16*, bf16*, float*, float*, const int*, const int*, int, int, int, int, const _Float16*);
+template __global__ void k_fwd_fused3<128, 4>(const bf16*, const bf16*, const bf16*, bf16*, float*, float*, const int*, const int*, int, int, int, int, const _Float16*);
 UA_INST(bf16, 64, 1, 8, false) UA_INST(bf16, 64, 2, 8, false) UA_INST(bf16, 64, 2, 12, false) UA_INST(bf16, 64, 2, 16, false)
 UA_INST(bf16, 128, 2, 4, false) UA_INST(bf16, 64, 2, 4, false) UA_INST(bf16, 128, 1, 8, false) UA_INST(bf16, 128, 2, 8, false) UA_INST(bf16, 128, 2, 12, false) UA_INST(bf16, 128, 2, 16, false)
 UA_INST(float, 64, 1, 8, false) UA_INST(float, 128, 1, 8, false)
@@ -66,26 +74,33 @@ static hipError_t fused_t(const void* Qp, const void* Kp, const void* VT, const 
                      (const T*)Kp, (const T*)VT, lsrc, ldest, C, (T*)O, lse, lse2, reach, minkey, R, L, Lp, d, ChunkOut<T>{}, none);
   return hipGetLastError();
 }
-// bf16 with bias tiles from launch_carry
+// bf16 with bias tiles from launch_carry; variant: UA_TUNE_FWD_TILES
+//   0: k_fwd_fused3, one 32-query block per wave (256-query workgroups, two LDS stages)
+//   1: k_fwd_fused2<BI>, 8-wave workgroups of 128 queries with a single LDS stage, two per CU, which cover each other's waits
+//   2: the same in 64-query pieces (r = 1; small launches are bound by their longest workgroups)
+// grouped queries: the groups of a kv head share the tiles of a 32-query block (see RB)
 template <int D>
-static hipError_t fused_bi(const void* Qp, const void* Kp, const void* VT, const float* lsrc, const float* ldest,
+static hipError_t fused_bi(int variant, const void* Qp, const void* Kp, const void* VT, const float* lsrc, const float* ldest,
                            const float* C, void* O, float* lse, float* lse2, const int* reach, const int* minkey, int R, int L,
                            int Lp, int d, int Zq, hipStream_t s, const void* Bt) {
   using T = bf16;
-  // 8-wave workgroups (128 queries) with a single LDS stage, two per CU, which cover each other's waits.  The kernel
-  // is bound by the key / value tiles it pulls from L2 (without those loads it runs 28 % faster), so queries per
-  // workgroup count: same box, b=1 h=32 L=8192 d=128: 1.07 ms, against 1.15 ms for three 4-wave workgroups per CU and
-  // 1.25 ms for one 8-wave workgroup with two stages
-  // Small launches (under about six 128-query workgroups per CU) are bound by their longest workgroups instead and
-  // run faster in 64-query pieces (config 3: 0.30 vs 0.33 ms; b=2 h=16 L=2048 d=64: 0.075 vs 0.085 ms).
-  // grouped queries: the groups of a kv head share the tiles of a 32-query block (see RB)
+  if (variant == 0) {
+#define UA_F3(RB_)                                                                                                          \
+  hipLaunchKernelGGL((k_fwd_fused3<D, RB_>), dim3((Lp / 32 + 8 / RB_ - 1) / (8 / RB_), Zq / RB_), dim3(512), 0, s, (const T*)Qp, \
+                     (const T*)Kp, (const T*)VT, (T*)O, lse, lse2, reach, minkey, R, L, Lp, d, (const _Float16*)Bt)
+    if (R % 4 == 0) UA_F3(4);
+    else if (R % 2 == 0) UA_F3(2);
+    else UA_F3(1);
+#undef UA_F3
+    return hipGetLastError();
+  }
 #define UA_SHARED(RB_)                                                                                                     \
   hipLaunchKernelGGL((k_fwd_fused2<T, D, 1, 8, false, true, RB_>), dim3(Lp / (128 / RB_), Zq / RB_), dim3(512), 0, s, (const T*)Qp, \
                      (const T*)Kp, (const T*)VT, lsrc, ldest, C, (T*)O, lse, lse2, reach, minkey, R, L, Lp, d, ChunkOut<T>{},      \
                      (const _Float16*)Bt)
   if (R % 4 == 0) UA_SHARED(4);
   else if (R % 2 == 0) UA_SHARED(2);
-  else if ((long)Zq * (Lp / 128) >= 1536)
+  else if (variant == 1)
     hipLaunchKernelGGL((k_fwd_fused2<T, D, 1, 8, false, true>), dim3(Lp / 128, Zq), dim3(512), 0, s, (const T*)Qp, (const T*)Kp,
                        (const T*)VT, lsrc, ldest, C, (T*)O, lse, lse2, reach, minkey, R, L, Lp, d, ChunkOut<T>{}, (const _Float16*)Bt);
   else
@@ -116,7 +131,7 @@ hipError_t launch_fwd_fused(int dtype, int D, int variant, const void* Qp, const
                             const int* reach, const int* minkey, int R, int L, int Lp, int d, int Zq, hipStream_t s,
                             const void* Bt) {
 #define UA_ARGS Qp, Kp, VT, lsrc, ldest, C, O, lse, lse2, reach, minkey, R, L, Lp, d, Zq, s
-  if (dtype == 1 && Bt) return D == 64 ? fused_bi<64>(UA_ARGS, Bt) : fused_bi<128>(UA_ARGS, Bt);
+  if (dtype == 1 && Bt) return D == 64 ? fused_bi<64>(variant, UA_ARGS, Bt) : fused_bi<128>(variant, UA_ARGS, Bt);
   if (dtype == 1) return D == 64 ? fused_v<bf16, 64>(variant, UA_ARGS) : fused_v<bf16, 128>(variant, UA_ARGS);
   return D == 64 ? fused_t<float, 64, 1, 8>(UA_ARGS) : fused_t<float, 128, 1, 8>(UA_ARGS);
 #undef UA_ARGS

@@ -25,14 +25,15 @@ struct BwdArgsV {
 // knorm2 [Zk][Lp/32], qnorm2 [Zk*R][Lp/32] (optional): largest squared row norm of every block of 32 keys / queries,
 // enables pruning; reach (optional): [Zk][Lp/16] out.  With reach given, minkey [Zk][Lp/32] is filled as well.
 // Bt (optional, bf16 + tiled): fp16 bias tiles [Zk][Lp/32][Lp/16][1 KB] are written instead of the carries C
+// variant (bias tiles only): UA_TUNE_CARRY
 hipError_t launch_carry(int dtype, int D, const void* Kp, const float* lsrc, const float* ldest, float* C, int Lp, int Zk,
                         int tiled, const float* knorm2, const float* qnorm2, int R, int* reach, int* minkey, hipStream_t s,
-                        void* Bt = nullptr);
+                        void* Bt = nullptr, int variant = 0);
 int fwd_fused_variants(int dtype, int D);
 hipError_t launch_fwd_fused(int dtype, int D, int variant, const void* Qp, const void* Kp, const void* VT,
                             const float* lsrc, const float* ldest, const float* C, void* O, float* lse, float* lse2,
                             const int* reach, const int* minkey, int R, int L, int Lp, int d, int Zq, hipStream_t s,
-                            const void* Bt = nullptr);   // Bt (bf16): bias tiles of launch_carry; overrides the variant
+                            const void* Bt = nullptr);   // Bt (bf16): bias tiles of launch_carry; variant is then UA_TUNE_FWD_TILES
 hipError_t launch_fwd_chunked(int dtype, int D, const void* Qp, const void* Kp, const void* VT, const float* lsrc,
                               const float* ldest, void* out, void* denom, float* lse2, long o_sz, long o_st, long o_sd,
                               long o_si, int R, int L, int Lp, int d, int c, int nch, int Zk, hipStream_t s);
@@ -49,7 +50,8 @@ hipError_t launch_fwd_chunked2(int dtype, int D, const void* Qp, const void* Kp,
 hipError_t launch_bwd_keys(int dtype, int D, const BwdArgsV& a, int Zk, int cols, hipStream_t s);
 hipError_t launch_bwd_queries(int dtype, int D, const BwdArgsV& a, void* dq, int d, int Zk, hipStream_t s);
 // bf16 only, a.dS_st / a.dG_st filled by launch_bwd_keys (cols == 0): the query side as pure matrix work over those tiles
-hipError_t launch_bwd_queries_from_tiles(int D, const BwdArgsV& a, void* dq, int d, int Zq, hipStream_t s);
+// variant: UA_TUNE_BWD_QUERIES
+hipError_t launch_bwd_queries_from_tiles(int D, const BwdArgsV& a, void* dq, int d, int Zq, hipStream_t s, int variant = 0);
 
 // Stand-alone decay bias (affinity scores): aff [Z][L][L] in the dtype; working tensors tiled like the fused operator's.
 hipError_t launch_aff_fwd(int dtype, int D, const void* Kp, const float* lsrc, const float* ldest, void* aff, int L, int Lp, int Z,

@@ -152,7 +152,8 @@ def fused_forward(kc, vc, xq, static_src, static_dest, for_backward=False, prune
     return O, lse, ws
 
 
-def fused_backward(kc, vc, xq, static_src, static_dest, O, lse, dO, ws=None, prune=False, recompute=False, share_groups=False):
+def fused_backward(kc, vc, xq, static_src, static_dest, O, lse, dO, ws=None, prune=False, recompute=False, share_groups=False,
+                   _ws_override=None):
     """ws: the state fused_forward returned for the same inputs (skips the recompute and keeps its pruning);
     prune only matters when ws is None.  recompute: UA_FLAG_RECOMPUTE (small workspace, slower; bf16 only)."""
     kc, vc, xq, src, dest = _prep(kc, vc, xq, static_src, static_dest)
@@ -163,7 +164,9 @@ def fused_backward(kc, vc, xq, static_src, static_dest, O, lse, dO, ws=None, pru
     desc = _desc(kc, xq, False, _fused_flags(prune, recompute, share_groups))
     has_fwd = ws is not None
     need = lib.ua_workspace_bytes(ctypes.byref(desc), _lib.UA_OP_FUSED_BWD)
-    if ws is None or ws.numel() < need:
+    if _ws_override is not None:
+        ws, has_fwd = _ws_override, False
+    elif ws is None or ws.numel() < need:
         ws, has_fwd = _workspace(desc, _lib.UA_OP_FUSED_BWD, xq.device), False
     O = O.contiguous()
     dO = dO.to(xq.dtype).contiguous()
@@ -226,28 +229,60 @@ def merge_backward(mat, vec, g):
     return d_mat, d_vec.to(vec.dtype)
 
 
-def autotune(kc, vc, xq, static_src, static_dest, op=_lib.UA_OP_FUSED_FWD):
-    """Times the kernel variants of `op` for this problem on the current stream and records the fastest in the
-    library's table (what the reference's @triton.autotune does on first call).  Returns the variant id."""
-    kc, vc, xq, src, dest = _prep(kc, vc, xq, static_src, static_dest)
+def autotune(kc, vc, xq, static_src, static_dest, dO=None, backward=True):
+    """What the reference's @triton.autotune does on first call: runs the fused operator once on these inputs, then
+    times every variant of every kernel on its path on the device (ua_autotune) and records the fastest of each in the
+    library's table.  Returns {slot name: variant} for the slots that have more than one variant here."""
     lib = _lib.load()
-    desc = _desc(kc, xq, op in (_lib.UA_OP_FWD, _lib.UA_OP_BWD))
-    ws = _workspace(desc, _lib.UA_OP_FUSED_BWD if op >= _lib.UA_OP_FUSED_FWD else _lib.UA_OP_BWD, xq.device)
-    v = lib.ua_autotune(ctypes.byref(desc), op, ws.data_ptr(), ws.numel(), _stream())
-    _lib.check(v, "ua_autotune")
-    return v
+    O, lse, ws = fused_forward(kc, vc, xq, static_src, static_dest, for_backward=True)
+    kc_, vc_, xq_, _, _ = _prep(kc, vc, xq, static_src, static_dest)
+    desc = _desc(kc_, xq_, False)
+    _lib.check(lib.ua_autotune(ctypes.byref(desc), _lib.UA_OP_FUSED_FWD, ws.data_ptr(), ws.numel(), _stream()), "ua_autotune")
+    if backward and xq.dtype == torch.bfloat16:
+        # the number of key-side parts changes the workspace: tune it on a workspace large enough for every choice
+        if dO is None:
+            dO = torch.ones_like(O)
+        need = max(_with_parts(desc, v, lambda: lib.ua_workspace_bytes(ctypes.byref(desc), _lib.UA_OP_FUSED_BWD))
+                   for v in range(lib.ua_tune_variants(ctypes.byref(desc), _lib.UA_TUNE_BWD_PARTS)))
+        big = torch.empty(need, dtype=torch.uint8, device=xq.device)
+        fused_backward(kc, vc, xq, static_src, static_dest, O, lse, dO, ws=None, _ws_override=big)
+        _lib.check(lib.ua_autotune(ctypes.byref(desc), _lib.UA_OP_FUSED_BWD, big.data_ptr(), big.numel(), _stream()), "ua_autotune")
+    out = {name: lib.ua_tune_get(ctypes.byref(desc), slot) for name, slot in _lib.TUNE_SLOTS.items()
+           if lib.ua_tune_variants(ctypes.byref(desc), slot) > 1 and lib.ua_tune_get(ctypes.byref(desc), slot) >= 0}
+    from . import tune
+    for name, v in out.items():
+        tune.record(desc, name, v)
+    return out
 
 
-def tune_variants(kc, xq, op=_lib.UA_OP_FUSED_FWD):
-    return _lib.load().ua_tune_variants(ctypes.byref(_desc(kc, xq, False)), op)
+def _with_parts(desc, variant, fn):
+    lib = _lib.load()
+    old = lib.ua_tune_get(ctypes.byref(desc), _lib.UA_TUNE_BWD_PARTS)
+    lib.ua_tune_set(ctypes.byref(desc), _lib.UA_TUNE_BWD_PARTS, variant)
+    try:
+        return fn()
+    finally:
+        lib.ua_tune_set(ctypes.byref(desc), _lib.UA_TUNE_BWD_PARTS, old)
 
 
-def tune_set(kc, xq, variant, op=_lib.UA_OP_FUSED_FWD):
-    _lib.check(_lib.load().ua_tune_set(ctypes.byref(_desc(kc, xq, False)), op, variant), "ua_tune_set")
+def _slot(slot):
+    return _lib.TUNE_SLOTS[slot] if isinstance(slot, str) else slot
 
 
-def tune_get(kc, xq, op=_lib.UA_OP_FUSED_FWD):
-    return _lib.load().ua_tune_get(ctypes.byref(_desc(kc, xq, False)), op)
+def tune_variants(kc, xq, slot="fwd_tiles"):
+    return _lib.load().ua_tune_variants(ctypes.byref(_desc(kc, xq, False)), _slot(slot))
+
+
+def tune_set(kc, xq, variant, slot="fwd_tiles"):
+    _lib.check(_lib.load().ua_tune_set(ctypes.byref(_desc(kc, xq, False)), _slot(slot), variant), "ua_tune_set")
+
+
+def tune_get(kc, xq, slot="fwd_tiles"):
+    return _lib.load().ua_tune_get(ctypes.byref(_desc(kc, xq, False)), _slot(slot))
+
+
+def tune_choice(kc, xq, slot="fwd_tiles"):
+    return _lib.load().ua_tune_choice(ctypes.byref(_desc(kc, xq, False)), _slot(slot))
 
 
 def _affinity_args(k, src, dest):
