@@ -109,6 +109,26 @@ def cpu_baseline(cfg, index, budget_s=10.0):
                       % (heads, cfg["b"] * cfg["h"], cfg["r"], cfg["L"], cfg["d"], cfg["c"], " + backward" if cfg["bwd"] else "")}
 
 
+def parity_one_head(cfg, inp, O, grads, head=(0, 0)):
+    """Largest relative error (Frobenius norm per tensor) of O and the five gradients of one (batch, kv head) against the
+    oracle, the reference's chunked torch operator restated, evaluated in float32 on the same dtype-rounded inputs."""
+    from oracle import ua_oracle as orc
+    names = ("kc", "vc", "xq", "static_src", "static_dest")
+    bi, hi = head
+    one = [inp[k][bi:bi + 1, hi:hi + 1].float() for k in names]
+    out, denom = orc.chunked_forward(*one)
+    errs = {"O": float(((O[bi:bi + 1, hi:hi + 1].float().cpu() - orc.merge(out, denom)).norm() / orc.merge(out, denom).norm()))}
+    if grads is not None:
+        d_out, d_denom = orc.merge_backward(out, denom, inp["dO"][bi:bi + 1, hi:hi + 1].float())
+        ref = orc.chunked_backward(*one, d_out, d_denom.float())
+        for k, g, r in zip(names, grads, ref):
+            g1 = g[bi:bi + 1, hi:hi + 1].float().cpu().reshape(r.shape)
+            errs["d" + k] = float((g1 - r).norm() / r.norm())
+    worst = max(errs, key=errs.get)
+    return {"max_rel_err": round(errs[worst], 6), "tensor": worst, "head": list(head), "tolerance": 2e-2 if cfg["dtype"] == "bf16" else 1e-4,
+            "against": "oracle (reference torch operator restated, float32) on the same inputs, one (batch, kv head)"}
+
+
 # HBM bytes per launch of the roofline kernel, from the TCC counters FETCH_SIZE and WRITE_SIZE of two `rocprofv3 --pmc`
 # runs of this script, each scaled by what the same counter reads for the plain 1 GiB copy of --calibrate-copy
 # (profiles/bench_cfg2_fused_fwd_bwd.md: 3.74 GB read + 4.58 GB written by k_bwd_keys2).  A measured constant, not
@@ -157,10 +177,12 @@ def bench_affinity(args, cfg, inp):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=None, help="timed steps (default: enough for a timed region of about 1 s)")
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", type=int, default=2)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-parity", action="store_true", help="skip the one-head oracle check of the outputs and gradients")
+    ap.add_argument("--chunk", type=int, default=None, help="--api chunked: keys per chunk (default: the config's, 128)")
     ap.add_argument("--api", choices=["fused", "chunked", "affinity"], default="fused",
                     help="fused (default): universal_attention(); chunked: the reference's call sequence "
                          "UniversalAttention.apply + SMVecMatMul.apply, which materialises out[b,h,r,L,d,n]")
@@ -181,7 +203,11 @@ def main():
         _build.build()
     from universal_attention_triton_amd.universal_attention import universal_attention
 
-    cfg = CONFIGS[args.config]
+    cfg = dict(CONFIGS[args.config])
+    if args.chunk:
+        cfg["c"] = args.chunk
+    if args.steps is None:      # about one second of timed steps
+        args.steps = {0: 2000, 1: 2000, 2: 200, 3: 600, 4: 50}[args.config] if args.api == "fused" else 40
     dt = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float32
     inp = orc.make_inputs(cfg["b"], cfg["h"], cfg["r"], cfg["L"], cfg["d"], cfg["c"], dtype=dt, seed=1000 + args.config,
                           gate_mean=cfg["mu"])
@@ -261,6 +287,22 @@ def main():
         hk = hbm_kernels(cfg, kern)
         if hk:
             out["config"]["hbm_kernels"] = hk
+        if cfg["bwd"]:
+            from universal_attention_triton_amd import ops
+            out["config"]["bytes_retained_fwd_to_bwd"] = {
+                "forward_state": ops.retained_bytes(*[x.detach() for x in leaves]),
+                "O_and_lse": leaves[2].numel() * leaves[2].element_size() + leaves[2].numel() // cfg["d"] * 4,
+                "note": "the backward's scratch is allocated inside backward; keep_state=False retains O and lse only"}
+    if not args.no_parity and args.api in ("fused", "chunked"):
+        res = step()
+        torch.cuda.synchronize()
+        if cfg["bwd"]:
+            with torch.no_grad():
+                O_chk = universal_attention(*leaves)
+            out["parity"] = parity_one_head(cfg, inp, O_chk, res)
+        else:
+            out["parity"] = parity_one_head(cfg, inp, res, None)
+        del res
     if args.api == "chunked":
         out["roofline"] = roof
         out["config"]["workload"] += "; chunked API (reference call sequence, chunk %d)" % cfg["c"]

@@ -35,7 +35,9 @@ enum {
   UA_OP_FWD = 0,       /* ua_fwd        */
   UA_OP_BWD = 1,       /* ua_bwd        */
   UA_OP_FUSED_FWD = 2, /* ua_fused_fwd  */
-  UA_OP_FUSED_BWD = 3  /* ua_fused_bwd  */
+  UA_OP_FUSED_BWD = 3, /* ua_fused_bwd  */
+  UA_OP_BWD_SCRATCH = 4,       /* ua_workspace_bytes only: ua_bwd's workspace when it is given the forward state */
+  UA_OP_FUSED_BWD_SCRATCH = 5  /* ua_workspace_bytes only: likewise for ua_fused_bwd */
 };
 enum {
   UA_FLAG_SKIP_MASKED = 1, /* ua_bwd: the upstream gradient is zero for (query, chunk) pairs in which the
@@ -54,10 +56,13 @@ enum {
                               Without the flag it does so only when there are enough kv heads to fill the device and
                               otherwise divides the groups into parts with a sweep each (more workspace: the key-side
                               partial sums are then kept per part).  Same results up to summation order. */
+  UA_FLAG_GATES_F32 = 16,  /* bf16 ops: static_src, static_dest and the gradients dsrc, ddest are float32 tensors (the
+                              reference allocates dstatic_src in static_src.dtype and accepts float32 gates next to
+                              bf16 q, k, v: universal_attention_kernel.py:825-829).  float32 ops: always so. */
   UA_FLAG_PRUNE = 2        /* fused ops: skip (key, query) pairs whose softmax weight is provably below 2^-48 because
                               of the accumulated decay (no counterpart in the reference, which visits every pair).
                               The bound uses the largest key and query norms of the head; results change by less
-                              than float32 rounding.  ua_fused_bwd with ws_has_fwd follows what the forward recorded. */
+                              than float32 rounding.  ua_fused_bwd with the forward state follows what the forward recorded. */
 };
 
 /* Problem description.  kc, vc: [b,h,L,d] seen as [b,h,n,c,d]; xq: [b,h,r,L,d]; gates: [b,h,L]. */
@@ -89,8 +94,10 @@ int ua_version(void);
 const char* ua_last_error(void);
 
 /* Bytes of scratch `ws` the given op needs (0 and an error string if the shape is unsupported).
- * The backward ops can reuse the forward's workspace contents: size it with the backward op and pass
- * the same buffer to both calls. */
+ * A forward op leaves its state (packed inputs, log-gates, bias tiles or carries, normalisers) in its workspace.  A
+ * backward op either receives that buffer as `fwd_state` -- its own `ws` then needs UA_OP_(FUSED_)BWD_SCRATCH bytes -- or
+ * rebuilds the state inside a `ws` of UA_OP_(FUSED_)BWD bytes (= forward state + scratch).  What a caller keeps alive
+ * between forward and backward is therefore the forward state at most, and nothing with fwd_state = NULL. */
 size_t ua_workspace_bytes(const ua_desc* desc, int op);
 
 /* Chunked forward: replaces _universal_attention_fwd
@@ -104,10 +111,11 @@ int ua_fwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
  * UniversalAttention.backward (universal_attention_autograd.py:47-99).
  * out: the forward's result; g_out: same indexing; g_denom: contiguous float32 [b,h,r,L,n].
  * Gradients are written contiguous: dkc, dvc [b,h,L,d]; dxq [b,h,r,L,d]; dsrc, ddest [b,h,L].
- * ws_has_fwd != 0: `ws` still holds what ua_fwd left there for the same inputs (skips the recompute). */
+ * fwd_state: NULL, or the workspace ua_fwd ran on for the same inputs and flags, contents intact (skips the recompute;
+ * the backward rewrites parts of it with the same values). */
 int ua_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
            const void* static_dest, const ua_chunked* out, const ua_chunked* g_out, const float* g_denom, void* dkc,
-           void* dvc, void* dxq, void* dsrc, void* ddest, void* ws, size_t ws_bytes, int ws_has_fwd, ua_stream_t stream);
+           void* dvc, void* dxq, void* dsrc, void* ddest, void* fwd_state, void* ws, size_t ws_bytes, ua_stream_t stream);
 
 /* Fused forward: the chunked operator followed by SMVecMatMul (universal_attention_autograd.py:278-283)
  * without materialising the per-chunk tensor; same role as the reference's second-generation
@@ -122,7 +130,7 @@ int ua_fused_fwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, cons
  * the library's load until the process ends.  Problems whose ua_workspace_bytes(desc, UA_OP_FUSED_FWD) exceeds it are
  * refused with UA_EWORKSPACE.  Calls no hipMalloc / hipFree.  All calls on one GPU share the array: two calls that
  * overlap on one GPU (different streams or threads) race, and the forward state a later ua_fused_bwd could reuse is not
- * kept (call ua_fused_bwd with ws_has_fwd = 0). */
+ * kept (call ua_fused_bwd with fwd_state = NULL). */
 #define UA_NOALLOC_SCRATCH_BYTES (64u << 20)
 size_t ua_noalloc_scratch_bytes(void);
 int ua_fused_fwd_noalloc(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
@@ -130,10 +138,11 @@ int ua_fused_fwd_noalloc(const ua_desc* desc, const ua_rows* kc, const ua_rows* 
 
 /* Fused backward: replaces SMVecMatMul.backward + UniversalAttention.backward
  * (universal_attention_autograd.py:291-297, :47-99) / _attention.backward (universal_attention_kernel_opt.py:504-581).
- * O, lse: as produced by ua_fused_fwd; dO contiguous [b,h,r,L,d]. */
+ * O, lse: as produced by ua_fused_fwd; dO contiguous [b,h,r,L,d].  fwd_state: as for ua_bwd (the workspace of
+ * ua_fused_fwd, or NULL). */
 int ua_fused_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
                  const void* static_dest, const void* O, const float* lse, const void* dO, void* dkc, void* dvc,
-                 void* dxq, void* dsrc, void* ddest, void* ws, size_t ws_bytes, int ws_has_fwd, ua_stream_t stream);
+                 void* dxq, void* dsrc, void* ddest, void* fwd_state, void* ws, size_t ws_bytes, ua_stream_t stream);
 
 /* Chunk merge: replaces SMVecMatMul.forward / .backward (universal_attention_autograd.py:278-297).
  * rows = number of (b,h,r,t) rows, n chunks, d features.  mat element (row, dd, i) at
@@ -178,9 +187,10 @@ enum {
 };
 /* ua_autotune(desc, op, ...) with op = UA_OP_FUSED_FWD or UA_OP_FUSED_BWD times every variant of every kernel slot on
  * that op's path for desc (hipEvents on `stream`, synchronises) and records the fastest of each.  `ws` must hold what
- * the op itself left there for desc: call ua_fused_fwd (resp. ua_fused_fwd + ua_fused_bwd with ws_has_fwd) on the same
- * workspace first; the tuning runs re-launch the kernels on that state.  UA_OP_FUSED_BWD clobbers the backward part of
- * the workspace (the forward state stays valid).  Returns 0 or a negative error. */
+ * the op itself left there for desc, state and scratch in ONE buffer of ua_workspace_bytes(desc, UA_OP_FUSED_BWD) bytes:
+ * call ua_fused_fwd on it, and for the backward also ua_fused_bwd with fwd_state = ws and its scratch at
+ * ws + ua_workspace_bytes(desc, UA_OP_FUSED_FWD); the tuning runs re-launch the kernels on that state.  UA_OP_FUSED_BWD
+ * clobbers the scratch part (the forward state stays valid).  Returns 0 or a negative error. */
 int ua_autotune(const ua_desc* desc, int op, void* ws, size_t ws_bytes, ua_stream_t stream);
 /* Table access for persistence: entry of (slot, desc) set by ua_tune_set / ua_autotune, -1 if none. */
 int ua_tune_get(const ua_desc* desc, int slot);

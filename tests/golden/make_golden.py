@@ -3,7 +3,7 @@ operator (reference ``universal_attention_autograd.py``) on the CPU, once, in th
 build container.  The reference is only imported here; the fixtures it writes
 are data (inputs + expected outputs) and are what the tests read.
 
-    python tests/golden/make_golden.py [/root/reference]
+    python tests/golden/make_golden.py [/root/reference] [--only-2d]
 
 What the vectors pin that nothing else does: the bit-level behaviour of the
 torch path at its cast points (bf16 K.K^T / pow rounding, bf16 ``denom``), the
@@ -56,6 +56,29 @@ def run_case(ref, name, b, h, r, l, d, c, dtype, seed):
     print("wrote", name, {k: v.shape for k, v in data.items() if k in ("out", "denom", "dkc")})
 
 
+def run_case_2d(ref, name, b, h, r, l, d, c, qc, dtype, seed):
+    """UniversalAttention2 (reference universal_attention_autograd.py:102-276) with query chunks of qc != c positions:
+    forward and the five gradients of its own hand-written backward under an arbitrary upstream gradient."""
+    inp = make_inputs(b, h, r, l, d, c, dtype=dtype, seed=seed)
+    n = l // c
+    g = torch.Generator().manual_seed(seed + 9)
+    g_out = torch.randn(b, h, r, l, d, n, generator=g).to(dtype)
+    g_denom = torch.randn(b, h, r, l, n, generator=g)
+    xq2 = inp["xq"].view(b, h, r, l // qc, qc, d)
+    sd2 = inp["static_dest"].view(b, h, l // qc, qc)
+    leaves = [x.clone().requires_grad_() for x in (inp["kc"], inp["vc"], xq2, inp["static_src"], sd2)]
+    out, denom = ref.UniversalAttention2.apply(*leaves)
+    grads = torch.autograd.grad([out, denom], leaves, [g_out, g_denom.to(denom.dtype)])
+    data = {k: f32(v) for k, v in inp.items()}
+    data.update(g_out=f32(g_out), g_denom=f32(g_denom), out=f32(out), denom=f32(denom))
+    for nm, gr in zip(("dkc", "dvc", "dxq", "dsrc", "ddest"), grads):
+        data[nm] = f32(gr)
+    data["meta"] = np.array([b, h, r, l, d, c, seed, 1 if dtype == torch.bfloat16 else 0])
+    data["qc"] = np.array([qc])
+    np.savez_compressed(os.path.join(HERE, name + ".npz"), **data)
+    print("wrote", name, {k: v.shape for k, v in data.items() if k in ("out", "denom", "dxq", "ddest")})
+
+
 def run_cfg0(ref):
     """BASELINE config 0 at full size, forward only, fp32; inputs are regenerated
     from the seed by the test (a checksum guards the regeneration)."""
@@ -72,10 +95,17 @@ def run_cfg0(ref):
 
 
 def main():
-    ref_root = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
+    args = [a for a in sys.argv[1:] if not a.startswith("--")]
+    ref_root = args[0] if args else "/root/reference"
     sys.path.insert(0, ref_root)
     import universal_attention_autograd as ref
     torch.manual_seed(0)
+    if "--only-2d" in sys.argv:      # adds the 2-D fixtures without rewriting the others
+        run_case_2d(ref, "tiny2d_fp32", 1, 2, 2, 64, 16, 16, 32, torch.float32, 13)
+        run_case_2d(ref, "tiny2d_bf16", 1, 2, 2, 64, 16, 16, 32, torch.bfloat16, 13)
+        return
+    run_case_2d(ref, "tiny2d_fp32", 1, 2, 2, 64, 16, 16, 32, torch.float32, 13)
+    run_case_2d(ref, "tiny2d_bf16", 1, 2, 2, 64, 16, 16, 32, torch.bfloat16, 13)
     run_case(ref, "tiny_fp32", 1, 2, 2, 64, 16, 16, torch.float32, 11)
     run_case(ref, "tiny_bf16", 1, 2, 2, 64, 16, 16, torch.bfloat16, 11)
     run_case(ref, "small_fp32", 1, 1, 1, 128, 32, 32, torch.float32, 12)

@@ -144,3 +144,51 @@ def test_tune_table_persists_through_json(tmp_path):
     assert lib.ua_tune_get(ctypes.byref(d2), _lib.UA_TUNE_BWD_QUERIES) == 1
     lib.ua_tune_set(ctypes.byref(d1), _lib.UA_TUNE_FWD_TILES, -1)
     lib.ua_tune_set(ctypes.byref(d2), _lib.UA_TUNE_BWD_QUERIES, -1)
+
+
+def test_forward_state_plus_backward_scratch_is_the_whole_workspace():
+    """Sizing rule of the split workspace: what a backward needs next to the forward state is the total minus the state."""
+    lib = _lib.load()
+    for d in (_lib.UaDesc(1, 32, 1, 8192, 128, 128, _lib.UA_BF16, 0), _lib.UaDesc(2, 3, 2, 300, 48, 0, _lib.UA_F32, 0),
+              _lib.UaDesc(1, 8, 4, 4096, 128, 128, _lib.UA_BF16, _lib.UA_FLAG_RECOMPUTE)):
+        for fwd, bwd, scratch in ((_lib.UA_OP_FUSED_FWD, _lib.UA_OP_FUSED_BWD, _lib.UA_OP_FUSED_BWD_SCRATCH),
+                                  (_lib.UA_OP_FWD, _lib.UA_OP_BWD, _lib.UA_OP_BWD_SCRATCH)):
+            if d.chunk == 0 and fwd == _lib.UA_OP_FWD:
+                continue
+            f, t, s = (lib.ua_workspace_bytes(ctypes.byref(d), op) for op in (fwd, bwd, scratch))
+            assert f > 0 and s > 0 and f + s == t and f % 256 == 0
+    big = _lib.UaDesc(1, 32, 1, 8192, 128, 128, _lib.UA_BF16, 0)
+    assert lib.ua_workspace_bytes(ctypes.byref(big), _lib.UA_OP_FUSED_FWD) <= int(2.6e9)       # kept between forward and backward
+    assert lib.ua_workspace_bytes(ctypes.byref(big), _lib.UA_OP_FUSED_BWD_SCRATCH) >= int(4e9)  # allocated inside backward
+
+
+def test_mismatched_shapes_and_dtypes_are_refused_before_any_launch():
+    """The kernels trust the descriptor, so the host checks the five tensors against one another (the reference fails in
+    its own views / asserts on such inputs); runs on CPU tensors because the checks come before the device check."""
+    import torch
+    from universal_attention_triton_amd import ops
+    b, h, n, c, d, r = 1, 2, 4, 16, 32, 2
+    L = n * c
+    kc, vc = torch.zeros(b, h, n, c, d), torch.zeros(b, h, n, c, d)
+    xq, src, dest = torch.zeros(b, h, r, L, d), torch.ones(b, h, n, c), torch.ones(b, h, L)
+    bad = [
+        (kc, vc[:, :, :2], xq, src, dest),                         # vc shorter than kc
+        (kc, vc, xq[:, :, :, : L // 2], src, dest),                # xq shorter than the keys
+        (kc, vc, torch.zeros(b, h + 1, r, L, d), src, dest),       # other head count
+        (kc, vc, torch.zeros(b, h, r, L, d + 8), src, dest),       # other head dim
+        (kc, vc, xq, src[:, :, :2], dest),                         # gates of another length
+        (kc, vc, xq, src, dest[:, :, : L - 1]),
+        (kc, vc, torch.zeros(b, h, r, n, c // 2, d), src, dest),   # 2-D layout that does not cover L
+        (kc[0], vc[0], xq[0], src[0], dest[0]),                    # wrong rank
+    ]
+    for args in bad:
+        with pytest.raises(ValueError):
+            ops.fused_forward(*args)
+        with pytest.raises(ValueError):
+            ops.chunked_forward(*args)
+    with pytest.raises(TypeError):
+        ops.fused_forward(kc, vc.bfloat16(), xq, src, dest)
+    with pytest.raises(TypeError):
+        ops.fused_forward(kc.half(), vc.half(), xq.half(), src, dest)
+    with pytest.raises(_lib.UaError):                                  # well-formed, but not on the GPU
+        ops.fused_forward(kc, vc, xq, src, dest)

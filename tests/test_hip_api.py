@@ -1,7 +1,11 @@
 """Drop-in interface on the GPU: the reference's module paths, class names, shapes, error behaviour and
 autograd wiring, the fused entry points, the tune table, and edge cases of the inputs."""
+import ctypes
+
 import pytest
 import torch
+
+from universal_attention_triton_amd import _lib
 
 from oracle import ua_oracle as orc
 from tests.util import NAMES, TOL, dense_reference, load_golden, rel_err
@@ -129,9 +133,9 @@ def test_recomputing_and_tile_exchanging_bf16_kernels_agree(shape, prune):
     a = [dev[k] for k in NAMES]
     res = {}
     for rec in (False, True):
-        O, lse, ws = ops.fused_forward(*a, for_backward=True, prune=prune, recompute=rec)
-        grads = ops.fused_backward(*a, O, lse, dev["dO"], ws=ws, prune=prune, recompute=rec)
-        g2 = ops.fused_backward(*a, O, lse, dev["dO"], ws=None, prune=prune, recompute=rec)     # without the forward's state
+        O, lse, ws = ops.fused_forward(*a, keep_state=True, prune=prune, recompute=rec)
+        grads = ops.fused_backward(*a, O, lse, dev["dO"], state=ws, prune=prune, recompute=rec)
+        g2 = ops.fused_backward(*a, O, lse, dev["dO"], state=None, prune=prune, recompute=rec)     # without the forward's state
         torch.cuda.synchronize()
         res[rec] = (O, lse) + tuple(grads)
         for x, y in zip(grads, g2):
@@ -164,14 +168,15 @@ def test_grouped_queries_shared_and_separate_key_sweeps_agree(shape, prune):
     a = [dev[k] for k in NAMES]
     res = {}
     for share in (False, True):
-        O, lse, ws = ops.fused_forward(*a, for_backward=True, prune=prune, share_groups=share)
-        grads = ops.fused_backward(*a, O, lse, dev["dO"], ws=ws, prune=prune, share_groups=share)
-        g2 = ops.fused_backward(*a, O, lse, dev["dO"], ws=None, prune=prune, share_groups=share)
+        O, lse, ws = ops.fused_forward(*a, keep_state=True, prune=prune, share_groups=share)
+        grads = ops.fused_backward(*a, O, lse, dev["dO"], state=ws, prune=prune, share_groups=share)
+        g2 = ops.fused_backward(*a, O, lse, dev["dO"], state=None, prune=prune, share_groups=share)
         torch.cuda.synchronize()
         res[share] = (O, lse) + tuple(grads)
         for x, y in zip(grads, g2):
             assert rel_err(y, x) <= 1e-3
-        res[share, "bytes"] = ws.numel()
+        desc = ops._desc(a[0], a[2], False, _lib.UA_FLAG_SHARE_GROUPS if share else 0)
+        res[share, "bytes"] = _lib.load().ua_workspace_bytes(ctypes.byref(desc), _lib.UA_OP_FUSED_BWD_SCRATCH)
     assert res[True, "bytes"] < res[False, "bytes"]       # separate sweeps keep the key-side sums per query head
     assert torch.equal(res[False][0], res[True][0]) and torch.equal(res[False][1], res[True][1])
     O_ref, lse_ref, g_ref = dense_reference(inp)
@@ -215,8 +220,8 @@ def test_edge_cases_of_the_inputs(case, dtype):
     O_ref, lse_ref, g_ref = dense_reference(inp)
     dev = {k: v.cuda() for k, v in inp.items()}
     a = [dev[k] for k in NAMES]
-    O, lse, ws = ops.fused_forward(*a, for_backward=True)
-    grads = ops.fused_backward(*a, O, lse, dev["dO"], ws=ws)
+    O, lse, ws = ops.fused_forward(*a, keep_state=True)
+    grads = ops.fused_backward(*a, O, lse, dev["dO"], state=ws)
     torch.cuda.synchronize()
     tol = TOL[dtype]
     assert torch.isfinite(O.float()).all() and all(torch.isfinite(g.float()).all() for g in grads)
@@ -247,8 +252,8 @@ def test_zero_upstream_gradient_gives_zero_gradients():
     from universal_attention_triton_amd import ops
     inp = orc.make_inputs(1, 2, 1, 256, 64, 64, dtype=torch.bfloat16, seed=71)
     a = [inp[k].cuda() for k in NAMES]
-    O, lse, ws = ops.fused_forward(*a, for_backward=True)
-    grads = ops.fused_backward(*a, O, lse, torch.zeros_like(O), ws=ws)
+    O, lse, ws = ops.fused_forward(*a, keep_state=True)
+    grads = ops.fused_backward(*a, O, lse, torch.zeros_like(O), state=ws)
     for g in grads:
         assert float(g.float().abs().max()) == 0.0
 
@@ -276,12 +281,12 @@ def test_pruning_of_negligible_pairs_changes_nothing(case, dtype):
     a = [dev[k] for k in NAMES]
     res = {}
     for prune in (False, True):
-        O, lse, ws = ops.fused_forward(*a, for_backward=True, prune=prune)
-        grads = ops.fused_backward(*a, O, lse, dev["dO"], ws=ws)
+        O, lse, ws = ops.fused_forward(*a, keep_state=True, prune=prune)
+        grads = ops.fused_backward(*a, O, lse, dev["dO"], state=ws)
         torch.cuda.synchronize()
         res[prune] = (O, lse) + tuple(grads)
     # the backward alone (no forward state) with the flag
-    g2 = ops.fused_backward(*a, res[True][0], res[True][1], dev["dO"], ws=None, prune=True)
+    g2 = ops.fused_backward(*a, res[True][0], res[True][1], dev["dO"], state=None, prune=True)
     torch.cuda.synchronize()
     tight = 1e-6 if dtype == torch.float32 else 1e-3
     for name, x, y, y2 in zip(("O", "lse", "dk", "dv", "dq", "dsrc", "ddest"), res[False], res[True], (None, None) + tuple(g2)):
@@ -340,8 +345,8 @@ def test_entry_points_can_be_captured_in_a_hip_graph():
     a = [static[k] for k in NAMES]
 
     def step():
-        O, lse, ws = ops.fused_forward(*a, for_backward=True)
-        return (O, lse) + tuple(ops.fused_backward(*a, O, lse, static["dO"], ws=ws))
+        O, lse, ws = ops.fused_forward(*a, keep_state=True)
+        return (O, lse) + tuple(ops.fused_backward(*a, O, lse, static["dO"], state=ws))
 
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())

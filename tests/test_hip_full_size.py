@@ -36,10 +36,10 @@ def _oracle_head(inp, z, with_backward, dtype=torch.float32):
 def _run_fused(dev, backward=True, scale=1.0, prune=False):
     from universal_attention_triton_amd import ops
     a = [dev[k] for k in NAMES]
-    O, lse, ws = ops.fused_forward(*a, for_backward=backward, prune=prune)
+    O, lse, ws = ops.fused_forward(*a, keep_state=backward, prune=prune)
     if not backward:
         return O, lse, None
-    grads = ops.fused_backward(*a, O, lse, dev["dO"] * scale if scale != 1.0 else dev["dO"], ws=ws, prune=prune)
+    grads = ops.fused_backward(*a, O, lse, dev["dO"] * scale if scale != 1.0 else dev["dO"], state=ws, prune=prune)
     torch.cuda.synchronize()
     return O, lse, grads
 
@@ -156,6 +156,12 @@ def test_config4_long_context_h8_L32768_d128_gates_near_one():
     ref_O, ref_grads = _oracle_head(cpu_short, z, True)
     _, _, gshort = _run_fused(short)
     _check_head(Os, gshort, ref_O, ref_grads, z, TOL[BF16])
-    print("case cfg4 oracle full-length head, forward", flush=True)
-    ref_O, _ = _oracle_head(inp, z, False)
-    _check_head(O, None, ref_O, None, z, TOL[BF16])
+    # ... and of the whole sequence, forward and all five gradients (the merged result and its gradients do not
+    # depend on the chunk size, so the oracle runs with chunks of 1024 keys to keep its per-chunk tensors small)
+    print("case cfg4 oracle full-length head, forward + backward", flush=True)
+    wide = dict(inp)
+    for k in ("kc", "vc"):
+        wide[k] = inp[k].reshape(1, 8, L // 1024, 1024, 128)
+    wide["static_src"] = inp["static_src"].reshape(1, 8, L // 1024, 1024)
+    ref_O, ref_grads = _oracle_head(wide, z, True)
+    _check_head(O, grads, ref_O, ref_grads, z, TOL[BF16])

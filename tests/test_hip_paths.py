@@ -1,0 +1,185 @@
+"""Paths of the drop-in that share kernels with the main ones but have host code of their own: backward through the
+2-D layout (reference UniversalAttention2.backward, universal_attention_autograd.py:172-276, and the Triton-side entry,
+Universal_Attention/universal_attention.py:34-46) with query chunks that differ from the key chunks; all five gradients
+through the (q, k, v) calling convention (universal_attention_kernel_opt.py:504-581); gates in another dtype than
+q, k, v (universal_attention_kernel.py:825-829); well-conditioned float32 keys held to the plain 1e-4; what stays
+allocated between forward and backward."""
+import pytest
+import torch
+
+from oracle import ua_oracle as orc
+from tests.util import NAMES, TOL, dense_reference, load_golden, rel_err
+
+pytestmark = pytest.mark.gpu
+GRADS = ("dkc", "dvc", "dxq", "dsrc", "ddest")
+
+
+def _table(tag, got, want, tol):
+    errs = {n: rel_err(g.reshape(w.shape), w) for n, g, w in zip(GRADS, got, want)}
+    print(tag, {k: "%.2e" % v for k, v in errs.items()}, flush=True)
+    bad = {k: v for k, v in errs.items() if not v <= tol}
+    assert not bad, (tag, bad)
+
+
+@pytest.mark.parametrize("entry", ["autograd2", "triton_side"])
+@pytest.mark.parametrize("name", ["tiny2d_fp32", "tiny2d_bf16"])
+def test_backward_through_the_2d_layout_matches_reference_golden(name, entry):
+    """Key chunks of 16, query chunks of 32, arbitrary (g_out, g_denom): the reference's UniversalAttention2 wrote these."""
+    import numpy as np
+    import os
+    from universal_attention_triton_amd import universal_attention_autograd as ua
+    from universal_attention_triton_amd.universal_attention import UniversalAttention as TritonSide
+    t, dtype, (b, h, r, l, d, c, seed) = load_golden(name)
+    qc = int(np.load(os.path.join(os.path.dirname(__file__), "golden", name + ".npz"))["qc"][0])
+    tol = TOL[dtype] if dtype == torch.float32 else 2.5e-2     # bf16: the golden carries the reference's own bf16 noise
+    fn = ua.UniversalAttention2 if entry == "autograd2" else TritonSide
+    xq2 = t["xq"].to(dtype).view(b, h, r, l // qc, qc, d)
+    sd2 = t["static_dest"].to(dtype).view(b, h, l // qc, qc)
+    leaves = [x.cuda().requires_grad_() for x in (t["kc"].to(dtype), t["vc"].to(dtype), xq2, t["static_src"].to(dtype), sd2)]
+    out, denom = fn.apply(*leaves)
+    assert out.shape == (b, h, r, l, d, l // c) and denom.shape == (b, h, r, l, l // c)
+    grads = torch.autograd.grad([out, denom], leaves, [t["g_out"].to(dtype).cuda(), t["g_denom"].to(dtype).cuda()])
+    torch.cuda.synchronize()
+    assert grads[2].shape == xq2.shape and grads[4].shape == sd2.shape
+    assert rel_err(out, t["out"]) <= tol
+    _table("2-D layout %s %s" % (name, entry), grads, [t[n] for n in GRADS], tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_backward_through_the_2d_layout_matches_oracle_larger_case(dtype):
+    """Chunk 64 keys x 32 queries, L = 256, arbitrary upstream: against the oracle's restatement of the 1-D backward."""
+    from universal_attention_triton_amd import universal_attention_autograd as ua
+    b, h, r, L, d, c, qc = 1, 2, 2, 256, 64, 64, 32
+    inp = orc.make_inputs(b, h, r, L, d, c, dtype=dtype, seed=71)
+    g = torch.Generator().manual_seed(9)
+    g_out = torch.randn(b, h, r, L, d, L // c, generator=g).to(dtype)
+    g_denom = torch.randn(b, h, r, L, L // c, generator=g).to(dtype)
+    want = orc.chunked_backward(*[inp[k].float() for k in NAMES], g_out.float(), g_denom.float())
+    xq2 = inp["xq"].view(b, h, r, L // qc, qc, d)
+    sd2 = inp["static_dest"].view(b, h, L // qc, qc)
+    leaves = [x.cuda().requires_grad_() for x in (inp["kc"], inp["vc"], xq2, inp["static_src"], sd2)]
+    out, denom = ua.UniversalAttention2.apply(*leaves)
+    grads = torch.autograd.grad([out, denom], leaves, [g_out.cuda(), g_denom.cuda()])
+    torch.cuda.synchronize()
+    _table("2-D layout oracle %s" % dtype, grads, want, 4e-4 if dtype == torch.float32 else TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_all_five_gradients_through_the_qkv_calling_convention(dtype):
+    """attention(q, k, v, ...): r-major grouped queries (query head j uses kv head j % H_kv), head dim 80, ragged L;
+    forward and backward against float64 autograd of the dense oracle; ac=True (keep no state) gives the same."""
+    from universal_attention_triton_amd.universal_attention import attention
+    B, Hkv, r, L, d = 1, 2, 3, 200, 80
+    inp = orc.make_inputs(B, Hkv, r, L, d, 8, dtype=dtype, seed=43)
+    O_ref, _, g_ref = dense_reference(inp)
+    k = inp["kc"].reshape(B, Hkv, L, d).cuda().requires_grad_()
+    v = inp["vc"].reshape(B, Hkv, L, d).cuda().requires_grad_()
+    q = inp["xq"].transpose(1, 2).reshape(B, r * Hkv, L, d).cuda().requires_grad_()       # head j = rep * Hkv + kv
+    src = inp["static_src"].reshape(B, Hkv, L).cuda().requires_grad_()
+    dest = inp["static_dest"].cuda().requires_grad_()
+    dO = inp["dO"].transpose(1, 2).reshape(B, r * Hkv, L, d).cuda()
+    results = []
+    for ac in (False, True):
+        o = attention(q, k, v, True, 0.5, src, dest, ac=ac)
+        gq, gk, gv, gs, gd = torch.autograd.grad(o, [q, k, v, src, dest], dO)
+        torch.cuda.synchronize()
+        assert rel_err(o.view(B, r, Hkv, L, d).transpose(1, 2), O_ref) <= TOL[dtype]
+        got = [gk, gv, gq.view(B, r, Hkv, L, d).transpose(1, 2), gs, gd]
+        _table("attention() %s ac=%s" % (dtype, ac), got, g_ref, 4e-4 if dtype == torch.float32 else TOL[dtype])
+        results.append(got)
+    for a_, b_ in zip(*results):
+        assert rel_err(a_, b_) <= (1e-5 if dtype == torch.float32 else 2e-3)
+
+
+def test_fp32_key_gradient_meets_1e4_on_well_conditioned_keys():
+    """d/dG relu(G)^(2/3) is singular at G -> 0+, which is why the other float32 tests give dkc a wider bar.  With keys in
+    the positive orthant every product k_s.k_u is well above 1e-3 and every tensor, dkc included, meets the plain 1e-4,
+    through the fused and the chunked operator."""
+    from universal_attention_triton_amd import universal_attention_autograd as ua
+    from universal_attention_triton_amd.universal_attention import universal_attention
+    b, h, r, L, d, c = 1, 2, 2, 320, 64, 64
+    inp = orc.make_inputs(b, h, r, L, d, c, dtype=torch.float32, seed=77)
+    k = inp["kc"].abs() + 0.05
+    inp["kc"] = k / k.norm(dim=-1, keepdim=True)
+    flat = inp["kc"].reshape(b, h, L, d)
+    assert float((flat @ flat.transpose(-1, -2)).min()) > 1e-3
+    O_ref, _, g_ref = dense_reference(inp)
+    leaves = [inp[k_].cuda().requires_grad_() for k_ in NAMES]
+    O = universal_attention(*leaves)
+    grads = torch.autograd.grad(O, leaves, inp["dO"].cuda())
+    torch.cuda.synchronize()
+    assert rel_err(O, O_ref) <= 1e-4
+    _table("fused fp32 positive keys", grads, g_ref, 1e-4)
+    leaves = [inp[k_].cuda().requires_grad_() for k_ in NAMES]
+    out, denom = ua.UniversalAttention.apply(*leaves)
+    O2 = ua.SMVecMatMul.apply(out, denom)
+    grads2 = torch.autograd.grad(O2, leaves, inp["dO"].cuda())
+    torch.cuda.synchronize()
+    _table("chunked fp32 positive keys", grads2, g_ref, 1e-4)
+
+
+@pytest.mark.parametrize("gates", ["fp32_both", "fp32_src_only"])
+def test_float32_gates_next_to_bf16_tensors(gates):
+    """The reference allocates dstatic_src in static_src.dtype and everything else in xq.dtype, i.e. float32 gates next to
+    bf16 q, k, v are legal.  Checked against float64 autograd of the dense oracle on the same mixed-dtype inputs (the
+    gates are NOT rounded to bf16), through the fused and the chunked operator; gradients come back in the gates' dtypes."""
+    from universal_attention_triton_amd import universal_attention_autograd as ua
+    from universal_attention_triton_amd.universal_attention import universal_attention
+    b, h, r, L, d, c = 1, 2, 2, 256, 64, 64
+    bf = torch.bfloat16
+    inp = orc.make_inputs(b, h, r, L, d, c, dtype=torch.float32, seed=81)
+    mixed = {k_: (inp[k_].to(bf) if k_ in ("kc", "vc", "xq") else inp[k_].clone()) for k_ in NAMES}
+    if gates == "fp32_src_only":
+        mixed["static_dest"] = mixed["static_dest"].to(bf)
+    mixed["dO"] = inp["dO"].to(bf)
+    # gates whose bf16 rounding would be visible: the result must follow the float32 values
+    O_ref, _, g_ref = dense_reference(mixed)
+    O_rounded, _, _ = dense_reference({k_: (v.to(bf) if k_ != "dO" else v) for k_, v in mixed.items()})
+    leaves = [mixed[k_].cuda().requires_grad_() for k_ in NAMES]
+    O = universal_attention(*leaves)
+    grads = torch.autograd.grad(O, leaves, mixed["dO"].cuda())
+    torch.cuda.synchronize()
+    assert O.dtype == bf and grads[3].dtype == mixed["static_src"].dtype and grads[4].dtype == mixed["static_dest"].dtype
+    assert rel_err(O, O_ref) <= TOL[bf]
+    _table("fused mixed dtypes " + gates, grads, g_ref, TOL[bf])
+    leaves = [mixed[k_].cuda().requires_grad_() for k_ in NAMES]
+    out, denom = ua.UniversalAttention.apply(*leaves)
+    O2 = ua.SMVecMatMul.apply(out, denom)
+    grads2 = torch.autograd.grad(O2, leaves, mixed["dO"].cuda())
+    torch.cuda.synchronize()
+    assert grads2[3].dtype == mixed["static_src"].dtype
+    _table("chunked mixed dtypes " + gates, grads2, g_ref, TOL[bf])
+    if gates == "fp32_both":
+        # the float32 gates are really used: the fused result is closer to the float32-gate oracle than the
+        # oracle with rounded gates is
+        assert rel_err(O, O_ref) < rel_err(O_rounded, O_ref) or rel_err(O_rounded, O_ref) < 2e-3
+
+
+def test_memory_kept_between_forward_and_backward_at_the_headline_shape():
+    """BASELINE config 2 (b=1 h=32 L=8192 d=128 bf16): between forward and backward the fused operator holds its inputs,
+    O, lse and the forward state (packed inputs + bias tiles, <= 2.6 GB); the 4.8 GB of backward scratch only exist inside
+    backward; keep_state=False holds nothing beyond inputs, O and lse."""
+    from universal_attention_triton_amd import ops
+    from universal_attention_triton_amd.universal_attention import universal_attention
+    b, h, r, L, d = 1, 32, 1, 8192, 128
+    inp = orc.make_inputs(b, h, r, L, d, 128, dtype=torch.bfloat16, seed=1002)
+    leaves = [inp[k_].cuda().requires_grad_() for k_ in NAMES]
+    dO = inp["dO"].cuda()
+    torch.cuda.synchronize()
+    base = torch.cuda.memory_allocated()
+    out_bytes = b * h * r * L * d * 2 + b * h * r * L * 4
+    for keep, budget in ((True, int(2.6e9)), (False, 0)):
+        O = universal_attention(*leaves, keep_state=keep)
+        torch.cuda.synchronize()
+        held = torch.cuda.memory_allocated() - base
+        assert held <= out_bytes + budget + (8 << 20), (keep, held)
+        if keep:
+            assert held >= out_bytes + ops.retained_bytes(*[x.detach() for x in leaves]) - (8 << 20)
+        torch.cuda.reset_peak_memory_stats()
+        grads = torch.autograd.grad(O, leaves, dO)
+        torch.cuda.synchronize()
+        peak = torch.cuda.max_memory_allocated() - base
+        assert peak > held + int(4e9)            # the scratch lived inside backward only
+        del O, grads
+        torch.cuda.synchronize()
+        assert torch.cuda.memory_allocated() - base <= (8 << 20)

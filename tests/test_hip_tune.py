@@ -16,8 +16,8 @@ BF = torch.bfloat16
 
 
 def _step(a, dO):
-    O, lse, ws = ops.fused_forward(*a, for_backward=True)
-    g = ops.fused_backward(*a, O, lse, dO, ws=ws)
+    O, lse, ws = ops.fused_forward(*a, keep_state=True)
+    g = ops.fused_backward(*a, O, lse, dO, state=ws)
     return O, lse, g
 
 
@@ -92,12 +92,21 @@ def test_shipped_table_is_within_3_percent_of_autotune_on_this_device(cfg):
     dO = inp["dO"].cuda()
     slots = [s for s in ("carry", "fwd_tiles", "bwd_parts", "bwd_queries") if ops.tune_variants(a[0], a[2], s) > 1]
     shipped = {s: ops.tune_choice(a[0], a[2], s) for s in slots}
-    t_shipped = _median_ms(a, dO)
     tuned = ops.autotune(*a, dO=dO)
+    tuned = {s: tuned[s] for s in slots}
     try:
-        if {s: tuned[s] for s in slots} != shipped:
-            t_tuned = _median_ms(a, dO)
-            assert t_shipped <= 1.03 * t_tuned, (shipped, tuned, t_shipped, t_tuned)
+        if tuned != shipped:
+            # alternate between the two tables so that clock and temperature drift hit both alike
+            t = {"shipped": [], "tuned": []}
+            for _ in range(3):
+                for s in slots:
+                    ops.tune_set(a[0], a[2], -1, s)
+                t["shipped"].append(_median_ms(a, dO))
+                for s in slots:
+                    ops.tune_set(a[0], a[2], tuned[s], s)
+                t["tuned"].append(_median_ms(a, dO))
+            print("shipped", shipped, t["shipped"], "tuned", tuned, t["tuned"], flush=True)
+            assert min(t["shipped"]) <= 1.03 * min(t["tuned"]), (shipped, tuned, t)
     finally:
         for s in slots:
             ops.tune_set(a[0], a[2], -1, s)

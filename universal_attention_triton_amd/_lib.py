@@ -11,13 +11,14 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libua_hip.so")
 
 UA_F32, UA_BF16 = 0, 1
-UA_OP_FWD, UA_OP_BWD, UA_OP_FUSED_FWD, UA_OP_FUSED_BWD = 0, 1, 2, 3
+UA_OP_FWD, UA_OP_BWD, UA_OP_FUSED_FWD, UA_OP_FUSED_BWD, UA_OP_BWD_SCRATCH, UA_OP_FUSED_BWD_SCRATCH = 0, 1, 2, 3, 4, 5
 UA_TUNE_FWD_RECOMPUTE, UA_TUNE_CARRY, UA_TUNE_FWD_TILES, UA_TUNE_BWD_PARTS, UA_TUNE_BWD_QUERIES = 2, 16, 17, 18, 19
 TUNE_SLOTS = {"fwd_recompute": 2, "carry": 16, "fwd_tiles": 17, "bwd_parts": 18, "bwd_queries": 19}
 UA_FLAG_SKIP_MASKED = 1
 UA_FLAG_RECOMPUTE = 4
 UA_FLAG_PRUNE = 2
 UA_FLAG_SHARE_GROUPS = 8
+UA_FLAG_GATES_F32 = 16
 
 c_void_p, c_int, c_size_t, c_int64, c_int32 = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_int64, ctypes.c_int32
 
@@ -42,12 +43,12 @@ SIGNATURES = {
     "ua_workspace_bytes": (c_size_t, [P(UaDesc), c_int]),
     "ua_fwd": (c_int, [P(UaDesc), P(UaRows), P(UaRows), P(UaRows), c_void_p, c_void_p, P(UaChunked), c_void_p, c_void_p, c_size_t, c_void_p]),
     "ua_bwd": (c_int, [P(UaDesc), P(UaRows), P(UaRows), P(UaRows), c_void_p, c_void_p, P(UaChunked), P(UaChunked), c_void_p,
-                       c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
+                       c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "ua_fused_fwd": (c_int, [P(UaDesc), P(UaRows), P(UaRows), P(UaRows), c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "ua_noalloc_scratch_bytes": (c_size_t, []),
     "ua_fused_fwd_noalloc": (c_int, [P(UaDesc), P(UaRows), P(UaRows), P(UaRows), c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "ua_fused_bwd": (c_int, [P(UaDesc), P(UaRows), P(UaRows), P(UaRows), c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
+                             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "ua_merge_fwd": (c_int, [c_int, c_int64, c_int32, c_int32, c_int32, P(UaChunked), c_void_p, c_void_p, c_void_p]),
     "ua_merge_bwd": (c_int, [c_int, c_int64, c_int32, c_int32, c_int32, P(UaChunked), c_void_p, c_void_p, P(UaChunked), c_void_p, c_void_p]),
     "ua_affinity_workspace_bytes": (c_size_t, [P(UaDesc), c_int]),

@@ -282,13 +282,15 @@ __global__ void __launch_bounds__(64 * NW) k_bwd_keys(BwdArgs<T> a) {
 // Combine partial gradients into the caller's contiguous tensors:
 //   dk [Zk][L][d], dv [Zk][L][d], dq [Zq][L][d], dsrc [Zk][L], ddest [Zk][L]
 // grid (ceil(L/4), max(Zk, Zq)); one wave per row.  The fp32 partial gradients are row-major [Z][Lp][D].
-template <class T>
+// TG: dtype of the gates and of their gradients (the reference allocates dstatic_src in static_src.dtype,
+// Universal_Attention/triton/universal_attention_kernel.py:828)
+template <class T, class TG = T>
 __global__ void __launch_bounds__(256) k_bwd_finish(const float* __restrict__ dKrow, const float* __restrict__ dVrow,
                                                     const float* __restrict__ dKdacc, const float* __restrict__ dQacc,
                                                     const float* __restrict__ dsrc_raw, const T* __restrict__ Kp,
-                                                    const T* __restrict__ src, const T* __restrict__ dest,
+                                                    const TG* __restrict__ src, const TG* __restrict__ dest,
                                                     T* __restrict__ dk, T* __restrict__ dv, T* __restrict__ dq,
-                                                    T* __restrict__ dsrc, T* __restrict__ ddest, int Zk, int Zq, int L,
+                                                    TG* __restrict__ dsrc, TG* __restrict__ ddest, int Zk, int Zq, int L,
                                                     int Lp, int D, int d, int tiled, int RS, int RK) {
   const int z = blockIdx.y, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + wave;
@@ -320,10 +322,10 @@ __global__ void __launch_bounds__(256) k_bwd_finish(const float* __restrict__ dK
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) dot += __shfl_xor(dot, m, 64);
     if (lane == 0) {
-      ddest[(long)z * L + t] = cvt<T>(dot / (2.0f * sd));
+      ddest[(long)z * L + t] = cvt<TG>(dot / (2.0f * sd));
       float sr = 0.f;
       for (int r = 0; r < RK; ++r) sr += dsrc_raw[((long)z * RK + r) * Lp + t];
-      dsrc[(long)z * L + t] = cvt<T>(sr / (3.0f * (float)src[(long)z * L + t]));
+      dsrc[(long)z * L + t] = cvt<TG>(sr / (3.0f * (float)src[(long)z * L + t]));
     }
   }
 }

@@ -275,14 +275,26 @@ struct ProfScope {
     if (e_ != hipSuccess) return fail(UA_ELAUNCH, "%s: %s", #expr, hipGetErrorString(e_));   \
   } while (0)
 
-int check_common(const ua_desc* desc, bool chunked, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq,
-                 const void* src, const void* dest, void* ws, size_t ws_bytes, const Layout& l, bool bwd) {
-  (void)desc; (void)chunked;
+// Workspace conventions of the entry points.  Forward ops: `ws` holds the forward state (l.fwd_end bytes).  Backward ops:
+// `fwd_state` is null or the buffer the forward op ran on; `ws` then holds the backward scratch alone (l.total - l.fwd_end
+// bytes), else state and scratch together (l.total).  Bases: a forward-state field lives at wf + l.field, a backward
+// field at wb + l.field (wb is the scratch pointer minus l.fwd_end when the state is a separate buffer).
+int check_common(const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* src, const void* dest, void* ws,
+                 size_t ws_bytes, size_t need) {
   if (!kc || !vc || !xq || !kc->ptr || !vc->ptr || !xq->ptr || !src || !dest) return fail(UA_EINVAL, "null input tensor");
   if (!ws) return fail(UA_EWORKSPACE, "null workspace");
   if ((uintptr_t)ws % 256 != 0) return fail(UA_EWORKSPACE, "workspace must be 256-byte aligned");
-  const size_t need = bwd ? l.total : l.fwd_end;
   if (ws_bytes < need) return fail(UA_EWORKSPACE, "workspace has %zu bytes, %zu needed", ws_bytes, need);
+  return UA_OK;
+}
+int bwd_bases(const Layout& l, void* fwd_state, void* ws, char** wf, char** wb) {
+  if (fwd_state) {
+    if ((uintptr_t)fwd_state % 256 != 0) return fail(UA_EWORKSPACE, "forward state must be 256-byte aligned");
+    *wf = (char*)fwd_state;
+    *wb = (char*)ws - l.fwd_end;
+  } else {
+    *wf = *wb = (char*)ws;
+  }
   return UA_OK;
 }
 
@@ -293,65 +305,69 @@ hipError_t zero_fill(void* p, size_t bytes, hipStream_t s) {   // bytes is a mul
   return hipGetLastError();
 }
 
+// the gates (static_src, static_dest) and their gradients are float32: always with float32 tensors, with bf16 tensors
+// when the caller says so (the reference keeps dstatic_src in static_src.dtype whatever the dtype of q, k, v)
+bool gates_f32(const ua_desc& d) { return d.dtype == UA_F32 || (d.flags & UA_FLAG_GATES_F32); }
+
 // packs K, V and Q in both orientations and the log-gates
 // chunk sizes the query-stationary kernels handle (the others go through the key-chunk-stationary ones)
 bool fast_chunk(const ua_desc& d) { return d.chunk % 64 == 0; }
 
 // rowmajor: working tensors for the key-chunk-stationary (32x32 tile) kernels; otherwise the tiled layout
 int pack_inputs(const ua_desc& d, const Layout& l, bool rowmajor, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq,
-                const void* src, const void* dest, char* ws, hipStream_t s) {
+                const void* src, const void* dest, char* wf, hipStream_t s) {
   const bool chunked = rowmajor;
   UA_PROF("pack_inputs", s);
   const ua::RowsView K = rows_view(*kc, d.h, 1), V = rows_view(*vc, d.h, 1), Q = rows_view(*xq, d.h, d.r);
   // the chunked kernels work on 32x32 tiles, the fused ones on 16x16 tiles (and read V^T in natural order)
   const int mode = chunked ? TR_PERM16 : TR_PERM32;
   const bool prune = !chunked && (d.flags & UA_FLAG_PRUNE);
-  UA_HIP(pack(d.dtype, l.D, K, ws + l.Kp, ws + l.KT, d.d, d.L, l.Lp, l.Zk, mode, s, prune ? (float*)(ws + l.knorm2) : nullptr));
-  UA_HIP(pack(d.dtype, l.D, V, ws + l.Vp, ws + l.VT, d.d, d.L, l.Lp, l.Zk, chunked ? TR_PERM16 : TR_NATURAL, s));
-  UA_HIP(pack(d.dtype, l.D, Q, ws + l.Qp, l.grad_tiles ? nullptr : ws + l.QT, d.d, d.L, l.Lp, l.Zq, mode, s,
-              prune ? (float*)(ws + l.qnorm2) : nullptr));
+  UA_HIP(pack(d.dtype, l.D, K, wf + l.Kp, wf + l.KT, d.d, d.L, l.Lp, l.Zk, mode, s, prune ? (float*)(wf + l.knorm2) : nullptr));
+  UA_HIP(pack(d.dtype, l.D, V, wf + l.Vp, wf + l.VT, d.d, d.L, l.Lp, l.Zk, chunked ? TR_PERM16 : TR_NATURAL, s));
+  UA_HIP(pack(d.dtype, l.D, Q, wf + l.Qp, l.grad_tiles ? nullptr : wf + l.QT, d.d, d.L, l.Lp, l.Zq, mode, s,
+              prune ? (float*)(wf + l.qnorm2) : nullptr));
   const dim3 grid((l.Lp + 255) / 256, l.Zk);
-  if (d.dtype == UA_BF16)
+  if (!gates_f32(d))
     hipLaunchKernelGGL((ua::k_gates<ua::bf16>), grid, dim3(256), 0, s, (const ua::bf16*)src, (const ua::bf16*)dest,
-                       (float*)(ws + l.lsrc), (float*)(ws + l.ldest), d.L, l.Lp);
+                       (float*)(wf + l.lsrc), (float*)(wf + l.ldest), d.L, l.Lp);
   else
     hipLaunchKernelGGL((ua::k_gates<float>), grid, dim3(256), 0, s, (const float*)src, (const float*)dest,
-                       (float*)(ws + l.lsrc), (float*)(ws + l.ldest), d.L, l.Lp);
+                       (float*)(wf + l.lsrc), (float*)(wf + l.ldest), d.L, l.Lp);
   UA_HIP(hipGetLastError());
   return UA_OK;
 }
 
-int launch_carry_for(const ua_desc& d, const Layout& l, char* ws, int variant, hipStream_t s) {
-  UA_HIP(ua::launch_carry(d.dtype, l.D, ws + l.Kp, (const float*)(ws + l.lsrc), (const float*)(ws + l.ldest),
-                          (float*)(ws + l.C), l.Lp, l.Zk, 1, (d.flags & UA_FLAG_PRUNE) ? (const float*)(ws + l.knorm2) : nullptr,
-                          (const float*)(ws + l.qnorm2), d.r, (int*)(ws + l.reach), (int*)(ws + l.minkey), s,
-                          l.tiles ? ws + l.Bt : nullptr, variant));
+int launch_carry_for(const ua_desc& d, const Layout& l, char* wf, int variant, hipStream_t s) {
+  UA_HIP(ua::launch_carry(d.dtype, l.D, wf + l.Kp, (const float*)(wf + l.lsrc), (const float*)(wf + l.ldest),
+                          (float*)(wf + l.C), l.Lp, l.Zk, 1, (d.flags & UA_FLAG_PRUNE) ? (const float*)(wf + l.knorm2) : nullptr,
+                          (const float*)(wf + l.qnorm2), d.r, (int*)(wf + l.reach), (int*)(wf + l.minkey), s,
+                          l.tiles ? wf + l.Bt : nullptr, variant));
   return UA_OK;
 }
-int launch_fwd_for(const ua_desc& d, const Layout& l, char* ws, void* O, float* lse, int variant, hipStream_t s) {
-  UA_HIP(ua::launch_fwd_fused(d.dtype, l.D, variant, ws + l.Qp, ws + l.Kp, ws + l.VT, (const float*)(ws + l.lsrc),
-                              (const float*)(ws + l.ldest), (const float*)(ws + l.C), O, lse, (float*)(ws + l.lse2),
-                              (const int*)(ws + l.reach), (const int*)(ws + l.minkey), d.r, d.L, l.Lp, d.d, l.Zq, s,
-                              l.tiles ? ws + l.Bt : nullptr));
+int launch_fwd_for(const ua_desc& d, const Layout& l, char* wf, void* O, float* lse, int variant, hipStream_t s) {
+  UA_HIP(ua::launch_fwd_fused(d.dtype, l.D, variant, wf + l.Qp, wf + l.Kp, wf + l.VT, (const float*)(wf + l.lsrc),
+                              (const float*)(wf + l.ldest), (const float*)(wf + l.C), O, lse, (float*)(wf + l.lse2),
+                              (const int*)(wf + l.reach), (const int*)(wf + l.minkey), d.r, d.L, l.Lp, d.d, l.Zq, s,
+                              l.tiles ? wf + l.Bt : nullptr));
   return UA_OK;
 }
-int run_fused_fwd_kernels(const ua_desc& d, const Layout& l, char* ws, void* O, float* lse, hipStream_t s) {
+int run_fused_fwd_kernels(const ua_desc& d, const Layout& l, char* wf, void* O, float* lse, hipStream_t s) {
   {
     UA_PROF("k_carry", s);
-    if (int e = launch_carry_for(d, l, ws, l.tiles ? tuned_variant(d, UA_TUNE_CARRY) : 0, s)) return e;
+    if (int e = launch_carry_for(d, l, wf, l.tiles ? tuned_variant(d, UA_TUNE_CARRY) : 0, s)) return e;
   }
   UA_PROF("k_fwd_fused", s);
-  return launch_fwd_for(d, l, ws, O, lse, tuned_variant(d, l.tiles ? UA_TUNE_FWD_TILES : UA_TUNE_FWD_RECOMPUTE), s);
+  return launch_fwd_for(d, l, wf, O, lse, tuned_variant(d, l.tiles ? UA_TUNE_FWD_TILES : UA_TUNE_FWD_RECOMPUTE), s);
 }
 
-template <class T>
-hipError_t finish_t(const Layout& l, const ua_desc& d, char* ws, bool chunked, const void* src, const void* dest, void* dk,
+template <class T, class TG>
+hipError_t finish_t(const Layout& l, const ua_desc& d, char* wf, char* wb, bool chunked, const void* src, const void* dest, void* dk,
                     void* dv, void* dq, void* dsrc, void* ddest, hipStream_t s) {
   const int Z = l.Zq > l.Zk ? l.Zq : l.Zk;
-  hipLaunchKernelGGL((ua::k_bwd_finish<T>), dim3((d.L + 3) / 4, Z), dim3(256), 0, s, (const float*)(ws + l.dKrow),
-                     (const float*)(ws + l.dVrow), (const float*)(ws + l.dKdacc), chunked ? (const float*)(ws + l.dQacc) : nullptr,
-                     (const float*)(ws + l.dsrc_raw), (const T*)(ws + l.Kp), (const T*)src, (const T*)dest, (T*)dk, (T*)dv,
-                     (T*)dq, (T*)dsrc, (T*)ddest, l.Zk, l.Zq, d.L, l.Lp, l.D, d.d, chunked ? 0 : 1, chunked ? 1 : d.r,
+  hipLaunchKernelGGL((ua::k_bwd_finish<T, TG>), dim3((d.L + 3) / 4, Z), dim3(256), 0, s, (const float*)(wb + l.dKrow),
+                     (const float*)(wb + l.dVrow), (const float*)(wb + l.dKdacc), chunked ? (const float*)(wb + l.dQacc) : nullptr,
+                     (const float*)(wb + l.dsrc_raw), (const T*)(wf + l.Kp), (const TG*)src, (const TG*)dest, (T*)dk, (T*)dv,
+                     (T*)dq, (TG*)dsrc, (TG*)ddest, l.Zk, l.Zq, d.L, l.Lp, l.D, d.d, chunked ? 0 : 1, chunked ? 1 : d.r,
                      l.key_parts);
   return hipGetLastError();
 }
@@ -366,31 +382,31 @@ hipError_t delta_t(const ua::RowsView& O, const ua::RowsView& dO, const ua::Rows
 
 // chunked with a chunk that is not a multiple of 64: key-chunk-stationary kernel over row-major working tensors (atomics);
 // otherwise the key-stationary and query-stationary kernels over tiled working tensors
-int run_bwd_common(const ua_desc& d, const Layout& l, char* ws, bool chunked, const void* src, const void* dest, void* dkc,
+int run_bwd_common(const ua_desc& d, const Layout& l, char* wf, char* wb, bool chunked, const void* src, const void* dest, void* dkc,
                    void* dvc, void* dxq, void* dsrc, void* ddest, hipStream_t s) {
   const bool is_chunked = chunked;
   chunked = is_chunked && !fast_chunk(d);      // from here on: the atomics path
   if (chunked) {
     UA_PROF("k_zero", s);
-    UA_HIP(zero_fill(ws + l.dQacc, (size_t)l.Zq * l.Lp * l.D * 4, s));
-    UA_HIP(zero_fill(ws + l.dKdacc, (size_t)l.Zk * l.Lp * l.D * 4, s));
+    UA_HIP(zero_fill(wb + l.dQacc, (size_t)l.Zq * l.Lp * l.D * 4, s));
+    UA_HIP(zero_fill(wb + l.dKdacc, (size_t)l.Zk * l.Lp * l.D * 4, s));
   }
   ua::BwdArgsV a{};
-  a.Kp = ws + l.Kp; a.Vp = ws + l.Vp; a.KT = ws + l.KT; a.Qp = ws + l.Qp; a.QT = l.grad_tiles ? nullptr : ws + l.QT; a.dOp = ws + l.dOp;
-  a.dOT = l.grad_tiles ? nullptr : ws + l.dOT; a.lsrc = (const float*)(ws + l.lsrc); a.ldest = (const float*)(ws + l.ldest);
-  a.lse2 = (const float*)(ws + l.lse2); a.delta = (const float*)(ws + l.delta); a.C = (const float*)(ws + l.C);
-  a.reach = (const int*)(ws + l.reach); a.minkey = (const int*)(ws + l.minkey);
-  a.dQacc = (float*)(ws + l.dQacc); a.dKdacc = (float*)(ws + l.dKdacc); a.Dsuf = (float*)(ws + l.Dsuf);
-  a.dKrow = (float*)(ws + l.dKrow);
-  a.dVrow = (float*)(ws + l.dVrow); a.dsrc_raw = (float*)(ws + l.dsrc_raw);
-  a.masked_nz = (const int*)(ws + l.masked_nz);
-  a.dS_st = l.grad_tiles ? ws + l.dS_st : nullptr; a.dG_st = l.grad_tiles ? ws + l.dG_st : nullptr; a.Bt = l.tiles ? ws + l.Bt : nullptr;
+  a.Kp = wf + l.Kp; a.Vp = wf + l.Vp; a.KT = wf + l.KT; a.Qp = wf + l.Qp; a.QT = l.grad_tiles ? nullptr : wf + l.QT; a.dOp = wb + l.dOp;
+  a.dOT = l.grad_tiles ? nullptr : wb + l.dOT; a.lsrc = (const float*)(wf + l.lsrc); a.ldest = (const float*)(wf + l.ldest);
+  a.lse2 = (const float*)(wf + l.lse2); a.delta = (const float*)(wb + l.delta); a.C = (const float*)(wf + l.C);
+  a.reach = (const int*)(wf + l.reach); a.minkey = (const int*)(wf + l.minkey);
+  a.dQacc = (float*)(wb + l.dQacc); a.dKdacc = (float*)(wb + l.dKdacc); a.Dsuf = (float*)(wb + l.Dsuf);
+  a.dKrow = (float*)(wb + l.dKrow);
+  a.dVrow = (float*)(wb + l.dVrow); a.dsrc_raw = (float*)(wb + l.dsrc_raw);
+  a.masked_nz = (const int*)(wb + l.masked_nz);
+  a.dS_st = l.grad_tiles ? wb + l.dS_st : nullptr; a.dG_st = l.grad_tiles ? wb + l.dG_st : nullptr; a.Bt = l.tiles ? wf + l.Bt : nullptr;
   a.R = d.r; a.L = d.L; a.Lp = l.Lp; a.c = is_chunked ? d.chunk : 128; a.nch = l.nch; a.chunked = is_chunked ? 1 : 0;
   a.skip_masked = (d.flags & UA_FLAG_SKIP_MASKED) ? 1 : 0;
   a.split_r = (!chunked && d.r > 1) ? 1 : 0;
   a.key_parts = l.key_parts;
   // merged bf16 operator with one query group: the two kernels write the caller's gradients themselves
-  const bool direct = l.tiles && d.r == 1;
+  const bool direct = l.tiles && d.r == 1 && !gates_f32(d);
   a.direct = direct ? 1 : 0; a.d_out = d.d; a.dk_out = dkc; a.dv_out = dvc; a.dsrc_out = dsrc; a.ddest_out = ddest;
   a.src_in = src; a.dest_in = dest;
   {
@@ -405,8 +421,9 @@ int run_bwd_common(const ua_desc& d, const Layout& l, char* ws, bool chunked, co
   }
   if (direct) return UA_OK;
   UA_PROF("k_bwd_finish", s);
-  if (d.dtype == UA_BF16) UA_HIP(finish_t<ua::bf16>(l, d, ws, chunked, src, dest, dkc, dvc, dxq, dsrc, ddest, s));
-  else UA_HIP(finish_t<float>(l, d, ws, chunked, src, dest, dkc, dvc, dxq, dsrc, ddest, s));
+  if (d.dtype == UA_BF16 && gates_f32(d)) UA_HIP((finish_t<ua::bf16, float>(l, d, wf, wb, chunked, src, dest, dkc, dvc, dxq, dsrc, ddest, s)));
+  else if (d.dtype == UA_BF16) UA_HIP((finish_t<ua::bf16, ua::bf16>(l, d, wf, wb, chunked, src, dest, dkc, dvc, dxq, dsrc, ddest, s)));
+  else UA_HIP((finish_t<float, float>(l, d, wf, wb, chunked, src, dest, dkc, dvc, dxq, dsrc, ddest, s)));
   return UA_OK;
 }
 
@@ -457,23 +474,25 @@ int ua_version(void) { return 1; }
 const char* ua_last_error(void) { return g_err; }
 
 size_t ua_workspace_bytes(const ua_desc* desc, int op) {
-  const bool chunked = (op == UA_OP_FWD || op == UA_OP_BWD);
-  if (op < UA_OP_FWD || op > UA_OP_FUSED_BWD) { fail(UA_EINVAL, "unknown op %d", op); return 0; }
+  if (op < UA_OP_FWD || op > UA_OP_FUSED_BWD_SCRATCH) { fail(UA_EINVAL, "unknown op %d", op); return 0; }
+  const bool chunked = (op == UA_OP_FWD || op == UA_OP_BWD || op == UA_OP_BWD_SCRATCH);
   if (check_desc(desc, chunked) != UA_OK) return 0;
   const Layout l = make_layout(*desc, chunked);
-  return (op == UA_OP_FWD || op == UA_OP_FUSED_FWD) ? l.fwd_end : l.total;
+  if (op == UA_OP_FWD || op == UA_OP_FUSED_FWD) return l.fwd_end;
+  if (op == UA_OP_BWD_SCRATCH || op == UA_OP_FUSED_BWD_SCRATCH) return l.total - l.fwd_end;
+  return l.total;
 }
 
 int ua_fused_fwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
                  const void* static_dest, void* O, float* lse, void* ws, size_t ws_bytes, ua_stream_t stream) {
   if (int e = check_desc(desc, false)) return e;
   const Layout l = make_layout(*desc, false);
-  if (int e = check_common(desc, false, kc, vc, xq, static_src, static_dest, ws, ws_bytes, l, false)) return e;
+  if (int e = check_common(kc, vc, xq, static_src, static_dest, ws, ws_bytes, l.fwd_end)) return e;
   if (!O || !lse) return fail(UA_EINVAL, "null output tensor");
-  char* w = (char*)ws;
+  char* wf = (char*)ws;
   hipStream_t s = (hipStream_t)stream;
-  if (int e = pack_inputs(*desc, l, false, kc, vc, xq, static_src, static_dest, w, s)) return e;
-  return run_fused_fwd_kernels(*desc, l, w, O, lse, s);
+  if (int e = pack_inputs(*desc, l, false, kc, vc, xq, static_src, static_dest, wf, s)) return e;
+  return run_fused_fwd_kernels(*desc, l, wf, O, lse, s);
 }
 
 // ---- forward for callers that cannot allocate: scratch in a device array of the library itself ----------------
@@ -518,70 +537,72 @@ int ua_fused_fwd_noalloc(const ua_desc* desc, const ua_rows* kc, const ua_rows* 
 
 int ua_fused_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
                  const void* static_dest, const void* O, const float* lse, const void* dO, void* dkc, void* dvc, void* dxq,
-                 void* dsrc, void* ddest, void* ws, size_t ws_bytes, int ws_has_fwd, ua_stream_t stream) {
+                 void* dsrc, void* ddest, void* fwd_state, void* ws, size_t ws_bytes, ua_stream_t stream) {
   if (int e = check_desc(desc, false)) return e;
   const Layout l = make_layout(*desc, false);
-  if (int e = check_common(desc, false, kc, vc, xq, static_src, static_dest, ws, ws_bytes, l, true)) return e;
+  if (int e = check_common(kc, vc, xq, static_src, static_dest, ws, ws_bytes, fwd_state ? l.total - l.fwd_end : l.total)) return e;
   if (!O || !lse || !dO || !dkc || !dvc || !dxq || !dsrc || !ddest) return fail(UA_EINVAL, "null tensor");
-  char* w = (char*)ws;
+  char *wf, *wb;
+  if (int e = bwd_bases(l, fwd_state, ws, &wf, &wb)) return e;
   hipStream_t s = (hipStream_t)stream;
   const ua_desc& d = *desc;
-  if (!ws_has_fwd) {
-    if (int e = pack_inputs(d, l, false, kc, vc, xq, static_src, static_dest, w, s)) return e;
-    if (int e = launch_carry_for(d, l, w, l.tiles ? tuned_variant(d, UA_TUNE_CARRY) : 0, s)) return e;
+  if (!fwd_state) {
+    if (int e = pack_inputs(d, l, false, kc, vc, xq, static_src, static_dest, wf, s)) return e;
+    if (int e = launch_carry_for(d, l, wf, l.tiles ? tuned_variant(d, UA_TUNE_CARRY) : 0, s)) return e;
   }
   const long rowsz = (long)d.L * d.d;
   const ua::RowsView Ov = contiguous_view(O, rowsz, d.d), dOv = contiguous_view(dO, rowsz, d.d);
   const ua::RowsView lsev = contiguous_view(lse, d.L, 1), none = null_view();
   {
     UA_PROF("pack_dO+delta", s);
-    UA_HIP(pack(d.dtype, l.D, dOv, w + l.dOp, l.grad_tiles ? nullptr : w + l.dOT, d.d, d.L, l.Lp, l.Zq, TR_PERM32, s));
-    if (d.dtype == UA_BF16) UA_HIP(delta_t<ua::bf16>(Ov, dOv, none, lsev, (float*)(w + l.delta), (float*)(w + l.lse2), d.d, d.L, l.Lp, l.Zq, s));
-    else UA_HIP(delta_t<float>(Ov, dOv, none, lsev, (float*)(w + l.delta), (float*)(w + l.lse2), d.d, d.L, l.Lp, l.Zq, s));
+    UA_HIP(pack(d.dtype, l.D, dOv, wb + l.dOp, l.grad_tiles ? nullptr : wb + l.dOT, d.d, d.L, l.Lp, l.Zq, TR_PERM32, s));
+    if (d.dtype == UA_BF16) UA_HIP(delta_t<ua::bf16>(Ov, dOv, none, lsev, (float*)(wb + l.delta), (float*)(wf + l.lse2), d.d, d.L, l.Lp, l.Zq, s));
+    else UA_HIP(delta_t<float>(Ov, dOv, none, lsev, (float*)(wb + l.delta), (float*)(wf + l.lse2), d.d, d.L, l.Lp, l.Zq, s));
   }
-  return run_bwd_common(d, l, w, false, static_src, static_dest, dkc, dvc, dxq, dsrc, ddest, s);
+  return run_bwd_common(d, l, wf, wb, false, static_src, static_dest, dkc, dvc, dxq, dsrc, ddest, s);
 }
 
 int ua_fwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
            const void* static_dest, const ua_chunked* out, void* denom, void* ws, size_t ws_bytes, ua_stream_t stream) {
   if (int e = check_desc(desc, true)) return e;
   const Layout l = make_layout(*desc, true);
-  if (int e = check_common(desc, true, kc, vc, xq, static_src, static_dest, ws, ws_bytes, l, false)) return e;
+  if (int e = check_common(kc, vc, xq, static_src, static_dest, ws, ws_bytes, l.fwd_end)) return e;
   if (!out || !out->ptr || !denom) return fail(UA_EINVAL, "null output tensor");
-  char* w = (char*)ws;
+  char* wf = (char*)ws;
   hipStream_t s = (hipStream_t)stream;
   const ua_desc& d = *desc;
   if (fast_chunk(d)) {
-    if (int e = pack_inputs(d, l, false, kc, vc, xq, static_src, static_dest, w, s)) return e;
+    if (int e = pack_inputs(d, l, false, kc, vc, xq, static_src, static_dest, wf, s)) return e;
     {
       UA_PROF("k_carry", s);
-      UA_HIP(ua::launch_carry(d.dtype, l.D, w + l.Kp, (const float*)(w + l.lsrc), (const float*)(w + l.ldest), (float*)(w + l.C), l.Lp,
-                              l.Zk, 1, nullptr, nullptr, d.r, (int*)(w + l.reach), (int*)(w + l.minkey), s));
+      UA_HIP(ua::launch_carry(d.dtype, l.D, wf + l.Kp, (const float*)(wf + l.lsrc), (const float*)(wf + l.ldest), (float*)(wf + l.C), l.Lp,
+                              l.Zk, 1, nullptr, nullptr, d.r, (int*)(wf + l.reach), (int*)(wf + l.minkey), s));
     }
     UA_PROF("k_fwd_chunked", s);
-    UA_HIP(ua::launch_fwd_chunked2(d.dtype, l.D, w + l.Qp, w + l.Kp, w + l.Vp, w + l.VT, (const float*)(w + l.lsrc),
-                                   (const float*)(w + l.ldest), (const float*)(w + l.C), (const int*)(w + l.reach),
-                                   (const int*)(w + l.minkey), out->ptr, denom, (float*)(w + l.lse2), out->stride_z, out->stride_t,
+    UA_HIP(ua::launch_fwd_chunked2(d.dtype, l.D, wf + l.Qp, wf + l.Kp, wf + l.Vp, wf + l.VT, (const float*)(wf + l.lsrc),
+                                   (const float*)(wf + l.ldest), (const float*)(wf + l.C), (const int*)(wf + l.reach),
+                                   (const int*)(wf + l.minkey), out->ptr, denom, (float*)(wf + l.lse2), out->stride_z, out->stride_t,
                                    out->stride_d, out->stride_i, d.r, d.L, l.Lp, d.d, d.chunk, l.nch, l.Zq, s));
     return UA_OK;
   }
-  if (int e = pack_inputs(d, l, true, kc, vc, xq, static_src, static_dest, w, s)) return e;
+  if (int e = pack_inputs(d, l, true, kc, vc, xq, static_src, static_dest, wf, s)) return e;
   UA_PROF("k_fwd_chunked", s);
-  UA_HIP(ua::launch_fwd_chunked(d.dtype, l.D, w + l.Qp, w + l.Kp, w + l.VT, (const float*)(w + l.lsrc),
-                                (const float*)(w + l.ldest), out->ptr, denom, (float*)(w + l.lse2), out->stride_z, out->stride_t, out->stride_d, out->stride_i, d.r, d.L,
+  UA_HIP(ua::launch_fwd_chunked(d.dtype, l.D, wf + l.Qp, wf + l.Kp, wf + l.VT, (const float*)(wf + l.lsrc),
+                                (const float*)(wf + l.ldest), out->ptr, denom, (float*)(wf + l.lse2), out->stride_z, out->stride_t, out->stride_d, out->stride_i, d.r, d.L,
                                 l.Lp, d.d, d.chunk, l.nch, l.Zk, s));
   return UA_OK;
 }
 
 int ua_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
            const void* static_dest, const ua_chunked* out, const ua_chunked* g_out, const float* g_denom, void* dkc,
-           void* dvc, void* dxq, void* dsrc, void* ddest, void* ws, size_t ws_bytes, int ws_has_fwd, ua_stream_t stream) {
+           void* dvc, void* dxq, void* dsrc, void* ddest, void* fwd_state, void* ws, size_t ws_bytes, ua_stream_t stream) {
   if (int e = check_desc(desc, true)) return e;
   const Layout l = make_layout(*desc, true);
-  if (int e = check_common(desc, true, kc, vc, xq, static_src, static_dest, ws, ws_bytes, l, true)) return e;
+  if (int e = check_common(kc, vc, xq, static_src, static_dest, ws, ws_bytes, fwd_state ? l.total - l.fwd_end : l.total)) return e;
   if (!out || !out->ptr || !g_out || !g_out->ptr || !g_denom || !dkc || !dvc || !dxq || !dsrc || !ddest)
     return fail(UA_EINVAL, "null tensor");
-  char* w = (char*)ws;
+  char *wf, *wb;
+  if (int e = bwd_bases(l, fwd_state, ws, &wf, &wb)) return e;
   hipStream_t s = (hipStream_t)stream;
   const ua_desc& d = *desc;
   const ua::RowsView outv = chunked_view(*out, l.nch);
@@ -592,41 +613,41 @@ int ua_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
   gdv.p = g_denom; gdv.sb = (long)d.L * l.nch; gdv.sh = 0; gdv.sr = 0; gdv.sn = 1; gdv.so = 0; gdv.si = l.nch; gdv.sc = 1;
   gdv.inner = 1 << 30; gdv.H = 1; gdv.R = 1; gdv.N = l.nch;
   if (fast_chunk(d)) {
-    if (!ws_has_fwd) {
+    if (!fwd_state) {
       // recompute the carries and the per-chunk normalisers (the partial outputs themselves are passed in)
-      if (int e = pack_inputs(d, l, false, kc, vc, xq, static_src, static_dest, w, s)) return e;
-      UA_HIP(ua::launch_carry(d.dtype, l.D, w + l.Kp, (const float*)(w + l.lsrc), (const float*)(w + l.ldest), (float*)(w + l.C), l.Lp,
-                              l.Zk, 1, nullptr, nullptr, d.r, (int*)(w + l.reach), (int*)(w + l.minkey), s));
-      UA_HIP(ua::launch_fwd_chunked2(d.dtype, l.D, w + l.Qp, w + l.Kp, w + l.Vp, w + l.VT, (const float*)(w + l.lsrc),
-                                     (const float*)(w + l.ldest), (const float*)(w + l.C), (const int*)(w + l.reach),
-                                     (const int*)(w + l.minkey), nullptr, nullptr, (float*)(w + l.lse2), 0, 0, 0, 0, d.r, d.L, l.Lp,
+      if (int e = pack_inputs(d, l, false, kc, vc, xq, static_src, static_dest, wf, s)) return e;
+      UA_HIP(ua::launch_carry(d.dtype, l.D, wf + l.Kp, (const float*)(wf + l.lsrc), (const float*)(wf + l.ldest), (float*)(wf + l.C), l.Lp,
+                              l.Zk, 1, nullptr, nullptr, d.r, (int*)(wf + l.reach), (int*)(wf + l.minkey), s));
+      UA_HIP(ua::launch_fwd_chunked2(d.dtype, l.D, wf + l.Qp, wf + l.Kp, wf + l.Vp, wf + l.VT, (const float*)(wf + l.lsrc),
+                                     (const float*)(wf + l.ldest), (const float*)(wf + l.C), (const int*)(wf + l.reach),
+                                     (const int*)(wf + l.minkey), nullptr, nullptr, (float*)(wf + l.lse2), 0, 0, 0, 0, d.r, d.L, l.Lp,
                                      d.d, d.chunk, l.nch, l.Zq, s));
     }
     {
       UA_PROF("pack_dO+delta", s);
-      UA_HIP(zero_fill(w + l.masked_nz, 256, s));
+      UA_HIP(zero_fill(wb + l.masked_nz, 256, s));
       // with UA_FLAG_SKIP_MASKED the flag stays 0: rows before their chunk are neither checked nor packed
-      int* nz = (int*)(w + l.masked_nz);
+      int* nz = (int*)(wb + l.masked_nz);
       int* detect = (d.flags & UA_FLAG_SKIP_MASKED) ? nullptr : nz;
-      if (d.dtype == UA_BF16) UA_HIP(delta_t<ua::bf16>(outv, gv, gdv, none, (float*)(w + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s, detect, d.chunk));
-      else UA_HIP(delta_t<float>(outv, gv, gdv, none, (float*)(w + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s, detect, d.chunk));
-      UA_HIP(pack(d.dtype, l.D, gv, w + l.dOp, l.grad_tiles ? nullptr : w + l.dOT, d.d, d.L, l.Lp, l.Zq * l.nch, TR_PERM32, s, nullptr, nz,
+      if (d.dtype == UA_BF16) UA_HIP(delta_t<ua::bf16>(outv, gv, gdv, none, (float*)(wb + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s, detect, d.chunk));
+      else UA_HIP(delta_t<float>(outv, gv, gdv, none, (float*)(wb + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s, detect, d.chunk));
+      UA_HIP(pack(d.dtype, l.D, gv, wb + l.dOp, l.grad_tiles ? nullptr : wb + l.dOT, d.d, d.L, l.Lp, l.Zq * l.nch, TR_PERM32, s, nullptr, nz,
                   d.chunk));
     }
-    return run_bwd_common(d, l, w, true, static_src, static_dest, dkc, dvc, dxq, dsrc, ddest, s);
+    return run_bwd_common(d, l, wf, wb, true, static_src, static_dest, dkc, dvc, dxq, dsrc, ddest, s);
   }
-  if (!ws_has_fwd) {
+  if (!fwd_state) {
     // recompute the per-chunk normalisers (the partial outputs themselves are passed in)
-    if (int e = pack_inputs(d, l, true, kc, vc, xq, static_src, static_dest, w, s)) return e;
-    UA_HIP(ua::launch_fwd_chunked(d.dtype, l.D, w + l.Qp, w + l.Kp, w + l.VT, (const float*)(w + l.lsrc),
-                                  (const float*)(w + l.ldest), nullptr, nullptr, (float*)(w + l.lse2), 0, 0, 0, 0, d.r, d.L, l.Lp, d.d, d.chunk, l.nch, l.Zk, s));
+    if (int e = pack_inputs(d, l, true, kc, vc, xq, static_src, static_dest, wf, s)) return e;
+    UA_HIP(ua::launch_fwd_chunked(d.dtype, l.D, wf + l.Qp, wf + l.Kp, wf + l.VT, (const float*)(wf + l.lsrc),
+                                  (const float*)(wf + l.ldest), nullptr, nullptr, (float*)(wf + l.lse2), 0, 0, 0, 0, d.r, d.L, l.Lp, d.d, d.chunk, l.nch, l.Zk, s));
   }
-  UA_HIP(ua::launch_carry(d.dtype, l.D, w + l.Kp, (const float*)(w + l.lsrc), (const float*)(w + l.ldest),
-                          (float*)(w + l.C), l.Lp, l.Zk, 0, nullptr, nullptr, 1, nullptr, nullptr, s));
-  UA_HIP(pack(d.dtype, l.D, gv, w + l.dOp, w + l.dOT, d.d, d.L, l.Lp, l.Zq * l.nch, TR_PERM16, s));
-  if (d.dtype == UA_BF16) UA_HIP(delta_t<ua::bf16>(outv, gv, gdv, none, (float*)(w + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s));
-  else UA_HIP(delta_t<float>(outv, gv, gdv, none, (float*)(w + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s));
-  return run_bwd_common(d, l, w, true, static_src, static_dest, dkc, dvc, dxq, dsrc, ddest, s);
+  UA_HIP(ua::launch_carry(d.dtype, l.D, wf + l.Kp, (const float*)(wf + l.lsrc), (const float*)(wf + l.ldest),
+                          (float*)(wf + l.C), l.Lp, l.Zk, 0, nullptr, nullptr, 1, nullptr, nullptr, s));
+  UA_HIP(pack(d.dtype, l.D, gv, wb + l.dOp, wb + l.dOT, d.d, d.L, l.Lp, l.Zq * l.nch, TR_PERM16, s));
+  if (d.dtype == UA_BF16) UA_HIP(delta_t<ua::bf16>(outv, gv, gdv, none, (float*)(wb + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s));
+  else UA_HIP(delta_t<float>(outv, gv, gdv, none, (float*)(wb + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s));
+  return run_bwd_common(d, l, wf, wb, true, static_src, static_dest, dkc, dvc, dxq, dsrc, ddest, s);
 }
 
 // 16-byte accesses to every (row, chunk) slice of a chunked tensor, with d / V lanes per slice (a power of two <= 64)
@@ -812,11 +833,12 @@ int ua_autotune(const ua_desc* desc, int op, void* ws, size_t ws_bytes, ua_strea
   if (!ws || (uintptr_t)ws % 256 != 0) return fail(UA_EWORKSPACE, "autotune needs the 256-byte aligned workspace the op ran on");
   if (ws_bytes < l.total) return fail(UA_EWORKSPACE, "autotune needs the backward-sized workspace (%zu bytes)", l.total);
   char* w = (char*)ws;
+  char *wf = w, *wb = w;      // state and scratch in one buffer
   hipStream_t s = (hipStream_t)stream;
   // throw-away outputs live in the backward part of the workspace
   if (op == UA_OP_FUSED_FWD) {
-    void* Otmp = w + l.dOp;                  // [Zq][L][d] fits in [Zq][Lp][D]
-    float* lsetmp = (float*)(w + l.delta);
+    void* Otmp = wb + l.dOp;                  // [Zq][L][d] fits in [Zq][Lp][D]
+    float* lsetmp = (float*)(wb + l.delta);
     if (l.tiles) {
       if (int e = tune_slot(d, UA_TUNE_FWD_TILES, s, [&](int v) { return launch_fwd_for(d, l, w, Otmp, lsetmp, v, s); })) return e;
       // the pre-pass rewrites the bias tiles, the reach table and the first-key table with the same values
@@ -830,13 +852,13 @@ int ua_autotune(const ua_desc* desc, int op, void* ws, size_t ws_bytes, ua_strea
   // key side first (it reads the packed upstream gradient, which the query side's throw-away dQ then overwrites)
   auto bwd_args = [&](const Layout& ll) {
     ua::BwdArgsV a{};
-    a.Kp = w + ll.Kp; a.Vp = w + ll.Vp; a.KT = w + ll.KT; a.Qp = w + ll.Qp; a.dOp = w + ll.dOp;
-    a.lsrc = (const float*)(w + ll.lsrc); a.ldest = (const float*)(w + ll.ldest); a.lse2 = (const float*)(w + ll.lse2);
-    a.delta = (const float*)(w + ll.delta); a.C = (const float*)(w + ll.C);
-    a.reach = (const int*)(w + ll.reach); a.minkey = (const int*)(w + ll.minkey);
-    a.dKdacc = (float*)(w + ll.dKdacc); a.dKrow = (float*)(w + ll.dKrow); a.dVrow = (float*)(w + ll.dVrow);
-    a.dsrc_raw = (float*)(w + ll.dsrc_raw); a.masked_nz = (const int*)(w + ll.masked_nz);
-    a.dS_st = w + ll.dS_st; a.dG_st = w + ll.dG_st; a.Bt = w + ll.Bt;
+    a.Kp = wf + ll.Kp; a.Vp = wf + ll.Vp; a.KT = wf + ll.KT; a.Qp = wf + ll.Qp; a.dOp = wb + ll.dOp;
+    a.lsrc = (const float*)(wf + ll.lsrc); a.ldest = (const float*)(wf + ll.ldest); a.lse2 = (const float*)(wf + ll.lse2);
+    a.delta = (const float*)(wb + ll.delta); a.C = (const float*)(wf + ll.C);
+    a.reach = (const int*)(wf + ll.reach); a.minkey = (const int*)(wf + ll.minkey);
+    a.dKdacc = (float*)(wb + ll.dKdacc); a.dKrow = (float*)(wb + ll.dKrow); a.dVrow = (float*)(wb + ll.dVrow);
+    a.dsrc_raw = (float*)(wb + ll.dsrc_raw); a.masked_nz = (const int*)(wb + ll.masked_nz);
+    a.dS_st = wb + ll.dS_st; a.dG_st = wb + ll.dG_st; a.Bt = wf + ll.Bt;
     a.R = d.r; a.L = d.L; a.Lp = ll.Lp; a.c = 128; a.nch = 1; a.key_parts = ll.key_parts;
     return a;
   };
@@ -855,7 +877,7 @@ int ua_autotune(const ua_desc* desc, int op, void* ws, size_t ws_bytes, ua_strea
   }
   {
     const ua::BwdArgsV a = bwd_args(l);
-    void* dqtmp = w + l.dOp;
+    void* dqtmp = wb + l.dOp;
     if (int e = tune_slot(d, UA_TUNE_BWD_QUERIES, s, [&](int v) {
           UA_HIP(ua::launch_bwd_queries_from_tiles(l.D, a, dqtmp, d.d, l.Zq, s, v));
           return (int)UA_OK;

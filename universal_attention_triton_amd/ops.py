@@ -68,26 +68,49 @@ def _workspace(desc, op, device):
 
 
 def _prep(kc, vc, xq, static_src, static_dest):
-    _require_gpu(kc, vc, xq, static_src, static_dest)
-    if not (kc.dtype == vc.dtype == xq.dtype == static_src.dtype == static_dest.dtype):
-        raise TypeError("all five inputs must share one dtype")
+    """Checks the shapes against one another (the kernels trust the descriptor), makes the feature stride 1 and the
+    gates contiguous [b,h,L].  -> kc, vc, xq, src, dest, gate flag.
+
+    dtypes: kc, vc and xq share one dtype (float32 or bfloat16).  The gates may have it too; any other combination
+    (float32 gates next to bfloat16 tensors, as the reference allows: its dstatic_src follows static_src.dtype,
+    Universal_Attention/triton/universal_attention_kernel.py:825-829) runs with float32 gates."""
+    if kc.dim() != 5 or vc.dim() != 5 or xq.dim() not in (5, 6):
+        raise ValueError("kc, vc [b,h,n,c,d] and xq [b,h,r,l,d] or [b,h,r,_n,_c,d] expected, got %s %s %s"
+                         % (tuple(kc.shape), tuple(vc.shape), tuple(xq.shape)))
+    if not (kc.dtype == vc.dtype == xq.dtype):
+        raise TypeError("kc, vc and xq must share one dtype, got %s %s %s" % (kc.dtype, vc.dtype, xq.dtype))
     b, h, n, c, d = kc.shape
+    L = n * c
+    seq = xq.shape[3] if xq.dim() == 5 else xq.shape[3] * xq.shape[4]
+    if vc.shape != kc.shape:
+        raise ValueError("vc %s does not match kc %s" % (tuple(vc.shape), tuple(kc.shape)))
+    if xq.shape[0] != b or xq.shape[1] != h or xq.shape[-1] != d or seq != L:
+        raise ValueError("xq %s does not match kc %s: need [b=%d, h=%d, r, %d positions, d=%d]" % (tuple(xq.shape), tuple(kc.shape), b, h, L, d))
+    if static_src.numel() != b * h * L or static_dest.numel() != b * h * L or static_src.shape[:2] != (b, h) or static_dest.shape[:2] != (b, h):
+        raise ValueError("gates %s / %s do not match [b=%d, h=%d, %d positions]" % (tuple(static_src.shape), tuple(static_dest.shape), b, h, L))
+    _dtype_code(xq)
+    _require_gpu(kc, vc, xq, static_src, static_dest)
     kc, vc, xq = _last_contig(kc), _last_contig(vc), _last_contig(xq)
-    src = static_src.reshape(b, h, n * c).contiguous()
-    dest = static_dest.reshape(b, h, n * c).contiguous()
-    return kc, vc, xq, src, dest
+    same = static_src.dtype == xq.dtype and static_dest.dtype == xq.dtype
+    gdt = xq.dtype if same else torch.float32
+    src = static_src.reshape(b, h, L).to(gdt).contiguous()
+    dest = static_dest.reshape(b, h, L).to(gdt).contiguous()
+    gflag = _lib.UA_FLAG_GATES_F32 if (gdt == torch.float32 and xq.dtype != torch.float32) else 0
+    return kc, vc, xq, src, dest, gflag
 
 
-def chunked_forward(kc, vc, xq, static_src, static_dest, for_backward=False, recompute=False):
+def chunked_forward(kc, vc, xq, static_src, static_dest, keep_state=False, recompute=False):
     """-> out [b,h,r,l,d,n] (chunk-major storage, returned as a permuted view), denom [b,h,r,l,n], state
-    recompute: size the state for a backward that runs with UA_FLAG_RECOMPUTE (pass the same value to chunked_backward)."""
-    kc, vc, xq, src, dest = _prep(kc, vc, xq, static_src, static_dest)
+    keep_state: return the forward state (the workspace, ua_workspace_bytes(UA_OP_FWD) bytes) for chunked_backward;
+    otherwise state is None and the backward rebuilds it.
+    recompute: the flags of the state must match the backward's (pass the same value to chunked_backward)."""
+    kc, vc, xq, src, dest, gflag = _prep(kc, vc, xq, static_src, static_dest)
     lib = _lib.load()
     b, h, n, c, d = kc.shape
     r = xq.shape[2]
     L = n * c
-    desc = _desc(kc, xq, True, _lib.UA_FLAG_RECOMPUTE if recompute else 0)
-    ws = _workspace(desc, _lib.UA_OP_BWD if for_backward else _lib.UA_OP_FWD, xq.device)
+    desc = _desc(kc, xq, True, (_lib.UA_FLAG_RECOMPUTE if recompute else 0) | gflag)
+    ws = _workspace(desc, _lib.UA_OP_FWD, xq.device)
     store = torch.empty(b, h, r, n, L, d, dtype=xq.dtype, device=xq.device)
     out = store.permute(0, 1, 2, 4, 5, 3)
     denom = torch.empty(b, h, r, L, n, dtype=xq.dtype, device=xq.device)
@@ -95,34 +118,39 @@ def chunked_forward(kc, vc, xq, static_src, static_dest, for_backward=False, rec
     _lib.check(lib.ua_fwd(ctypes.byref(desc), ctypes.byref(_rows_k(kc)), ctypes.byref(_rows_k(vc)), ctypes.byref(_rows_q(xq)),
                           src.data_ptr(), dest.data_ptr(), ctypes.byref(oc), denom.data_ptr(), ws.data_ptr(), ws.numel(), _stream()),
                "ua_fwd")
-    return out, denom, ws
+    return out, denom, (ws if keep_state else None)
 
 
-def chunked_backward(kc, vc, xq, static_src, static_dest, out, g_out, g_denom, ws=None, skip_masked=False, recompute=False):
-    kc, vc, xq, src, dest = _prep(kc, vc, xq, static_src, static_dest)
+def _gate_grads(b, h, L, src, static_src, static_dest):
+    dsrc = torch.empty(b, h, L, dtype=src.dtype, device=src.device)
+    return dsrc, torch.empty_like(dsrc)
+
+
+def chunked_backward(kc, vc, xq, static_src, static_dest, out, g_out, g_denom, state=None, skip_masked=False, recompute=False):
+    """state: what chunked_forward(keep_state=True) returned for the same inputs and flags, or None."""
+    src_dtype, dest_dtype = static_src.dtype, static_dest.dtype
+    kc, vc, xq, src, dest, gflag = _prep(kc, vc, xq, static_src, static_dest)
     lib = _lib.load()
     b, h, n, c, d = kc.shape
     r = xq.shape[2]
     L = n * c
-    desc = _desc(kc, xq, True, (_lib.UA_FLAG_SKIP_MASKED if skip_masked else 0) | (_lib.UA_FLAG_RECOMPUTE if recompute else 0))
-    has_fwd = ws is not None
-    need = lib.ua_workspace_bytes(ctypes.byref(desc), _lib.UA_OP_BWD)
-    if ws is None or ws.numel() < need:
-        ws, has_fwd = _workspace(desc, _lib.UA_OP_BWD, xq.device), False
+    desc = _desc(kc, xq, True, (_lib.UA_FLAG_SKIP_MASKED if skip_masked else 0) | (_lib.UA_FLAG_RECOMPUTE if recompute else 0) | gflag)
+    if state is not None and state.numel() < lib.ua_workspace_bytes(ctypes.byref(desc), _lib.UA_OP_FWD):
+        state = None
+    ws = _workspace(desc, _lib.UA_OP_BWD_SCRATCH if state is not None else _lib.UA_OP_BWD, xq.device)
     out_t, oc = _chunked(out)
     g_out_t, gc = _chunked(g_out.to(xq.dtype))
     gd = g_denom.float().contiguous()
     dk = torch.empty(b, h, n, c, d, dtype=kc.dtype, device=kc.device)
     dv = torch.empty_like(dk)
     dq = torch.empty(b, h, r, L, d, dtype=xq.dtype, device=xq.device)
-    dsrc = torch.empty(b, h, L, dtype=src.dtype, device=src.device)
-    ddest = torch.empty_like(dsrc)
+    dsrc, ddest = _gate_grads(b, h, L, src, static_src, static_dest)
     _lib.check(lib.ua_bwd(ctypes.byref(desc), ctypes.byref(_rows_k(kc)), ctypes.byref(_rows_k(vc)), ctypes.byref(_rows_q(xq)),
                           src.data_ptr(), dest.data_ptr(), ctypes.byref(oc), ctypes.byref(gc), gd.data_ptr(), dk.data_ptr(),
-                          dv.data_ptr(), dq.data_ptr(), dsrc.data_ptr(), ddest.data_ptr(), ws.data_ptr(), ws.numel(),
-                          1 if has_fwd else 0, _stream()), "ua_bwd")
+                          dv.data_ptr(), dq.data_ptr(), dsrc.data_ptr(), ddest.data_ptr(),
+                          state.data_ptr() if state is not None else None, ws.data_ptr(), ws.numel(), _stream()), "ua_bwd")
     del out_t, g_out_t
-    return dk, dv, dq, dsrc, ddest
+    return dk, dv, dq, dsrc.to(src_dtype), ddest.to(dest_dtype)
 
 
 def _fused_flags(prune, recompute, share_groups=False):
@@ -130,57 +158,65 @@ def _fused_flags(prune, recompute, share_groups=False):
             | (_lib.UA_FLAG_SHARE_GROUPS if share_groups else 0))
 
 
-def fused_forward(kc, vc, xq, static_src, static_dest, for_backward=False, prune=False, recompute=False, share_groups=False):
+def fused_forward(kc, vc, xq, static_src, static_dest, keep_state=False, prune=False, recompute=False, share_groups=False,
+                  _ws=None):
     """-> O [b,h,r,l,d], lse [b,h,r,l] (float32), state
 
+    keep_state: return the forward state (the workspace: packed inputs and, for bf16, the bias tiles;
+    ua_workspace_bytes(UA_OP_FUSED_FWD) bytes) so that fused_backward need not rebuild it; otherwise state is None.
     prune: skip (key, query) pairs whose softmax weight is provably below 2^-48 because of the accumulated decay
-    (UA_FLAG_PRUNE); the backward that receives the returned state follows the same selection.
-    recompute: size the state for a backward that runs with UA_FLAG_RECOMPUTE (pass the same value to fused_backward).
-    share_groups: likewise for UA_FLAG_SHARE_GROUPS (grouped queries: one key-side sweep per kv head whatever the shape)."""
-    kc, vc, xq, src, dest = _prep(kc, vc, xq, static_src, static_dest)
+    (UA_FLAG_PRUNE); a backward that receives the returned state follows the same selection.
+    recompute, share_groups: flags of the state; pass the same values to fused_backward."""
+    kc, vc, xq, src, dest, gflag = _prep(kc, vc, xq, static_src, static_dest)
     lib = _lib.load()
     b, h, n, c, d = kc.shape
     r = xq.shape[2]
     L = n * c
-    desc = _desc(kc, xq, False, _fused_flags(prune, recompute, share_groups))
-    ws = _workspace(desc, _lib.UA_OP_FUSED_BWD if for_backward else _lib.UA_OP_FUSED_FWD, xq.device)
+    desc = _desc(kc, xq, False, _fused_flags(prune, recompute, share_groups) | gflag)
+    ws = _ws if _ws is not None else _workspace(desc, _lib.UA_OP_FUSED_FWD, xq.device)
     O = torch.empty(b, h, r, L, d, dtype=xq.dtype, device=xq.device)
     lse = torch.empty(b, h, r, L, dtype=torch.float32, device=xq.device)
     _lib.check(lib.ua_fused_fwd(ctypes.byref(desc), ctypes.byref(_rows_k(kc)), ctypes.byref(_rows_k(vc)), ctypes.byref(_rows_q(xq)),
                                 src.data_ptr(), dest.data_ptr(), O.data_ptr(), lse.data_ptr(), ws.data_ptr(), ws.numel(), _stream()),
                "ua_fused_fwd")
-    return O, lse, ws
+    return O, lse, (ws if keep_state else None)
 
 
-def fused_backward(kc, vc, xq, static_src, static_dest, O, lse, dO, ws=None, prune=False, recompute=False, share_groups=False,
-                   _ws_override=None):
-    """ws: the state fused_forward returned for the same inputs (skips the recompute and keeps its pruning);
-    prune only matters when ws is None.  recompute: UA_FLAG_RECOMPUTE (small workspace, slower; bf16 only)."""
-    kc, vc, xq, src, dest = _prep(kc, vc, xq, static_src, static_dest)
+def fused_backward(kc, vc, xq, static_src, static_dest, O, lse, dO, state=None, prune=False, recompute=False, share_groups=False,
+                   _ws=None):
+    """state: what fused_forward(keep_state=True) returned for the same inputs and flags (skips the recompute and keeps
+    its pruning), or None; prune only matters without it.  recompute: UA_FLAG_RECOMPUTE (small workspace, slower; bf16)."""
+    src_dtype, dest_dtype = static_src.dtype, static_dest.dtype
+    kc, vc, xq, src, dest, gflag = _prep(kc, vc, xq, static_src, static_dest)
     lib = _lib.load()
     b, h, n, c, d = kc.shape
     r = xq.shape[2]
     L = n * c
-    desc = _desc(kc, xq, False, _fused_flags(prune, recompute, share_groups))
-    has_fwd = ws is not None
-    need = lib.ua_workspace_bytes(ctypes.byref(desc), _lib.UA_OP_FUSED_BWD)
-    if _ws_override is not None:
-        ws, has_fwd = _ws_override, False
-    elif ws is None or ws.numel() < need:
-        ws, has_fwd = _workspace(desc, _lib.UA_OP_FUSED_BWD, xq.device), False
+    desc = _desc(kc, xq, False, _fused_flags(prune, recompute, share_groups) | gflag)
+    if state is not None and state.numel() < lib.ua_workspace_bytes(ctypes.byref(desc), _lib.UA_OP_FUSED_FWD):
+        state = None
+    ws = _ws if _ws is not None else _workspace(desc, _lib.UA_OP_FUSED_BWD_SCRATCH if state is not None else _lib.UA_OP_FUSED_BWD, xq.device)
     O = O.contiguous()
     dO = dO.to(xq.dtype).contiguous()
     lse = lse.float().contiguous()
     dk = torch.empty(b, h, n, c, d, dtype=kc.dtype, device=kc.device)
     dv = torch.empty_like(dk)
     dq = torch.empty(b, h, r, L, d, dtype=xq.dtype, device=xq.device)
-    dsrc = torch.empty(b, h, L, dtype=src.dtype, device=src.device)
-    ddest = torch.empty_like(dsrc)
+    dsrc, ddest = _gate_grads(b, h, L, src, static_src, static_dest)
     _lib.check(lib.ua_fused_bwd(ctypes.byref(desc), ctypes.byref(_rows_k(kc)), ctypes.byref(_rows_k(vc)), ctypes.byref(_rows_q(xq)),
                                 src.data_ptr(), dest.data_ptr(), O.data_ptr(), lse.data_ptr(), dO.data_ptr(), dk.data_ptr(),
-                                dv.data_ptr(), dq.data_ptr(), dsrc.data_ptr(), ddest.data_ptr(), ws.data_ptr(), ws.numel(),
-                                1 if has_fwd else 0, _stream()), "ua_fused_bwd")
-    return dk, dv, dq, dsrc, ddest
+                                dv.data_ptr(), dq.data_ptr(), dsrc.data_ptr(), ddest.data_ptr(),
+                                state.data_ptr() if state is not None else None, ws.data_ptr(), ws.numel(), _stream()), "ua_fused_bwd")
+    return dk, dv, dq, dsrc.to(src_dtype), ddest.to(dest_dtype)
+
+
+def retained_bytes(kc, vc, xq, static_src, static_dest, recompute=False):
+    """Bytes of forward state the fused operator keeps alive between forward and backward (0 with recompute)."""
+    kc, vc, xq, src, dest, gflag = _prep(kc, vc, xq, static_src, static_dest)
+    if recompute:
+        return 0
+    desc = _desc(kc, xq, False, gflag)
+    return _lib.load().ua_workspace_bytes(ctypes.byref(desc), _lib.UA_OP_FUSED_FWD)
 
 
 def _merge_views(mat):
@@ -234,18 +270,23 @@ def autotune(kc, vc, xq, static_src, static_dest, dO=None, backward=True):
     times every variant of every kernel on its path on the device (ua_autotune) and records the fastest of each in the
     library's table.  Returns {slot name: variant} for the slots that have more than one variant here."""
     lib = _lib.load()
-    O, lse, ws = fused_forward(kc, vc, xq, static_src, static_dest, for_backward=True)
-    kc_, vc_, xq_, _, _ = _prep(kc, vc, xq, static_src, static_dest)
-    desc = _desc(kc_, xq_, False)
-    _lib.check(lib.ua_autotune(ctypes.byref(desc), _lib.UA_OP_FUSED_FWD, ws.data_ptr(), ws.numel(), _stream()), "ua_autotune")
-    if backward and xq.dtype == torch.bfloat16:
-        # the number of key-side parts changes the workspace: tune it on a workspace large enough for every choice
+    kc_, vc_, xq_, _, _, gflag = _prep(kc, vc, xq, static_src, static_dest)
+    desc = _desc(kc_, xq_, False, gflag)
+    bwd = backward and xq.dtype == torch.bfloat16
+    # state and scratch in one buffer; the number of key-side parts changes its size: large enough for every choice
+    n_parts = lib.ua_tune_variants(ctypes.byref(desc), _lib.UA_TUNE_BWD_PARTS) if bwd else 1
+    need = max(_with_parts(desc, v if n_parts > 1 else -1, lambda: lib.ua_workspace_bytes(ctypes.byref(desc), _lib.UA_OP_FUSED_BWD))
+               for v in range(n_parts))
+    fwd_bytes = lib.ua_workspace_bytes(ctypes.byref(desc), _lib.UA_OP_FUSED_FWD)
+    if need == 0 or fwd_bytes == 0:
+        raise _lib.UaError("unsupported problem: " + lib.ua_last_error().decode())
+    big = torch.empty(need, dtype=torch.uint8, device=xq.device)
+    O, lse, _ = fused_forward(kc, vc, xq, static_src, static_dest, _ws=big)
+    _lib.check(lib.ua_autotune(ctypes.byref(desc), _lib.UA_OP_FUSED_FWD, big.data_ptr(), big.numel(), _stream()), "ua_autotune")
+    if bwd:
         if dO is None:
             dO = torch.ones_like(O)
-        need = max(_with_parts(desc, v, lambda: lib.ua_workspace_bytes(ctypes.byref(desc), _lib.UA_OP_FUSED_BWD))
-                   for v in range(lib.ua_tune_variants(ctypes.byref(desc), _lib.UA_TUNE_BWD_PARTS)))
-        big = torch.empty(need, dtype=torch.uint8, device=xq.device)
-        fused_backward(kc, vc, xq, static_src, static_dest, O, lse, dO, ws=None, _ws_override=big)
+        fused_backward(kc, vc, xq, static_src, static_dest, O, lse, dO, state=big, _ws=big[fwd_bytes:])
         _lib.check(lib.ua_autotune(ctypes.byref(desc), _lib.UA_OP_FUSED_BWD, big.data_ptr(), big.numel(), _stream()), "ua_autotune")
     out = {name: lib.ua_tune_get(ctypes.byref(desc), slot) for name, slot in _lib.TUNE_SLOTS.items()
            if lib.ua_tune_variants(ctypes.byref(desc), slot) > 1 and lib.ua_tune_get(ctypes.byref(desc), slot) >= 0}
@@ -257,6 +298,8 @@ def autotune(kc, vc, xq, static_src, static_dest, dO=None, backward=True):
 
 def _with_parts(desc, variant, fn):
     lib = _lib.load()
+    if variant < 0:
+        return fn()
     old = lib.ua_tune_get(ctypes.byref(desc), _lib.UA_TUNE_BWD_PARTS)
     lib.ua_tune_set(ctypes.byref(desc), _lib.UA_TUNE_BWD_PARTS, variant)
     try:
@@ -343,6 +386,11 @@ def fused_forward_noalloc(kc, vc, xq, static_src, static_dest, O, lse):
             raise ValueError("gates and outputs must be contiguous (no copies are made)")
     lib = _lib.load()
     desc = _desc(kc, xq, False, 0)
+    b, h, n, c, d = kc.shape
+    if vc.shape != kc.shape or xq.shape[:2] != (b, h) or xq.shape[-1] != d or xq.numel() != b * h * xq.shape[2] * n * c * d \
+            or static_src.numel() != b * h * n * c or static_dest.numel() != b * h * n * c \
+            or O.numel() != xq.numel() or lse.numel() * d != xq.numel():
+        raise ValueError("shapes of the tensors do not match one another")
     _lib.check(lib.ua_fused_fwd_noalloc(ctypes.byref(desc), ctypes.byref(_rows_k(kc)), ctypes.byref(_rows_k(vc)),
                                         ctypes.byref(_rows_q(xq)), static_src.data_ptr(), static_dest.data_ptr(), O.data_ptr(),
                                         lse.data_ptr(), _stream()), "ua_fused_fwd_noalloc")

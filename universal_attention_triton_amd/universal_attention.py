@@ -14,19 +14,19 @@ import torch
 from torch.autograd import Function
 
 from . import ops
-from .universal_attention_autograd import _ChunkedBase
+from .universal_attention_autograd import _ChunkedBase, _put_state, _take_state
 
 
 class UniversalAttention(_ChunkedBase):
     @staticmethod
-    def forward(ctx, kc, vc, xq, static_src, static_dest):
+    def forward(kc, vc, xq, static_src, static_dest):
         b, h, r, _n, _c, d = xq.shape
         _, _, n_, c_, _ = kc.shape
         assert kc.shape == (b, h, n_, c_, d)
         assert vc.shape == (b, h, n_, c_, d)
         assert static_src.shape == (b, h, n_, c_)
         assert static_dest.shape == (b, h, _n, _c)
-        return _ChunkedBase.forward(ctx, kc, vc, xq, static_src, static_dest)
+        return _ChunkedBase.forward(kc, vc, xq, static_src, static_dest)
 
     @staticmethod
     def backward(ctx, dout, ddenom):
@@ -40,34 +40,48 @@ class UniversalAttention(_ChunkedBase):
 
 class _FusedUniversalAttention(Function):
     @staticmethod
-    def forward(ctx, kc, vc, xq, static_src, static_dest, prune=False, recompute=False):
-        need_grad = any(ctx.needs_input_grad)
-        O, lse, ws = ops.fused_forward(kc, vc, xq, static_src, static_dest, for_backward=need_grad, prune=prune,
-                                       recompute=recompute)
+    def forward(kc, vc, xq, static_src, static_dest, prune=False, recompute=False, keep_state=True):
+        # the forward state (packed inputs + bias tiles) is kept for the backward unless the caller asks for the
+        # reference's footprint (its five inputs, plus O and lse here)
+        keep = keep_state and not recompute and any(t.requires_grad for t in (kc, vc, xq, static_src, static_dest))
+        O, lse, state = ops.fused_forward(kc, vc, xq, static_src, static_dest, keep_state=keep, prune=prune, recompute=recompute)
+        O = O.view(*xq.shape)
+        _put_state(O, state)
+        return O, lse
+
+    @staticmethod
+    def setup_context(ctx, inputs, output):
+        kc, vc, xq, static_src, static_dest, prune, recompute, _ = inputs
+        O, lse = output
         ctx.prune, ctx.recompute = prune, recompute
         ctx.save_for_backward(kc, vc, xq, static_src, static_dest, O, lse)
-        ctx.ws = ws if need_grad else None
+        ctx.state = _take_state(O)
         ctx.mark_non_differentiable(lse)
-        return O.view(*xq.shape), lse
 
     @staticmethod
     def backward(ctx, dO, _dlse):
         kc, vc, xq, static_src, static_dest, O, lse = ctx.saved_tensors
         b, h, n, c, d = kc.shape
-        dO = dO.reshape(b, h, xq.shape[2], n * c, d)
-        dk, dv, dq, dsrc, ddest = ops.fused_backward(kc, vc, xq, static_src, static_dest, O, lse, dO, ws=ctx.ws, prune=ctx.prune,
-                                                     recompute=ctx.recompute)
-        ctx.ws = None
-        return dk, dv, dq.view(xq.shape), dsrc.view(static_src.shape), ddest.view(static_dest.shape), None, None
+        r = xq.shape[2]
+        dO = dO.reshape(b, h, r, n * c, d)
+        dk, dv, dq, dsrc, ddest = ops.fused_backward(kc, vc, xq, static_src, static_dest, O.reshape(b, h, r, n * c, d), lse, dO,
+                                                     state=ctx.state, prune=ctx.prune, recompute=ctx.recompute)
+        ctx.state = None
+        return dk, dv, dq.view(xq.shape), dsrc.view(static_src.shape), ddest.view(static_dest.shape), None, None, None
 
 
-def universal_attention(kc, vc, xq, static_src, static_dest, return_lse=False, prune=False, recompute=False):
+def universal_attention(kc, vc, xq, static_src, static_dest, return_lse=False, prune=False, recompute=False, keep_state=True):
     """Fused forward/backward.  Accepts the 1-D (xq [b,h,r,l,d]) and the 2-D (xq [b,h,r,_n,_c,d]) layouts;
     the result has xq's shape.  prune=True skips (key, query) pairs whose softmax weight is provably below 2^-48
     because of the accumulated decay: same results to float32 rounding, less work on long sequences.
-    recompute=True (bf16): the backward keeps its workspace at O(L*L/16) bytes per head by recomputing the score and
-    decay gradients in its second kernel instead of exchanging them through 2*L*L bytes per head (UA_FLAG_RECOMPUTE)."""
-    O, lse = _FusedUniversalAttention.apply(kc, vc, xq, static_src, static_dest, prune, recompute)
+
+    Memory between forward and backward: by default the forward state (packed inputs and, for bf16, the bias tiles: about
+    Lp*Lp bytes per kv head, ops.retained_bytes) stays alive until the backward, whose scratch is allocated there.
+    keep_state=False keeps nothing but the five inputs, O and lse, as the reference does
+    (Universal_Attention/universal_attention.py:27-31); the backward then rebuilds the state first.
+    recompute=True (bf16) implies that and also keeps the backward's workspace at O(L*L/16) bytes per head by
+    recomputing the score and decay gradients in every kernel instead of exchanging tiles (UA_FLAG_RECOMPUTE)."""
+    O, lse = _FusedUniversalAttention.apply(kc, vc, xq, static_src, static_dest, prune, recompute, keep_state)
     return (O, lse) if return_lse else O
 
 
@@ -82,5 +96,7 @@ def attention(q, k, v, causal=True, sm_scale=None, static_src=None, static_dest=
     assert Hq % Hkv == 0
     r = Hq // Hkv
     xq = q.view(B, r, Hkv, L, d).transpose(1, 2)                 # [B, H_kv, r, L, d]
-    O = universal_attention(k.unsqueeze(2), v.unsqueeze(2), xq, static_src.unsqueeze(2), static_dest)
+    # ac ("activation checkpointing" of the reference: do not keep the bias between forward and backward,
+    # universal_attention_kernel_opt.py:494-497, :551-553) = keep no forward state here
+    O = universal_attention(k.unsqueeze(2), v.unsqueeze(2), xq, static_src.unsqueeze(2), static_dest, keep_state=not ac)
     return O.transpose(1, 2).reshape(B, Hq, L, d)

@@ -10,10 +10,27 @@
 `out` is returned with chunk-major storage (a permuted view): its values and shape are the
 reference's, its strides are not.  All compute happens in libua_hip.so; tensors must live on the GPU.
 """
+import threading
+
 import torch
 from torch.autograd import Function
 
 from . import ops
+
+
+# forward() has no ctx (new-style Function, like the reference's Triton-backed entry point,
+# Universal_Attention/universal_attention.py:5-31); the forward state travels to setup_context through this slot
+_handoff = threading.local()
+
+
+def _put_state(out, state):
+    _handoff.item = (out.data_ptr(), state)
+
+
+def _take_state(out):
+    item = getattr(_handoff, "item", None)
+    _handoff.item = None
+    return item[1] if item is not None and item[0] == out.data_ptr() else None
 
 
 class _ChunkedBase(Function):
@@ -23,23 +40,34 @@ class _ChunkedBase(Function):
     # bf16, chunk a multiple of 64: True keeps the backward's workspace small (UA_FLAG_RECOMPUTE: its second kernel
     # recomputes the score and decay gradients instead of reading them from 2*L*L bytes per head)
     recompute = False
+    # True: keep the forward state (packed inputs, carries, per-chunk normalisers) for the backward instead of
+    # rebuilding it there; costs ua_workspace_bytes(UA_OP_FWD) bytes per call between forward and backward.  The
+    # reference keeps its five inputs only (universal_attention.py:27-31), which is the default here too.
+    keep_state = False
 
     @staticmethod
-    def forward(ctx, kc, vc, xq, static_src, static_dest):
-        need_grad = any(ctx.needs_input_grad)
-        out, denom, ws = ops.chunked_forward(kc, vc, xq, static_src, static_dest, for_backward=need_grad,
-                                             recompute=_ChunkedBase.recompute)
-        ctx.save_for_backward(kc, vc, xq, static_src, static_dest, out)
-        ctx.ws = ws if need_grad else None
+    def forward(kc, vc, xq, static_src, static_dest):
+        keep = _ChunkedBase.keep_state and any(t.requires_grad for t in (kc, vc, xq, static_src, static_dest))
+        out, denom, state = ops.chunked_forward(kc, vc, xq, static_src, static_dest, keep_state=keep,
+                                                recompute=_ChunkedBase.recompute)
+        _put_state(out, state)
         return out, denom
+
+    @staticmethod
+    def setup_context(ctx, inputs, output):
+        kc, vc, xq, static_src, static_dest = inputs
+        out, _ = output
+        # `out` is the tensor the caller holds anyway (SMVecMatMul saves it too): saving it costs no memory
+        ctx.save_for_backward(kc, vc, xq, static_src, static_dest, out)
+        ctx.state = _take_state(out)
 
     @staticmethod
     def backward(ctx, g_out, g_denom):
         kc, vc, xq, static_src, static_dest, out = ctx.saved_tensors
         dk, dv, dq, dsrc, ddest = ops.chunked_backward(kc, vc, xq, static_src, static_dest, out, g_out, g_denom,
-                                                       ws=ctx.ws, skip_masked=_ChunkedBase.skip_masked,
+                                                       state=ctx.state, skip_masked=_ChunkedBase.skip_masked,
                                                        recompute=_ChunkedBase.recompute)
-        ctx.ws = None
+        ctx.state = None
         return dk, dv, dq.view(xq.shape), dsrc.view(static_src.shape), ddest.view(static_dest.shape)
 
 
@@ -47,20 +75,20 @@ class UniversalAttention(_ChunkedBase):
     """1-D layout: xq [b,h,r,l,d], static_dest [b,h,l]."""
 
     @staticmethod
-    def forward(ctx, kc, vc, xq, static_src, static_dest):
+    def forward(kc, vc, xq, static_src, static_dest):
         b, h, r, l, d = xq.shape
         _, _, n, c, _ = kc.shape
-        return _ChunkedBase.forward(ctx, kc, vc, xq, static_src, static_dest)
+        return _ChunkedBase.forward(kc, vc, xq, static_src, static_dest)
 
 
 class UniversalAttention2(_ChunkedBase):
     """2-D layout: xq [b,h,r,_n,_c,d], static_dest [b,h,_n,_c]; the query tiling does not change the result."""
 
     @staticmethod
-    def forward(ctx, kc, vc, xq, static_src, static_dest):
+    def forward(kc, vc, xq, static_src, static_dest):
         b, h, r, _n, _c, d = xq.shape
         _, _, n_, c_, _ = kc.shape
-        return _ChunkedBase.forward(ctx, kc, vc, xq, static_src, static_dest)
+        return _ChunkedBase.forward(kc, vc, xq, static_src, static_dest)
 
 
 class SMVecMatMul(Function):
