@@ -65,7 +65,10 @@ enum {
                               than float32 rounding.  ua_fused_bwd with the forward state follows what the forward recorded. */
 };
 
-/* Problem description.  kc, vc: [b,h,L,d] seen as [b,h,n,c,d]; xq: [b,h,r,L,d]; gates: [b,h,L]. */
+/* Problem description.  kc, vc: [b,h,L,d] seen as [b,h,n,c,d]; xq: [b,h,r,L,d]; gates: [b,h,L].
+ * Head dim d: 1..128 everywhere (zero-padded to 64 or 128 inside); 129..256 (padded to 256, as the reference's
+ * second-generation kernel pads to a power of two up to 256, universal_attention_kernel_opt.py:441-456) for the bf16
+ * fused operator without UA_FLAG_RECOMPUTE. */
 typedef struct ua_desc {
   int32_t b, h, r, L, d;
   int32_t chunk; /* keys per chunk c (L % c == 0; c == 16 or c % 32 == 0, c <= 256); ignored by fused ops */
@@ -90,6 +93,9 @@ typedef struct ua_chunked {
 } ua_chunked;
 
 int ua_version(void);
+/* Hash of the sources this library was compiled from (csrc/ and this header), as computed by the build script; a host
+ * binding can compare it with the sources it sees to refuse a stale binary.  No counterpart in the reference. */
+const char* ua_source_hash(void);
 /* Thread-local description of the last failure on this thread ("" if none). */
 const char* ua_last_error(void);
 

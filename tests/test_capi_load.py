@@ -192,3 +192,8 @@ def test_mismatched_shapes_and_dtypes_are_refused_before_any_launch():
         ops.fused_forward(kc.half(), vc.half(), xq.half(), src, dest)
     with pytest.raises(_lib.UaError):                                  # well-formed, but not on the GPU
         ops.fused_forward(kc, vc, xq, src, dest)
+
+
+def test_library_reports_the_hash_of_the_sources_it_was_built_from():
+    from universal_attention_triton_amd import build
+    assert _lib.load().ua_source_hash().decode() == build.source_hash()

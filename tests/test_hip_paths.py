@@ -183,3 +183,61 @@ def test_memory_kept_between_forward_and_backward_at_the_headline_shape():
         del O, grads
         torch.cuda.synchronize()
         assert torch.cuda.memory_allocated() - base <= (8 << 20)
+
+
+@pytest.mark.parametrize("shape", [(1, 2, 1, 320, 160), (1, 1, 2, 200, 256), (2, 1, 4, 128, 136)])
+def test_head_dims_above_128_bf16_fused_operator(shape):
+    """The reference's second-generation kernel takes head dims up to 256 (zero-padded to a power of two,
+    universal_attention_kernel_opt.py:441-456): forward and the five gradients at d = 160, 256 and 136 (r = 1, 2, 4)
+    against float64 autograd of the dense oracle; float32 and the chunked operator refuse such head dims."""
+    from universal_attention_triton_amd import _lib, ops
+    from universal_attention_triton_amd.universal_attention import universal_attention
+    b, h, r, L, d = shape
+    bf = torch.bfloat16
+    inp = orc.make_inputs(b, h, r, L, d, 8, dtype=bf, seed=91)
+    O_ref, lse_ref, g_ref = dense_reference(inp)
+    leaves = [inp[k_].cuda().requires_grad_() for k_ in NAMES]
+    O, lse = universal_attention(*leaves, return_lse=True)
+    grads = torch.autograd.grad(O, leaves, inp["dO"].cuda())
+    torch.cuda.synchronize()
+    assert rel_err(O, O_ref) <= TOL[bf], rel_err(O, O_ref)
+    assert float((lse.cpu().double() - lse_ref).abs().max()) <= 2e-2
+    _table("head dim %d" % d, grads, g_ref, TOL[bf])
+    with pytest.raises(_lib.UaError):
+        ops.fused_forward(*[x.detach().float() for x in leaves])
+    with pytest.raises(_lib.UaError):
+        ops.chunked_forward(*[x.detach() for x in leaves])
+
+
+@pytest.mark.parametrize("recompute", [False, True])
+def test_large_scores_and_deep_decay_bf16(recompute):
+    """Unscaled scores of +-25 and gates near one: rows whose weight sits on keys with a decay bias of -20 to -40 (in
+    log2 units).  The default bf16 path hands the bias from kernel to kernel as fp16 tiles (resolution 2^-6 between 16 and
+    32, 2^-5 up to 64); the recomputing path keeps it in float32.  Both must meet the float64 dense oracle."""
+    from universal_attention_triton_amd import ops
+    bf = torch.bfloat16
+    b, h, r, L, d = 1, 2, 1, 768, 64
+    inp = orc.make_inputs(b, h, r, L, d, 64, dtype=bf, seed=95, gate_mean=2.0)
+    inp["xq"] = (inp["xq"].float() * 8).to(bf)
+    # make the decay deep: similar keys prune one another quickly
+    k = inp["kc"].float().reshape(b, h, L, d)
+    k = k * 0.5 + k.mean(dim=2, keepdim=True) * 4
+    inp["kc"] = (k / k.norm(dim=-1, keepdim=True)).reshape(inp["kc"].shape).to(bf)
+    O_ref, lse_ref, g_ref = dense_reference(inp)
+    bias = orc.dense_bias(inp["kc"].double().reshape(b, h, L, d), inp["static_src"].double().reshape(b, h, L),
+                          inp["static_dest"].double().reshape(b, h, L))
+    scores = torch.einsum("bhsd,bhrtd->bhrst", inp["kc"].double().reshape(b, h, L, d), inp["xq"].double())
+    causal = torch.ones(L, L, dtype=torch.bool).triu()                    # [s, t]: s <= t
+    w = torch.softmax((scores + bias.unsqueeze(2)).masked_fill(~causal, float("-inf")), dim=-2)
+    top = w.argmax(dim=-2)                                                # key carrying the most weight per query
+    top_bias = bias.unsqueeze(2).expand_as(w).gather(-2, top.unsqueeze(-2)).squeeze(-2) / 0.6931471805599453
+    print("scores up to %.1f, bias of the heaviest key: median %.1f, min %.1f (log2 units)"
+          % (float(scores.abs().max()), float(top_bias.median()), float(top_bias.min())), flush=True)
+    assert float(scores.abs().max()) > 15 and float(top_bias.min()) < -20
+    dev = {k_: v.cuda() for k_, v in inp.items()}
+    a = [dev[k_] for k_ in NAMES]
+    O, lse, state = ops.fused_forward(*a, keep_state=True, recompute=recompute)
+    grads = ops.fused_backward(*a, O, lse, dev["dO"], state=state, recompute=recompute)
+    torch.cuda.synchronize()
+    assert rel_err(O, O_ref) <= TOL[bf], rel_err(O, O_ref)
+    _table("large scores recompute=%s" % recompute, grads, g_ref, TOL[bf])

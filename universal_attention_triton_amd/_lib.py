@@ -40,6 +40,7 @@ P = ctypes.POINTER
 SIGNATURES = {
     "ua_version": (c_int, []),
     "ua_last_error": (ctypes.c_char_p, []),
+    "ua_source_hash": (ctypes.c_char_p, []),
     "ua_workspace_bytes": (c_size_t, [P(UaDesc), c_int]),
     "ua_fwd": (c_int, [P(UaDesc), P(UaRows), P(UaRows), P(UaRows), c_void_p, c_void_p, P(UaChunked), c_void_p, c_void_p, c_size_t, c_void_p]),
     "ua_bwd": (c_int, [P(UaDesc), P(UaRows), P(UaRows), P(UaRows), c_void_p, c_void_p, P(UaChunked), P(UaChunked), c_void_p,
@@ -85,6 +86,14 @@ def load():
             for name, (res, args) in SIGNATURES.items():
                 fn = getattr(lib, name)
                 fn.restype, fn.argtypes = res, args
+            # a library older than the sources beside it would silently test and benchmark other code
+            csrc = os.path.join(HERE, "csrc")
+            if os.path.isdir(csrc) and os.environ.get("UA_ALLOW_STALE_LIB") != "1":
+                from .build import source_hash
+                built, now = lib.ua_source_hash().decode(), source_hash()
+                if built != now:
+                    raise UaError("%s was built from other sources (hash %s, sources now %s): rebuild it with "
+                                  "`python -m universal_attention_triton_amd.build`" % (LIB_PATH, built, now))
             _lib = lib
             env_file = os.environ.get("UA_TUNE_FILE")
     if env_file and os.path.exists(env_file) and not getattr(load, "_env_done", False):

@@ -12,6 +12,20 @@ UNITS = ["ua_capi", "ua_inst_fwd", "ua_inst_bwd", "ua_inst_aff"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-honor-nans", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
+def source_hash():
+    """Hash of everything the library is compiled from; the library reports the hash it was built with
+    (ua_source_hash) and _lib.load refuses a library whose sources have changed since."""
+    import hashlib
+    h = hashlib.sha256()
+    files = sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hip", ".hpp", ".inc")))
+    files.append(os.path.join(HERE, "..", "include", "ua.h"))
+    for f in files:
+        h.update(os.path.basename(f).encode())
+        with open(f, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
 def _compile(unit, objdir, extra):
     src, obj = os.path.join(CSRC, unit + ".hip"), os.path.join(objdir, unit + ".o")
     cmd = ["hipcc", *FLAGS, *extra, "-c", src, "-o", obj]
@@ -25,8 +39,9 @@ def _compile(unit, objdir, extra):
 def build(verbose=False, extra=()):
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
+    tag = ['-DUA_SOURCE_HASH="%s"' % source_hash()]
     with concurrent.futures.ThreadPoolExecutor(max_workers=len(UNITS)) as ex:
-        results = list(ex.map(lambda u: _compile(u, objdir, list(extra)), UNITS))
+        results = list(ex.map(lambda u: _compile(u, objdir, list(extra) + (tag if u == "ua_capi" else [])), UNITS))
     objs = [o for o, _ in results]
     res = subprocess.run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs], capture_output=True, text=True)
     if res.returncode != 0:

@@ -307,7 +307,7 @@ __global__ void __launch_bounds__(256) k_bwd_finish(const float* __restrict__ dK
       float kd = 0.f;
       for (int r = 0; r < RS; ++r) kd += dKdacc[(((long)z * RS + r) * Lp + t) * D + c];
       // the packed keys are row-major in chunked mode and tiled (nat_off) in fused mode
-      const long ik = !tiled ? i : (D == 64 ? nat_off<64>(z, Lp, t, c) : nat_off<128>(z, Lp, t, c));
+      const long ik = !tiled ? i : (D == 64 ? nat_off<64>(z, Lp, t, c) : (D == 128 ? nat_off<128>(z, Lp, t, c) : nat_off<256>(z, Lp, t, c)));
       dot += kd * (float)Kp[ik];
       // RK > 1: so does the row side, and dV
       float kr = 0.f, vr = 0.f;

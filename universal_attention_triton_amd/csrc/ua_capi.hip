@@ -43,11 +43,17 @@ struct Layout {
   int key_parts;    // key side of the backward: sweeps per kv head, each over r / key_parts query groups (see make_layout)
 };
 
+// head dims are zero-padded to 64, 128 or 256 (as the reference's second-generation kernel pads to a power of two up to
+// 256, Universal_Attention/triton/universal_attention_kernel_opt.py:441-456)
+int padded_dim(int d) { return d <= 64 ? 64 : (d <= 128 ? 128 : 256); }
+
 int check_desc(const ua_desc* d, bool chunked) {
   if (!d) return fail(UA_EINVAL, "null descriptor");
   if (d->dtype != UA_F32 && d->dtype != UA_BF16) return fail(UA_EINVAL, "dtype %d: only UA_F32 and UA_BF16 are supported", d->dtype);
   if (d->b < 1 || d->h < 1 || d->r < 1 || d->L < 1 || d->d < 1) return fail(UA_EINVAL, "b,h,r,L,d must be positive (got %d,%d,%d,%d,%d)", d->b, d->h, d->r, d->L, d->d);
-  if (d->d > 128) return fail(UA_EINVAL, "head dim %d > 128 is not supported", d->d);
+  if (d->d > 256) return fail(UA_EINVAL, "head dim %d > 256 is not supported", d->d);
+  if (d->d > 128 && (chunked || d->dtype != UA_BF16 || (d->flags & UA_FLAG_RECOMPUTE)))
+    return fail(UA_EINVAL, "head dim %d > 128: only the bf16 fused operator without UA_FLAG_RECOMPUTE", d->d);
   if ((long)d->b * d->h * d->r > 65535) return fail(UA_EINVAL, "b*h*r = %ld exceeds the grid limit 65535", (long)d->b * d->h * d->r);
   if (chunked) {
     const int c = d->chunk;
@@ -67,7 +73,7 @@ std::map<TuneKey, int> g_tune;
 int l_bucket(int L) { int b = 0; while ((128 << b) < L) ++b; return b; }
 int z_bucket(long z) { int b = 0; while ((1L << b) < z) ++b; return b; }
 TuneKey tune_key(const ua_desc& d, int slot) {
-  return TuneKey(slot, d.dtype, d.d <= 64 ? 64 : 128, d.r, l_bucket(d.L), z_bucket((long)d.b * d.h));
+  return TuneKey(slot, d.dtype, padded_dim(d.d), d.r, l_bucket(d.L), z_bucket((long)d.b * d.h));
 }
 bool known_slot(int slot) {
   return slot == UA_TUNE_FWD_RECOMPUTE || slot == UA_TUNE_CARRY || slot == UA_TUNE_FWD_TILES || slot == UA_TUNE_BWD_PARTS ||
@@ -79,11 +85,11 @@ int divisor_index(int r, int p) { int i = 0; for (int q = 1; q < p; ++q) i += r 
 int n_variants(const ua_desc& d, int slot) {
   const bool bf = d.dtype == UA_BF16;
   switch (slot) {
-    case UA_TUNE_FWD_RECOMPUTE: return ua::fwd_fused_variants(d.dtype, d.d <= 64 ? 64 : 128);
+    case UA_TUNE_FWD_RECOMPUTE: return ua::fwd_fused_variants(d.dtype, padded_dim(d.d));
     case UA_TUNE_CARRY: return bf ? 2 : 1;
-    case UA_TUNE_FWD_TILES: return bf ? (d.r % 2 == 0 ? 2 : 3) : 1;
+    case UA_TUNE_FWD_TILES: return bf ? (d.d > 128 ? 1 : (d.r % 2 == 0 ? 2 : 3)) : 1;     // above 128: 16 queries per wave only
     case UA_TUNE_BWD_PARTS: return bf ? n_divisors(d.r) : 1;
-    case UA_TUNE_BWD_QUERIES: return bf ? 2 : 1;
+    case UA_TUNE_BWD_QUERIES: return bf && d.d <= 128 ? 2 : 1;
   }
   return 1;
 }
@@ -144,7 +150,7 @@ int tuned_variant(const ua_desc& d, int slot) {
 
 Layout make_layout(const ua_desc& d, bool chunked, int force_parts = 0) {
   Layout l{};
-  l.D = d.d <= 64 ? 64 : 128;
+  l.D = padded_dim(d.d);
   l.Lp = (int)align_up((size_t)d.L, 128);
   l.nT = l.Lp / 16;     // carries are kept per 16-query tile
   l.nch = chunked ? d.L / d.chunk : 1;
@@ -237,7 +243,10 @@ hipError_t pack_t(int D, const ua::RowsView& x, void* nat, void* tr, int d, int 
                   hipStream_t s, const int* masked_nz, int c) {
   const int tiled = tr_mode != TR_PERM16;      // the fused kernels read tiled working tensors, the chunked ones row-major
   const int vec = vector_ok(x, sizeof(T), d) ? 1 : 0;
-  if (D == 64) hipLaunchKernelGGL((ua::k_pack<T, 64>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp, tr_mode, tiled, vec, norm2, masked_nz, c);
+  if (D == 256) {
+    if constexpr (sizeof(T) == 2) hipLaunchKernelGGL((ua::k_pack<T, 256>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp, tr_mode, tiled, vec, norm2, masked_nz, c);
+    else return hipErrorInvalidValue;
+  } else if (D == 64) hipLaunchKernelGGL((ua::k_pack<T, 64>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp, tr_mode, tiled, vec, norm2, masked_nz, c);
   else hipLaunchKernelGGL((ua::k_pack<T, 128>), dim3(Lp / 32, Z), dim3(256), 0, s, x, (T*)nat, (T*)tr, d, L, Lp, tr_mode, tiled, vec, norm2, masked_nz, c);
   return hipGetLastError();
 }
@@ -470,7 +479,11 @@ int tune_slot(const ua_desc& d, int slot, hipStream_t s, F launch) {
 
 extern "C" {
 
-int ua_version(void) { return 1; }
+int ua_version(void) { return 2; }
+#ifndef UA_SOURCE_HASH
+#define UA_SOURCE_HASH "unknown"
+#endif
+const char* ua_source_hash(void) { return UA_SOURCE_HASH; }
 const char* ua_last_error(void) { return g_err; }
 
 size_t ua_workspace_bytes(const ua_desc* desc, int op) {
@@ -724,6 +737,7 @@ AffLayout make_aff_layout(const ua_desc& d) {
 int aff_prepare(const ua_desc* desc, const ua_rows* k, const void* src, const void* dest, void* ws, size_t ws_bytes, bool bwd,
                 AffLayout& l, hipStream_t s) {
   if (int e = check_desc(desc, false)) return e;
+  if (desc->d > 128) return fail(UA_EINVAL, "head dim %d > 128 is not supported by the stand-alone bias", desc->d);
   l = make_aff_layout(*desc);
   if (!k || !k->ptr || !src || !dest) return fail(UA_EINVAL, "null input tensor");
   if (!ws) return fail(UA_EWORKSPACE, "null workspace");
@@ -748,6 +762,7 @@ int aff_prepare(const ua_desc* desc, const ua_rows* k, const void* src, const vo
 
 size_t ua_affinity_workspace_bytes(const ua_desc* desc, int backward) {
   if (check_desc(desc, false) != UA_OK) return 0;
+  if (desc->d > 128) { fail(UA_EINVAL, "head dim %d > 128 is not supported by the stand-alone bias", desc->d); return 0; }
   const AffLayout l = make_aff_layout(*desc);
   return backward ? l.total : l.fwd_end;
 }

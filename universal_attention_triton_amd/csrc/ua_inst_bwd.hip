@@ -42,6 +42,8 @@ template __global__ void k_bwd_keys2<bf16, 64, 2, false, false, true>(BwdArgs<bf
 template __global__ void k_bwd_keys2<bf16, 64, 2, true, false, true>(BwdArgs<bf16>);
 template __global__ void k_bwd_keys2<bf16, 128, 2, false, false, true>(BwdArgs<bf16>);
 template __global__ void k_bwd_keys2<bf16, 128, 2, true, false, true>(BwdArgs<bf16>);
+template __global__ void k_bwd_keys2<bf16, 256, 2, false, false, true>(BwdArgs<bf16>);
+template __global__ void k_bwd_keys2<bf16, 256, 2, true, false, true>(BwdArgs<bf16>);
 template __global__ void k_bwd_keys2<bf16, 64, 2, false, true, true>(BwdArgs<bf16>);
 template __global__ void k_bwd_keys2<bf16, 64, 2, true, true, true>(BwdArgs<bf16>);
 template __global__ void k_bwd_keys2<bf16, 128, 2, false, true, true>(BwdArgs<bf16>);
@@ -72,7 +74,15 @@ static hipError_t bwd_nw(const BwdArgsV& v, int Zk, int cols, hipStream_t s) {
   if (v.c > 32) return bwd_t<T, D, 2, true>(v, Zk, s);
   return bwd_t<T, D, 1, true>(v, Zk, s);
 }
+// head dims above 128: merged bf16 operator with tile exchange only
+static hipError_t bwd_keys_256(const BwdArgsV& v, int Zk, hipStream_t s) {
+  if (!v.dS_st || v.chunked) return hipErrorInvalidValue;
+  const BwdArgs<bf16> a = typed<bf16>(v);
+  return v.R / a.key_parts > 1 ? bwd2_mr<bf16, 256, 2, true, false, true>(a, v.Lp, Zk * a.key_parts, s)
+                               : bwd2_mr<bf16, 256, 2, false, false, true>(a, v.Lp, Zk * a.key_parts, s);
+}
 hipError_t launch_bwd_keys(int dtype, int D, const BwdArgsV& a, int Zk, int cols, hipStream_t s) {
+  if (D == 256) return (dtype == 1 && !cols) ? bwd_keys_256(a, Zk, s) : hipErrorInvalidValue;
   if (dtype == 1) return D == 64 ? bwd_nw<bf16, 64>(a, Zk, cols, s) : bwd_nw<bf16, 128>(a, Zk, cols, s);
   return D == 64 ? bwd_nw<float, 64>(a, Zk, cols, s) : bwd_nw<float, 128>(a, Zk, cols, s);
 }
@@ -93,6 +103,7 @@ static hipError_t bwdq_t(const BwdArgsV& v, void* dq, int d, int Zk, hipStream_t
   return hipGetLastError();
 }
 hipError_t launch_bwd_queries(int dtype, int D, const BwdArgsV& a, void* dq, int d, int Zk, hipStream_t s) {
+  if (D == 256) return hipErrorInvalidValue;   // the recomputing query side stops at 128
   if (dtype == 1) return D == 64 ? bwdq_t<bf16, 64, 2>(a, dq, d, Zk, s) : bwdq_t<bf16, 128, 2>(a, dq, d, Zk, s);
   return D == 64 ? bwdq_t<float, 64, 1>(a, dq, d, Zk, s) : bwdq_t<float, 128, 1>(a, dq, d, Zk, s);
 }
@@ -100,12 +111,14 @@ hipError_t launch_bwd_queries(int dtype, int D, const BwdArgsV& a, void* dq, int
 template __global__ void k_bwd_queries3<bf16, 64, 2, 1>(BwdArgs<bf16>, bf16*, int);
 template __global__ void k_bwd_queries3<bf16, 128, 2, 1>(BwdArgs<bf16>, bf16*, int);
 template __global__ void k_bwd_queries3<bf16, 64, 2, 2>(BwdArgs<bf16>, bf16*, int);
+template __global__ void k_bwd_queries3<bf16, 256, 2, 1>(BwdArgs<bf16>, bf16*, int);
 template __global__ void k_bwd_queries3<bf16, 128, 2, 2>(BwdArgs<bf16>, bf16*, int);
 hipError_t launch_bwd_queries_from_tiles(int D, const BwdArgsV& v, void* dq, int d, int Zq, hipStream_t s, int variant) {
   const BwdArgs<bf16> a = typed<bf16>(v);
   const dim3 grid(v.Lp / 128, Zq);
 #define UA_Q3(D_, HV_) hipLaunchKernelGGL((k_bwd_queries3<bf16, D_, 2, HV_>), grid, dim3(512), 0, s, a, (bf16*)dq, d)
-  if (variant == 1) { if (D == 64) UA_Q3(64, 2); else UA_Q3(128, 2); }
+  if (D == 256) UA_Q3(256, 1);              // steps of 32 keys only: a stage of 64 keys would not fit twice
+  else if (variant == 1) { if (D == 64) UA_Q3(64, 2); else UA_Q3(128, 2); }
   else { if (D == 64) UA_Q3(64, 1); else UA_Q3(128, 1); }
 #undef UA_Q3
   return hipGetLastError();

@@ -24,6 +24,7 @@ static hipError_t carry_t(const void* Kp, const float* lsrc, const float* ldest,
   if (tiled && Bt && sizeof(T) == 2 && variant == 1)
     hipLaunchKernelGGL((k_carry2<T, D, NST, true, true, 4>), dim3(Lp / 64, Zk), dim3(256), 0, s, (const T*)Kp, lsrc, ldest, C, Lp, knorm2, qnorm2, R, reach, (_Float16*)Bt);
   else if (tiled && Bt && sizeof(T) == 2) hipLaunchKernelGGL((k_carry2<T, D, NST, true, true>), dim3(Lp / 128, Zk), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, C, Lp, knorm2, qnorm2, R, reach, (_Float16*)Bt);
+  else if constexpr (D == 256) return hipErrorInvalidValue;
   else if (tiled) hipLaunchKernelGGL((k_carry2<T, D, NST, true, false>), dim3(Lp / 128, Zk), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, C, Lp, knorm2, qnorm2, R, reach, none);
   else hipLaunchKernelGGL((k_carry2<T, D, NST, false, false>), dim3(Lp / 128, Zk), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, C, Lp, knorm2, qnorm2, R, reach, none);
   hipError_t e = hipGetLastError();
@@ -37,6 +38,7 @@ hipError_t launch_carry(int dtype, int D, const void* Kp, const float* lsrc, con
                         int tiled, const float* knorm2, const float* qnorm2, int R, int* reach, int* minkey, hipStream_t s,
                         void* Bt, int variant) {
 #define UA_ARGS Kp, lsrc, ldest, C, Lp, Zk, tiled, knorm2, qnorm2, R, reach, minkey, s, Bt, variant
+  if (D == 256) return (dtype == 1 && tiled && Bt) ? carry_t<bf16, 256>(UA_ARGS) : hipErrorInvalidValue;   // bias tiles only
   if (dtype == 1) return D == 64 ? carry_t<bf16, 64>(UA_ARGS) : carry_t<bf16, 128>(UA_ARGS);
   return D == 64 ? carry_t<float, 64>(UA_ARGS) : carry_t<float, 128>(UA_ARGS);
 #undef UA_ARGS
@@ -50,6 +52,7 @@ hipError_t launch_carry(int dtype, int D, const void* Kp, const float* lsrc, con
 #define UA_INST2(T, D, NST, NW, CH, BI) UA_INST3(T, D, NST, NW, CH, BI, 1)
 #define UA_INST(T, D, NST, NW, CH) UA_INST2(T, D, NST, NW, CH, false)
 UA_INST3(bf16, 64, 1, 8, false, true, 2) UA_INST3(bf16, 128, 1, 8, false, true, 2) UA_INST3(bf16, 64, 1, 8, false, true, 4) UA_INST3(bf16, 128, 1, 8, false, true, 4)
+UA_INST3(bf16, 256, 1, 8, false, true, 2) UA_INST3(bf16, 256, 1, 8, false, true, 4) UA_INST2(bf16, 256, 1, 8, false, true)
 UA_INST2(bf16, 64, 1, 8, false, true) UA_INST2(bf16, 128, 1, 8, false, true) UA_INST2(bf16, 64, 1, 4, false, true) UA_INST2(bf16, 128, 1, 4, false, true)
 template __global__ void k_fwd_fused3<64, 1>(const bf16*, const bf16*, const bf16*, bf16*, float*, float*, const int*, const int*, int, int, int, int, const _Float16*);
 template __global__ void k_fwd_fused3<64, 2>(const bf16*, const bf16*, const bf16*, bf16*, float*, float*, const int*, const int*, int, int, int, int, const _Float16*);
@@ -84,7 +87,8 @@ static hipError_t fused_bi(int variant, const void* Qp, const void* Kp, const vo
                            const float* C, void* O, float* lse, float* lse2, const int* reach, const int* minkey, int R, int L,
                            int Lp, int d, int Zq, hipStream_t s, const void* Bt) {
   using T = bf16;
-  if (variant == 0) {
+  if constexpr (D == 256) variant = 1;       // 16 queries per wave: the accumulators of a 32-query block do not fit
+  if constexpr (D != 256) if (variant == 0) {
 #define UA_F3(RB_)                                                                                                          \
   hipLaunchKernelGGL((k_fwd_fused3<D, RB_>), dim3((Lp / 32 + 8 / RB_ - 1) / (8 / RB_), Zq / RB_), dim3(512), 0, s, (const T*)Qp, \
                      (const T*)Kp, (const T*)VT, (T*)O, lse, lse2, reach, minkey, R, L, Lp, d, (const _Float16*)Bt)
@@ -100,10 +104,10 @@ static hipError_t fused_bi(int variant, const void* Qp, const void* Kp, const vo
                      (const _Float16*)Bt)
   if (R % 4 == 0) UA_SHARED(4);
   else if (R % 2 == 0) UA_SHARED(2);
-  else if (variant == 1)
+  else if (variant == 1 || D == 256)
     hipLaunchKernelGGL((k_fwd_fused2<T, D, 1, 8, false, true>), dim3(Lp / 128, Zq), dim3(512), 0, s, (const T*)Qp, (const T*)Kp,
                        (const T*)VT, lsrc, ldest, C, (T*)O, lse, lse2, reach, minkey, R, L, Lp, d, ChunkOut<T>{}, (const _Float16*)Bt);
-  else
+  else if constexpr (D != 256)
     hipLaunchKernelGGL((k_fwd_fused2<T, D, 1, 4, false, true>), dim3(Lp / 64, Zq), dim3(256), 0, s, (const T*)Qp, (const T*)Kp,
                        (const T*)VT, lsrc, ldest, C, (T*)O, lse, lse2, reach, minkey, R, L, Lp, d, ChunkOut<T>{}, (const _Float16*)Bt);
 #undef UA_SHARED
@@ -131,6 +135,7 @@ hipError_t launch_fwd_fused(int dtype, int D, int variant, const void* Qp, const
                             const int* reach, const int* minkey, int R, int L, int Lp, int d, int Zq, hipStream_t s,
                             const void* Bt) {
 #define UA_ARGS Qp, Kp, VT, lsrc, ldest, C, O, lse, lse2, reach, minkey, R, L, Lp, d, Zq, s
+  if (D == 256) return (dtype == 1 && Bt) ? fused_bi<256>(variant, UA_ARGS, Bt) : hipErrorInvalidValue;
   if (dtype == 1 && Bt) return D == 64 ? fused_bi<64>(variant, UA_ARGS, Bt) : fused_bi<128>(variant, UA_ARGS, Bt);
   if (dtype == 1) return D == 64 ? fused_v<bf16, 64>(variant, UA_ARGS) : fused_v<bf16, 128>(variant, UA_ARGS);
   return D == 64 ? fused_t<float, 64, 1, 8>(UA_ARGS) : fused_t<float, 128, 1, 8>(UA_ARGS);
