@@ -109,19 +109,29 @@ size_t ua_workspace_bytes(const ua_desc* desc, int op);
 /* Chunked forward: replaces _universal_attention_fwd
  * (Universal_Attention/triton/universal_attention_kernel.py:192-239) and the torch operator
  * UniversalAttention.forward (universal_attention_autograd.py:9-38).
- * static_src, static_dest: contiguous [b,h,L].  denom: contiguous [b,h,r,L,n] in desc->dtype. */
+ * static_src, static_dest: contiguous [b,h,L].  denom: contiguous [b,h,r,L,n] in desc->dtype.
+ * lse2_out: NULL, or [b*h*r][L/chunk][Lp] float (Lp = L rounded up to 128) that receives the per-chunk normalisers in
+ * float32 (log2 units; `denom` in bf16 is too coarse for the backward): the one part of the forward state that is
+ * expensive to rebuild, 1/(d+1) of the size of `out`.  Hand it to ua_bwd as lse2_in. */
 int ua_fwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
-           const void* static_dest, const ua_chunked* out, void* denom, void* ws, size_t ws_bytes, ua_stream_t stream);
+           const void* static_dest, const ua_chunked* out, void* denom, float* lse2_out, void* ws, size_t ws_bytes,
+           ua_stream_t stream);
 
 /* Chunked backward: replaces _universal_attention_bwd (universal_attention_kernel.py:793-862) and
  * UniversalAttention.backward (universal_attention_autograd.py:47-99).
  * out: the forward's result; g_out: same indexing; g_denom: contiguous float32 [b,h,r,L,n].
  * Gradients are written contiguous: dkc, dvc [b,h,L,d]; dxq [b,h,r,L,d]; dsrc, ddest [b,h,L].
  * fwd_state: NULL, or the workspace ua_fwd ran on for the same inputs and flags, contents intact (skips the recompute;
- * the backward rewrites parts of it with the same values). */
+ * the backward rewrites parts of it with the same values).
+ * delta: NULL, or what ua_merge_bwd left when it produced exactly these (g_out, g_denom) from `out`
+ * ([b*h*r][L/chunk][Lp] float, Lp = L rounded up to 128, zero beyond L): the backward then skips its own pass over
+ * out and g_out (8.6 GB at b=1 h=32 L=8192 d=128).  Needs UA_FLAG_SKIP_MASKED and a chunk that is a multiple of 64.
+ * lse2_in: NULL, or what ua_fwd wrote to lse2_out: without fwd_state the backward then repacks the inputs and
+ * rebuilds the decay carries but does not run the forward kernel again for the normalisers. */
 int ua_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
            const void* static_dest, const ua_chunked* out, const ua_chunked* g_out, const float* g_denom, void* dkc,
-           void* dvc, void* dxq, void* dsrc, void* ddest, void* fwd_state, void* ws, size_t ws_bytes, ua_stream_t stream);
+           void* dvc, void* dxq, void* dsrc, void* ddest, const float* delta, const float* lse2_in, void* fwd_state, void* ws,
+           size_t ws_bytes, ua_stream_t stream);
 
 /* Fused forward: the chunked operator followed by SMVecMatMul (universal_attention_autograd.py:278-283)
  * without materialising the per-chunk tensor; same role as the reference's second-generation
@@ -156,9 +166,12 @@ int ua_fused_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, cons
  * vec: contiguous [rows, n] in `dtype`; result contiguous [rows, d]. */
 int ua_merge_fwd(int dtype, int64_t rows, int32_t L, int32_t d, int32_t n, const ua_chunked* mat, const void* vec,
                  void* result, ua_stream_t stream);
-/* g: contiguous [rows, d]; d_mat indexed like mat; d_vec contiguous [rows, n] in `dtype`. */
+/* g: contiguous [rows, d]; d_mat indexed like mat; d_vec contiguous [rows, n] in `dtype`.  Slices whose weight is exactly
+ * zero (chunks no key of which a query sees: normaliser -1e12) are not read, by either kernel.
+ * delta: NULL, or [rows / L][n][Lp] float (Lp = L rounded up to 128; the caller zeroes it beyond L) that receives
+ * sum_dd mat d_mat - d_vec per (row, chunk), for ua_bwd. */
 int ua_merge_bwd(int dtype, int64_t rows, int32_t L, int32_t d, int32_t n, const ua_chunked* mat, const void* vec,
-                 const void* g, const ua_chunked* d_mat, void* d_vec, ua_stream_t stream);
+                 const void* g, const ua_chunked* d_mat, void* d_vec, float* delta, ua_stream_t stream);
 
 /* Stand-alone decay bias ("affinity scores"): replaces _affinity_fwd / _affinity_bwd and the AffinityScores wrapper
  * (Universal_Attention/triton/affinity_kernel_opt.py:100-127, :130-423, :425-450).  desc: b, h, L, d, dtype (r, chunk and

@@ -42,16 +42,18 @@ SIGNATURES = {
     "ua_last_error": (ctypes.c_char_p, []),
     "ua_source_hash": (ctypes.c_char_p, []),
     "ua_workspace_bytes": (c_size_t, [P(UaDesc), c_int]),
-    "ua_fwd": (c_int, [P(UaDesc), P(UaRows), P(UaRows), P(UaRows), c_void_p, c_void_p, P(UaChunked), c_void_p, c_void_p, c_size_t, c_void_p]),
+    "ua_fwd": (c_int, [P(UaDesc), P(UaRows), P(UaRows), P(UaRows), c_void_p, c_void_p, P(UaChunked), c_void_p, c_void_p, c_void_p, c_size_t,
+                       c_void_p]),
     "ua_bwd": (c_int, [P(UaDesc), P(UaRows), P(UaRows), P(UaRows), c_void_p, c_void_p, P(UaChunked), P(UaChunked), c_void_p,
-                       c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+                       c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "ua_fused_fwd": (c_int, [P(UaDesc), P(UaRows), P(UaRows), P(UaRows), c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "ua_noalloc_scratch_bytes": (c_size_t, []),
     "ua_fused_fwd_noalloc": (c_int, [P(UaDesc), P(UaRows), P(UaRows), P(UaRows), c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "ua_fused_bwd": (c_int, [P(UaDesc), P(UaRows), P(UaRows), P(UaRows), c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                              c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "ua_merge_fwd": (c_int, [c_int, c_int64, c_int32, c_int32, c_int32, P(UaChunked), c_void_p, c_void_p, c_void_p]),
-    "ua_merge_bwd": (c_int, [c_int, c_int64, c_int32, c_int32, c_int32, P(UaChunked), c_void_p, c_void_p, P(UaChunked), c_void_p, c_void_p]),
+    "ua_merge_bwd": (c_int, [c_int, c_int64, c_int32, c_int32, c_int32, P(UaChunked), c_void_p, c_void_p, P(UaChunked), c_void_p, c_void_p,
+                             c_void_p]),
     "ua_affinity_workspace_bytes": (c_size_t, [P(UaDesc), c_int]),
     "ua_affinity_fwd": (c_int, [P(UaDesc), P(UaRows), c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "ua_affinity_bwd": (c_int, [P(UaDesc), P(UaRows), c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,

@@ -9,7 +9,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libua_hip.so")
 UNITS = ["ua_capi", "ua_inst_fwd", "ua_inst_bwd", "ua_inst_aff"]
 # packed-fp32 instructions are disabled for every device compile of this library
-FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-honor-nans", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-honor-nans", "-Wall", "-Wno-unused-function", "-Wno-unused-variable", "-Wno-unused-but-set-variable", "-Wno-unused-local-typedef", "-Wno-unused-value", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
 def source_hash():
@@ -46,10 +46,9 @@ def build(verbose=False, extra=()):
     res = subprocess.run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs], capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError("link failed:\n" + res.stderr)
-    if verbose:
-        for _, log in results:
-            if log.strip():
-                print(log)
+    for _, log in results:      # compiler warnings are always shown: an uninitialised pointer on the host side faults the GPU
+        if log.strip() and (verbose or "warning:" in log):
+            print(log)
     return LIB
 
 

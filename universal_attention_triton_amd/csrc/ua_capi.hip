@@ -392,7 +392,8 @@ hipError_t delta_t(const ua::RowsView& O, const ua::RowsView& dO, const ua::Rows
 // chunked with a chunk that is not a multiple of 64: key-chunk-stationary kernel over row-major working tensors (atomics);
 // otherwise the key-stationary and query-stationary kernels over tiled working tensors
 int run_bwd_common(const ua_desc& d, const Layout& l, char* wf, char* wb, bool chunked, const void* src, const void* dest, void* dkc,
-                   void* dvc, void* dxq, void* dsrc, void* ddest, hipStream_t s) {
+                   void* dvc, void* dxq, void* dsrc, void* ddest, hipStream_t s, const float* delta_given = nullptr,
+                   const float* lse2_given = nullptr) {
   const bool is_chunked = chunked;
   chunked = is_chunked && !fast_chunk(d);      // from here on: the atomics path
   if (chunked) {
@@ -403,7 +404,7 @@ int run_bwd_common(const ua_desc& d, const Layout& l, char* wf, char* wb, bool c
   ua::BwdArgsV a{};
   a.Kp = wf + l.Kp; a.Vp = wf + l.Vp; a.KT = wf + l.KT; a.Qp = wf + l.Qp; a.QT = l.grad_tiles ? nullptr : wf + l.QT; a.dOp = wb + l.dOp;
   a.dOT = l.grad_tiles ? nullptr : wb + l.dOT; a.lsrc = (const float*)(wf + l.lsrc); a.ldest = (const float*)(wf + l.ldest);
-  a.lse2 = (const float*)(wf + l.lse2); a.delta = (const float*)(wb + l.delta); a.C = (const float*)(wf + l.C);
+  a.lse2 = lse2_given ? lse2_given : (const float*)(wf + l.lse2); a.delta = delta_given ? delta_given : (const float*)(wb + l.delta); a.C = (const float*)(wf + l.C);
   a.reach = (const int*)(wf + l.reach); a.minkey = (const int*)(wf + l.minkey);
   a.dQacc = (float*)(wb + l.dQacc); a.dKdacc = (float*)(wb + l.dKdacc); a.Dsuf = (float*)(wb + l.Dsuf);
   a.dKrow = (float*)(wb + l.dKrow);
@@ -576,7 +577,8 @@ int ua_fused_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, cons
 }
 
 int ua_fwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
-           const void* static_dest, const ua_chunked* out, void* denom, void* ws, size_t ws_bytes, ua_stream_t stream) {
+           const void* static_dest, const ua_chunked* out, void* denom, float* lse2_out, void* ws, size_t ws_bytes,
+           ua_stream_t stream) {
   if (int e = check_desc(desc, true)) return e;
   const Layout l = make_layout(*desc, true);
   if (int e = check_common(kc, vc, xq, static_src, static_dest, ws, ws_bytes, l.fwd_end)) return e;
@@ -584,6 +586,7 @@ int ua_fwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
   char* wf = (char*)ws;
   hipStream_t s = (hipStream_t)stream;
   const ua_desc& d = *desc;
+  float* lse2 = lse2_out ? lse2_out : (float*)(wf + l.lse2);     // the per-chunk normalisers, float32, log2 units
   if (fast_chunk(d)) {
     if (int e = pack_inputs(d, l, false, kc, vc, xq, static_src, static_dest, wf, s)) return e;
     {
@@ -594,26 +597,28 @@ int ua_fwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
     UA_PROF("k_fwd_chunked", s);
     UA_HIP(ua::launch_fwd_chunked2(d.dtype, l.D, wf + l.Qp, wf + l.Kp, wf + l.Vp, wf + l.VT, (const float*)(wf + l.lsrc),
                                    (const float*)(wf + l.ldest), (const float*)(wf + l.C), (const int*)(wf + l.reach),
-                                   (const int*)(wf + l.minkey), out->ptr, denom, (float*)(wf + l.lse2), out->stride_z, out->stride_t,
+                                   (const int*)(wf + l.minkey), out->ptr, denom, lse2, out->stride_z, out->stride_t,
                                    out->stride_d, out->stride_i, d.r, d.L, l.Lp, d.d, d.chunk, l.nch, l.Zq, s));
     return UA_OK;
   }
   if (int e = pack_inputs(d, l, true, kc, vc, xq, static_src, static_dest, wf, s)) return e;
   UA_PROF("k_fwd_chunked", s);
   UA_HIP(ua::launch_fwd_chunked(d.dtype, l.D, wf + l.Qp, wf + l.Kp, wf + l.VT, (const float*)(wf + l.lsrc),
-                                (const float*)(wf + l.ldest), out->ptr, denom, (float*)(wf + l.lse2), out->stride_z, out->stride_t, out->stride_d, out->stride_i, d.r, d.L,
+                                (const float*)(wf + l.ldest), out->ptr, denom, lse2, out->stride_z, out->stride_t, out->stride_d, out->stride_i, d.r, d.L,
                                 l.Lp, d.d, d.chunk, l.nch, l.Zk, s));
   return UA_OK;
 }
 
 int ua_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
            const void* static_dest, const ua_chunked* out, const ua_chunked* g_out, const float* g_denom, void* dkc,
-           void* dvc, void* dxq, void* dsrc, void* ddest, void* fwd_state, void* ws, size_t ws_bytes, ua_stream_t stream) {
+           void* dvc, void* dxq, void* dsrc, void* ddest, const float* delta, const float* lse2_in, void* fwd_state, void* ws,
+           size_t ws_bytes, ua_stream_t stream) {
   if (int e = check_desc(desc, true)) return e;
   const Layout l = make_layout(*desc, true);
   if (int e = check_common(kc, vc, xq, static_src, static_dest, ws, ws_bytes, fwd_state ? l.total - l.fwd_end : l.total)) return e;
   if (!out || !out->ptr || !g_out || !g_out->ptr || !g_denom || !dkc || !dvc || !dxq || !dsrc || !ddest)
     return fail(UA_EINVAL, "null tensor");
+  if (delta && !(desc->flags & UA_FLAG_SKIP_MASKED)) return fail(UA_EINVAL, "a precomputed delta needs UA_FLAG_SKIP_MASKED and a chunk that is a multiple of 64");
   char *wf, *wb;
   if (int e = bwd_bases(l, fwd_state, ws, &wf, &wb)) return e;
   hipStream_t s = (hipStream_t)stream;
@@ -631,10 +636,11 @@ int ua_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
       if (int e = pack_inputs(d, l, false, kc, vc, xq, static_src, static_dest, wf, s)) return e;
       UA_HIP(ua::launch_carry(d.dtype, l.D, wf + l.Kp, (const float*)(wf + l.lsrc), (const float*)(wf + l.ldest), (float*)(wf + l.C), l.Lp,
                               l.Zk, 1, nullptr, nullptr, d.r, (int*)(wf + l.reach), (int*)(wf + l.minkey), s));
-      UA_HIP(ua::launch_fwd_chunked2(d.dtype, l.D, wf + l.Qp, wf + l.Kp, wf + l.Vp, wf + l.VT, (const float*)(wf + l.lsrc),
-                                     (const float*)(wf + l.ldest), (const float*)(wf + l.C), (const int*)(wf + l.reach),
-                                     (const int*)(wf + l.minkey), nullptr, nullptr, (float*)(wf + l.lse2), 0, 0, 0, 0, d.r, d.L, l.Lp,
-                                     d.d, d.chunk, l.nch, l.Zq, s));
+      if (!lse2_in)
+        UA_HIP(ua::launch_fwd_chunked2(d.dtype, l.D, wf + l.Qp, wf + l.Kp, wf + l.Vp, wf + l.VT, (const float*)(wf + l.lsrc),
+                                       (const float*)(wf + l.ldest), (const float*)(wf + l.C), (const int*)(wf + l.reach),
+                                       (const int*)(wf + l.minkey), nullptr, nullptr, (float*)(wf + l.lse2), 0, 0, 0, 0, d.r, d.L, l.Lp,
+                                       d.d, d.chunk, l.nch, l.Zq, s));
     }
     {
       UA_PROF("pack_dO+delta", s);
@@ -642,25 +648,28 @@ int ua_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
       // with UA_FLAG_SKIP_MASKED the flag stays 0: rows before their chunk are neither checked nor packed
       int* nz = (int*)(wb + l.masked_nz);
       int* detect = (d.flags & UA_FLAG_SKIP_MASKED) ? nullptr : nz;
-      if (d.dtype == UA_BF16) UA_HIP(delta_t<ua::bf16>(outv, gv, gdv, none, (float*)(wb + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s, detect, d.chunk));
+      if (delta) { /* ua_merge_bwd left it: neither out nor g_out is read for it */ }
+      else if (d.dtype == UA_BF16) UA_HIP(delta_t<ua::bf16>(outv, gv, gdv, none, (float*)(wb + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s, detect, d.chunk));
       else UA_HIP(delta_t<float>(outv, gv, gdv, none, (float*)(wb + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s, detect, d.chunk));
       UA_HIP(pack(d.dtype, l.D, gv, wb + l.dOp, l.grad_tiles ? nullptr : wb + l.dOT, d.d, d.L, l.Lp, l.Zq * l.nch, TR_PERM32, s, nullptr, nz,
                   d.chunk));
     }
-    return run_bwd_common(d, l, wf, wb, true, static_src, static_dest, dkc, dvc, dxq, dsrc, ddest, s);
+    return run_bwd_common(d, l, wf, wb, true, static_src, static_dest, dkc, dvc, dxq, dsrc, ddest, s, delta, lse2_in);
   }
+  if (delta) return fail(UA_EINVAL, "a precomputed delta needs UA_FLAG_SKIP_MASKED and a chunk that is a multiple of 64");
   if (!fwd_state) {
     // recompute the per-chunk normalisers (the partial outputs themselves are passed in)
     if (int e = pack_inputs(d, l, true, kc, vc, xq, static_src, static_dest, wf, s)) return e;
-    UA_HIP(ua::launch_fwd_chunked(d.dtype, l.D, wf + l.Qp, wf + l.Kp, wf + l.VT, (const float*)(wf + l.lsrc),
-                                  (const float*)(wf + l.ldest), nullptr, nullptr, (float*)(wf + l.lse2), 0, 0, 0, 0, d.r, d.L, l.Lp, d.d, d.chunk, l.nch, l.Zk, s));
+    if (!lse2_in)
+      UA_HIP(ua::launch_fwd_chunked(d.dtype, l.D, wf + l.Qp, wf + l.Kp, wf + l.VT, (const float*)(wf + l.lsrc),
+                                    (const float*)(wf + l.ldest), nullptr, nullptr, (float*)(wf + l.lse2), 0, 0, 0, 0, d.r, d.L, l.Lp, d.d, d.chunk, l.nch, l.Zk, s));
   }
   UA_HIP(ua::launch_carry(d.dtype, l.D, wf + l.Kp, (const float*)(wf + l.lsrc), (const float*)(wf + l.ldest),
                           (float*)(wf + l.C), l.Lp, l.Zk, 0, nullptr, nullptr, 1, nullptr, nullptr, s));
   UA_HIP(pack(d.dtype, l.D, gv, wb + l.dOp, wb + l.dOT, d.d, d.L, l.Lp, l.Zq * l.nch, TR_PERM16, s));
   if (d.dtype == UA_BF16) UA_HIP(delta_t<ua::bf16>(outv, gv, gdv, none, (float*)(wb + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s));
   else UA_HIP(delta_t<float>(outv, gv, gdv, none, (float*)(wb + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s));
-  return run_bwd_common(d, l, wf, wb, true, static_src, static_dest, dkc, dvc, dxq, dsrc, ddest, s);
+  return run_bwd_common(d, l, wf, wb, true, static_src, static_dest, dkc, dvc, dxq, dsrc, ddest, s, nullptr, lse2_in);
 }
 
 // 16-byte accesses to every (row, chunk) slice of a chunked tensor, with d / V lanes per slice (a power of two <= 64)
@@ -691,7 +700,7 @@ int ua_merge_fwd(int dtype, int64_t rows, int32_t L, int32_t d, int32_t n, const
 }
 
 int ua_merge_bwd(int dtype, int64_t rows, int32_t L, int32_t d, int32_t n, const ua_chunked* mat, const void* vec,
-                 const void* g, const ua_chunked* d_mat, void* d_vec, ua_stream_t stream) {
+                 const void* g, const ua_chunked* d_mat, void* d_vec, float* delta, ua_stream_t stream) {
   if (!mat || !mat->ptr || !vec || !g || !d_mat || !d_mat->ptr || !d_vec) return fail(UA_EINVAL, "null tensor");
   if (rows < 1 || L < 1 || d < 1 || n < 1 || n > ua::kMergeMaxN) return fail(UA_EINVAL, "bad merge shape rows=%ld L=%d d=%d n=%d", (long)rows, L, d, n);
   if (dtype != UA_F32 && dtype != UA_BF16) return fail(UA_EINVAL, "dtype %d unsupported", dtype);
@@ -701,7 +710,8 @@ int ua_merge_bwd(int dtype, int64_t rows, int32_t L, int32_t d, int32_t n, const
   const size_t lds = 8 * (size_t)n * sizeof(float);
   hipStream_t s = (hipStream_t)stream;
   const bool vecp = merge_vector_ok(*mat, dtype, d) && merge_vector_ok(*d_mat, dtype, d) && (uintptr_t)g % 16 == 0;
-#define UA_MERGE_BWD(T, VEC) hipLaunchKernelGGL((ua::k_merge_bwd<T, VEC>), grid, dim3(256), lds, s, m, (const T*)vec, (const T*)g, dm, (T*)d_vec, (long)rows, L, d, n)
+  const int Lp = (int)align_up((size_t)L, 128);
+#define UA_MERGE_BWD(T, VEC) hipLaunchKernelGGL((ua::k_merge_bwd<T, VEC>), grid, dim3(256), lds, s, m, (const T*)vec, (const T*)g, dm, (T*)d_vec, (long)rows, L, d, n, delta, Lp)
   if (dtype == UA_BF16) { if (vecp) UA_MERGE_BWD(ua::bf16, true); else UA_MERGE_BWD(ua::bf16, false); }
   else { if (vecp) UA_MERGE_BWD(float, true); else UA_MERGE_BWD(float, false); }
 #undef UA_MERGE_BWD
@@ -805,7 +815,7 @@ int ua_prof_collect(char* buf, size_t cap) {
   for (auto& r : g_prof) {
     float ms = 0.f;
     if (hipEventElapsedTime(&ms, r.e0, r.e1) == hipSuccess) { auto& a = acc[r.name]; a.first += 1; a.second += ms; }
-    hipEventDestroy(r.e0); hipEventDestroy(r.e1);
+    (void)hipEventDestroy(r.e0); (void)hipEventDestroy(r.e1);
   }
   g_prof.clear();
   std::string out;

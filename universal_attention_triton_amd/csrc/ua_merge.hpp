@@ -45,9 +45,12 @@ __global__ void __launch_bounds__(256) k_merge_fwd(ChunkedView mat, const T* __r
 #pragma unroll
     for (int e = 0; e < V; ++e) acc[e] = 0.f;
     for (int i = grp; i < n; i += ng) {
+      const float wi = wts[i];
+      // a chunk whose normaliser is the reference's fill value (-1e12: no key of it is visible to this query) has a
+      // weight of exactly zero: its slice is not read (half of the tensor after the chunked operator)
+      if (wi == 0.f) continue;
       T x[V];
       *reinterpret_cast<uint4*>(x) = *reinterpret_cast<const uint4*>(m + sub * V + i * mat.si);
-      const float wi = wts[i];
 #pragma unroll
       for (int e = 0; e < V; ++e) acc[e] += wi * (float)x[e];
     }
@@ -65,14 +68,18 @@ __global__ void __launch_bounds__(256) k_merge_fwd(ChunkedView mat, const T* __r
   }
   for (int dd = lane; dd < d; dd += 64) {
     float acc = 0.f;
-    for (int i = 0; i < n; ++i) acc += wts[i] * (float)m[dd * mat.sd + i * mat.si];
+    for (int i = 0; i < n; ++i)
+      if (wts[i] != 0.f) acc += wts[i] * (float)m[dd * mat.sd + i * mat.si];
     res[row * d + dd] = cvt<T>(acc);
   }
 }
 
 template <class T, bool VEC>
+// delta (optional): [rows / L][n][Lp] float receives sum_dd mat[dd, i] d_mat[dd, i] - d_vec[i] = w_i (g . result), what
+// the chunked operator's backward needs first from exactly these gradients (rows of length Lp, written for t < L)
 __global__ void __launch_bounds__(256) k_merge_bwd(ChunkedView mat, const T* __restrict__ vec, const T* __restrict__ g,
-                                                   ChunkedView dmat, T* __restrict__ dvec, long rows, int L, int d, int n) {
+                                                   ChunkedView dmat, T* __restrict__ dvec, long rows, int L, int d, int n,
+                                                   float* __restrict__ delta, int Lp) {
   extern __shared__ __align__(16) char smem[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   float* wts = reinterpret_cast<float*>(smem) + wave * 2 * n;
@@ -97,10 +104,15 @@ __global__ void __launch_bounds__(256) k_merge_bwd(ChunkedView mat, const T* __r
       float acc = 0.f;
       if (i < n) {
         T x[V], y[V];
-        *reinterpret_cast<uint4*>(x) = *reinterpret_cast<const uint4*>(m + sub * V + i * mat.si);
         const float wi = wts[i];
+        // zero weight (see k_merge_fwd): the slice's gradient is zero whatever it holds, and so is its share of d_vec
+        if (wi != 0.f) {
+          *reinterpret_cast<uint4*>(x) = *reinterpret_cast<const uint4*>(m + sub * V + i * mat.si);
 #pragma unroll
-        for (int e = 0; e < V; ++e) { acc += gf[e] * (float)x[e]; y[e] = cvt<T>(gf[e] * wi); }
+          for (int e = 0; e < V; ++e) acc += gf[e] * (float)x[e];
+        }
+#pragma unroll
+        for (int e = 0; e < V; ++e) y[e] = cvt<T>(gf[e] * wi);
         *reinterpret_cast<uint4*>(dm + sub * V + i * dmat.si) = *reinterpret_cast<const uint4*>(y);
       }
       for (int k = 1; k < lpr; k <<= 1) acc += __shfl_xor(acc, k, 64);
@@ -115,7 +127,8 @@ __global__ void __launch_bounds__(256) k_merge_bwd(ChunkedView mat, const T* __r
   // d_w[i] = sum_dd g[dd] * mat[dd, i]
   for (int i = 0; i < n; ++i) {
     float acc = 0.f;
-    for (int dd = lane; dd < d; dd += 64) acc += (float)gr[dd] * (float)m[dd * mat.sd + i * mat.si];
+    if (wts[i] != 0.f)
+      for (int dd = lane; dd < d; dd += 64) acc += (float)gr[dd] * (float)m[dd * mat.sd + i * mat.si];
 #pragma unroll
     for (int k = 32; k >= 1; k >>= 1) acc += __shfl_xor(acc, k, 64);
     if (lane == 0) dw[i] = acc;
@@ -127,6 +140,10 @@ __global__ void __launch_bounds__(256) k_merge_bwd(ChunkedView mat, const T* __r
 #pragma unroll
   for (int k = 32; k >= 1; k >>= 1) dot += __shfl_xor(dot, k, 64);
   for (int i = lane; i < n; i += 64) dvec[row * n + i] = cvt<T>((dw[i] - dot) * wts[i]);
+  if (delta) {
+    float* dl = delta + (row / L) * (long)n * Lp + (row % L);
+    for (int i = lane; i < n; i += 64) dl[(long)i * Lp] = wts[i] * dot;
+  }
 }
 
 }  // namespace ua

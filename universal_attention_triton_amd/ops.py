@@ -101,8 +101,10 @@ def _prep(kc, vc, xq, static_src, static_dest):
 
 def chunked_forward(kc, vc, xq, static_src, static_dest, keep_state=False, recompute=False):
     """-> out [b,h,r,l,d,n] (chunk-major storage, returned as a permuted view), denom [b,h,r,l,n], state
-    keep_state: return the forward state (the workspace, ua_workspace_bytes(UA_OP_FWD) bytes) for chunked_backward;
-    otherwise state is None and the backward rebuilds it.
+    keep_state: what chunked_backward gets from the forward.  False: nothing (it rebuilds everything, including a
+    second run of the forward kernel).  "normalisers": the per-chunk normalisers in float32 (1/(d+1) of the size of
+    `out`; the backward then only repacks the inputs and rebuilds the decay carries).  True: the whole forward state (the
+    workspace, ua_workspace_bytes(UA_OP_FWD) bytes).
     recompute: the flags of the state must match the backward's (pass the same value to chunked_backward)."""
     kc, vc, xq, src, dest, gflag = _prep(kc, vc, xq, static_src, static_dest)
     lib = _lib.load()
@@ -115,10 +117,13 @@ def chunked_forward(kc, vc, xq, static_src, static_dest, keep_state=False, recom
     out = store.permute(0, 1, 2, 4, 5, 3)
     denom = torch.empty(b, h, r, L, n, dtype=xq.dtype, device=xq.device)
     _, oc = _chunked(out)
+    lse2 = None
+    if keep_state == "normalisers":
+        lse2 = torch.empty(b * h * r * n * (-(-L // 128) * 128), dtype=torch.float32, device=xq.device)
     _lib.check(lib.ua_fwd(ctypes.byref(desc), ctypes.byref(_rows_k(kc)), ctypes.byref(_rows_k(vc)), ctypes.byref(_rows_q(xq)),
-                          src.data_ptr(), dest.data_ptr(), ctypes.byref(oc), denom.data_ptr(), ws.data_ptr(), ws.numel(), _stream()),
-               "ua_fwd")
-    return out, denom, (ws if keep_state else None)
+                          src.data_ptr(), dest.data_ptr(), ctypes.byref(oc), denom.data_ptr(),
+                          lse2.data_ptr() if lse2 is not None else None, ws.data_ptr(), ws.numel(), _stream()), "ua_fwd")
+    return out, denom, (lse2 if lse2 is not None else (ws if keep_state else None))
 
 
 def _gate_grads(b, h, L, src, static_src, static_dest):
@@ -126,15 +131,46 @@ def _gate_grads(b, h, L, src, static_src, static_dest):
     return dsrc, torch.empty_like(dsrc)
 
 
+# What merge_backward leaves for a chunked_backward that receives exactly the gradients it produced: weak references
+# to the two gradient tensors (the entry dies with them) and the per-(row, chunk) term delta.
+_merge_handoff = {}
+
+
+def _delta_from_merge(out, g_out, g_denom, L, n):
+    item = _merge_handoff.pop("last", None)
+    if item is None:
+        return None
+    w_mat, w_vec, out_id, v_mat, v_vec, delta = item
+    # the gradients: the very objects (an entry dies with them, so a new tensor at an old address cannot match), unmodified;
+    # `out`: alive since the forward, so the tensor merged at that address with this shape and these strides was this one
+    if w_mat() is g_out and w_vec() is g_denom and out_id == (out.data_ptr(), tuple(out.shape), tuple(out.stride()), out._version) \
+            and g_out._version == v_mat and g_denom._version == v_vec and delta.shape[1] == n and delta.shape[2] >= L:
+        return delta
+    return None
+
+
 def chunked_backward(kc, vc, xq, static_src, static_dest, out, g_out, g_denom, state=None, skip_masked=False, recompute=False):
-    """state: what chunked_forward(keep_state=True) returned for the same inputs and flags, or None."""
+    """state: what chunked_forward(keep_state=True) returned for the same inputs and flags, or None.
+    When (g_out, g_denom) are the very tensors merge_backward produced from `out` (the reference's call sequence), the
+    backward takes delta = sum_d out g_out - g_denom from that call instead of reading both 4-GB-class tensors again,
+    and knows that the gradients vanish where a query precedes a chunk."""
     src_dtype, dest_dtype = static_src.dtype, static_dest.dtype
+    delta = None
+    if kc.shape[3] % 64 == 0:
+        delta = _delta_from_merge(out, g_out, g_denom, kc.shape[2] * kc.shape[3], kc.shape[2])
+        if delta is not None:
+            skip_masked = True
     kc, vc, xq, src, dest, gflag = _prep(kc, vc, xq, static_src, static_dest)
     lib = _lib.load()
     b, h, n, c, d = kc.shape
     r = xq.shape[2]
     L = n * c
     desc = _desc(kc, xq, True, (_lib.UA_FLAG_SKIP_MASKED if skip_masked else 0) | (_lib.UA_FLAG_RECOMPUTE if recompute else 0) | gflag)
+    lse2 = None
+    if state is not None and state.dtype == torch.float32:        # the normalisers alone
+        lse2, state = state, None
+        if lse2.numel() != b * h * r * n * (-(-L // 128) * 128):
+            lse2 = None
     if state is not None and state.numel() < lib.ua_workspace_bytes(ctypes.byref(desc), _lib.UA_OP_FWD):
         state = None
     ws = _workspace(desc, _lib.UA_OP_BWD_SCRATCH if state is not None else _lib.UA_OP_BWD, xq.device)
@@ -148,6 +184,7 @@ def chunked_backward(kc, vc, xq, static_src, static_dest, out, g_out, g_denom, s
     _lib.check(lib.ua_bwd(ctypes.byref(desc), ctypes.byref(_rows_k(kc)), ctypes.byref(_rows_k(vc)), ctypes.byref(_rows_q(xq)),
                           src.data_ptr(), dest.data_ptr(), ctypes.byref(oc), ctypes.byref(gc), gd.data_ptr(), dk.data_ptr(),
                           dv.data_ptr(), dq.data_ptr(), dsrc.data_ptr(), ddest.data_ptr(),
+                          delta.data_ptr() if delta is not None else None, lse2.data_ptr() if lse2 is not None else None,
                           state.data_ptr() if state is not None else None, ws.data_ptr(), ws.numel(), _stream()), "ua_bwd")
     del out_t, g_out_t
     return dk, dv, dq, dsrc.to(src_dtype), ddest.to(dest_dtype)
@@ -259,10 +296,16 @@ def merge_backward(mat, vec, g):
     d4 = store.permute(0, 2, 3, 1)
     dc = UaChunked(d4.data_ptr(), d4.stride(0), d4.stride(1), d4.stride(2), d4.stride(3))
     d_vec = torch.empty(*vec.shape, dtype=mat.dtype, device=mat.device)
+    Lp = -(-L // 128) * 128
+    delta = torch.zeros(m4.shape[0], n, Lp, dtype=torch.float32, device=mat.device)
     _lib.check(lib.ua_merge_bwd(_dtype_code(mat), rows, L, d, n, ctypes.byref(mc), vec_c.data_ptr(), g_c.data_ptr(), ctypes.byref(dc),
-                                d_vec.data_ptr(), _stream()), "ua_merge_bwd")
+                                d_vec.data_ptr(), delta.data_ptr(), _stream()), "ua_merge_bwd")
     d_mat = d4.unflatten(0, tuple(mat.shape[:-3])) if mat.dim() != 4 else d4
-    return d_mat, d_vec.to(vec.dtype)
+    d_vec = d_vec.to(vec.dtype)
+    import weakref
+    _merge_handoff["last"] = (weakref.ref(d_mat), weakref.ref(d_vec), (mat.data_ptr(), tuple(mat.shape), tuple(mat.stride()), mat._version),
+                              d_mat._version, d_vec._version, delta)
+    return d_mat, d_vec
 
 
 def autotune(kc, vc, xq, static_src, static_dest, dO=None, backward=True):

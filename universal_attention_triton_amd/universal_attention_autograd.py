@@ -40,14 +40,15 @@ class _ChunkedBase(Function):
     # bf16, chunk a multiple of 64: True keeps the backward's workspace small (UA_FLAG_RECOMPUTE: its second kernel
     # recomputes the score and decay gradients instead of reading them from 2*L*L bytes per head)
     recompute = False
-    # True: keep the forward state (packed inputs, carries, per-chunk normalisers) for the backward instead of
-    # rebuilding it there; costs ua_workspace_bytes(UA_OP_FWD) bytes per call between forward and backward.  The
-    # reference keeps its five inputs only (universal_attention.py:27-31), which is the default here too.
-    keep_state = False
+    # What the backward gets from the forward besides the five inputs the reference keeps (universal_attention.py:27-31)
+    # and `out`: "normalisers" (default): the per-chunk normalisers in float32, 1/(d+1) of the size of `out`, which spare
+    # the backward a second run of the forward kernel; True: the whole forward state (ua_workspace_bytes(UA_OP_FWD)
+    # bytes: packed inputs, decay carries, normalisers); False: nothing.
+    keep_state = "normalisers"
 
     @staticmethod
     def forward(kc, vc, xq, static_src, static_dest):
-        keep = _ChunkedBase.keep_state and any(t.requires_grad for t in (kc, vc, xq, static_src, static_dest))
+        keep = _ChunkedBase.keep_state if any(t.requires_grad for t in (kc, vc, xq, static_src, static_dest)) else False
         out, denom, state = ops.chunked_forward(kc, vc, xq, static_src, static_dest, keep_state=keep,
                                                 recompute=_ChunkedBase.recompute)
         _put_state(out, state)
