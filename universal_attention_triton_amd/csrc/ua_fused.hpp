@@ -13,9 +13,6 @@
 #include "ua_bwd.hpp"
 #include "ua_common.hpp"
 
-#ifndef UA_PF
-#define UA_PF 4
-#endif
 namespace ua {
 
 // One asynchronous instruction (1 KB, issued by one wave): lane l copies 16 bytes from src to base + 16*l.
@@ -104,7 +101,7 @@ struct FalseC { static constexpr bool value = false; };
 // softmax weight itself.
 // NW: waves per workgroup (8, or 4 for launches of few workgroups: twice as many, half as long in LDS and registers).
 template <class T, int D, int NST, bool CM, bool BO, int NW = 8>
-__global__ void __launch_bounds__(64 * NW) k_carry2(const T* __restrict__ Kp, const float* __restrict__ lsrc,
+__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) k_carry2(const T* __restrict__ Kp, const float* __restrict__ lsrc,
                                                 const float* __restrict__ ldest, float* __restrict__ C, int Lp,
                                                 const float* __restrict__ knorm2, const float* __restrict__ qnorm2, int R,
                                                 int* __restrict__ reach, _Float16* __restrict__ Bt) {
@@ -1041,17 +1038,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
           for (int v = 0; v < 4; ++v) bias[i][v] += cin;
       }
     }
-    // Operands of the products that contract over the block's queries: none depends on anything this step computes,
-    // so they are fetched from LDS a few matrix instructions ahead (a rolling window of PF fragments), the first ones
-    // before the elementwise chain, instead of each right before its use
-    constexpr int PF = UA_PF;
-    Frag<T> pre[PF > 0 ? PF : 1];
     {
-      if constexpr (TR && PF > 0) {
-#pragma unroll
-        for (int k = 0; k < PF; ++k) pre[k] = ld8_tr<T>(sdO, k, lane);
-        __builtin_amdgcn_sched_barrier(0x7f);      // the reads stay here; everything else may move across
-      }
       f32x4 P[2], dS[2];
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
@@ -1080,18 +1067,6 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
       // matrix instructions goes first, and the other one's vector work fills the gaps (k_bwd_keys2<TO>: -6 %; raising
       // the priority around the short dependent chains of the input products as well gives the gain back).
       __builtin_amdgcn_s_setprio(1);
-      if constexpr (TR && PF > 0) {
-#pragma unroll
-        for (int n = 0; n < ND; ++n) {
-          mma16(dVt[n], pre[n % PF], bp);
-          pre[n % PF] = n + PF < ND ? ld8_tr<T>(sdO, n + PF, lane) : ld8_tr<T>(sQ, n + PF - ND, lane);
-        }
-#pragma unroll
-        for (int n = 0; n < ND; ++n) {
-          mma16(dKt[n], pre[n % PF], bs);
-          pre[n % PF] = n + PF < ND ? ld8_tr<T>(sQ, n + PF, lane) : ld8_tr<T>(sKt, n + PF - ND, lane);
-        }
-      } else {
 #pragma unroll
       for (int n = 0; n < ND; ++n) {
         if constexpr (TR) mma16(dVt[n], ld8_tr<T>(sdO, n, lane), bp);
@@ -1101,7 +1076,6 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
       for (int n = 0; n < ND; ++n) {
         if constexpr (TR) mma16(dKt[n], ld8_tr<T>(sQ, n, lane), bs);
         else mma16(dKt[n], ld8(sQT + TT::at(n, col, 0, g)), bs);
-      }
       }
       if constexpr (MS) {
         // dB (+)= reverse running sums of this group's dS; the block totals of the groups add up in dtot4
@@ -1153,18 +1127,10 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
         __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&b)[1], reinterpret_cast<u32x2*>(p + 1024));
       }
       __builtin_amdgcn_s_setprio(1);
-      if constexpr (TR && PF > 0) {
-#pragma unroll
-        for (int n = 0; n < ND; ++n) {
-          mma16(dKt[n], pre[n % PF], b);
-          if (n + PF < ND) pre[n % PF] = ld8_tr<T>(sKt, n + PF, lane);
-        }
-      } else {
 #pragma unroll
       for (int n = 0; n < ND; ++n) {
         if constexpr (TR) mma16(dKt[n], ld8_tr<T>(sKt, n, lane), b);
         else mma16(dKt[n], ld8(sKT + TT::at(n, col, 0, g)), b);
-      }
       }
       __builtin_amdgcn_s_setprio(0);
     }
