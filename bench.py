@@ -131,8 +131,9 @@ def parity_one_head(cfg, inp, O, grads, head=(0, 0)):
 
 # HBM bytes per launch of the roofline kernel, from the TCC counters FETCH_SIZE and WRITE_SIZE of two `rocprofv3 --pmc`
 # runs of this script, each scaled by what the same counter reads for the plain 1 GiB copy of --calibrate-copy
-# (profiles/bench_cfg2_fused_fwd_bwd.md: 3.74 GB read + 4.58 GB written by k_bwd_keys2).  A measured constant, not
-# collected by a default run; configurations without such a measurement report null.
+# (profiles/bench_cfg2_fused_fwd_bwd.md, taken 2026-11-25: 2.65 GB read + 4.51 GB written by k_bwd_keys2; the reads
+# are the fp16 bias tiles plus operand tiles, the writes the dS / dG tiles k_bwd_queries3 consumes).  The counters cannot
+# be collected by a plain run of this script, so the figure is a dated measurement; configurations without one report null.
 MEASURED_TRAFFIC = {(2, "k_bwd_keys"): 7.17e9}
 
 
@@ -307,6 +308,23 @@ def main():
         out["roofline"] = roof
         out["config"]["workload"] += "; chunked API (reference call sequence, chunk %d)" % cfg["c"]
         out["config"].pop("pct_of_mfma_peak", None)
+        # the same sequence with the whole forward state kept for the backward (keep_state = True: + one forward state of
+        # memory between the two, no second decay pre-pass and no repacking in the backward)
+        from universal_attention_triton_amd import universal_attention_autograd as own_api
+        own_api._ChunkedBase.keep_state = True
+        try:
+            n_full = max(3, args.steps // 4)
+            for _ in range(2):
+                step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(n_full):
+                step()
+            torch.cuda.synchronize()
+            out["config"]["keep_state_true"] = {"ms_per_step": round((time.perf_counter() - t0) * 1e3 / n_full, 4),
+                                                "note": "optional: forward state retained for the backward; not `value`"}
+        finally:
+            own_api._ChunkedBase.keep_state = "normalisers"
         if not args.no_cpu:
             out["cpu_baseline"] = cpu_baseline(cfg, args.config)
         print(json.dumps(out))
