@@ -745,6 +745,8 @@ k_fwd_fused3(const bf16* __restrict__ Qp, const bf16* __restrict__ Kp, const bf1
         ST::put(sPw + (2 * i + (j >> 1)) * ST::BYTES, 16 * (j & 1) + col, g, p);
       }
     }
+    // the 32 independent matrix instructions of P V issue back to back while the SIMD's other wave fills the gaps
+    __builtin_amdgcn_s_setprio(1);
 #pragma unroll
     for (int kq = 0; kq < 2; ++kq) {                   // 32 keys per k-step
       if (!MASKED || 4 * kt + 2 * kq <= 2 * qb + 1) {
@@ -758,6 +760,7 @@ k_fwd_fused3(const bf16* __restrict__ Qp, const bf16* __restrict__ Kp, const bf1
         }
       }
     }
+    __builtin_amdgcn_s_setprio(0);
   };
   {
     // the key tiles visited first hold the diagonal blocks of the waves: those with keys of the workgroup's own blocks
@@ -797,8 +800,13 @@ k_fwd_fused3(const bf16* __restrict__ Qp, const bf16* __restrict__ Kp, const bf1
 // (k-group-major, see Tile): two transposing reads, each turning a block of 4 positions x 16 features (8 bytes per lane:
 // lane i of a 16-lane group supplies position i/4 of the block and features 4(i%4)..+3) into 4 positions of feature i
 // per lane.  The k index follows as_operand16: elements 0-3 are positions 4G..4G+3, elements 4-7 positions 16+4G..+3
-// (G = lane / 16).  The 64 lanes of one read touch 2 x 256 contiguous bytes, i.e. every bank twice, which is what 512
-// bytes cost anyway.
+// (G = lane / 16).  The 64 lanes of one read touch 2 x 256 contiguous bytes; the LDS pipe takes 32 lanes at a time and
+// the first 32 touch the first half of both pieces, i.e. half of the banks twice: 4.1 cycles of the pipe per read where
+// 2.5 are possible.  A layout without that conflict was built and measured (feature tiles made of k-groups n and
+// n + D/16, positions p and p ^ 8 exchanged in the upper k-groups on the source side of the copy; the exchange has to be
+// the same for the four k-groups of a 16-byte operand read, which takes lane groups in pairs and costs 8 cycles
+// instead of 4 when their patterns differ): k_bwd_keys2 was 1-2 % slower with it, so the LDS pipe is not what its
+// waves wait for, and the plain layout stays.
 template <class T>
 __device__ __forceinline__ Frag<T> ld8_tr(const T* tile, int n, int lane) {
   static_assert(sizeof(T) == 2, "transposing LDS reads are 16-bit");
