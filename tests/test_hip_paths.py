@@ -241,3 +241,42 @@ def test_large_scores_and_deep_decay_bf16(recompute):
     torch.cuda.synchronize()
     assert rel_err(O, O_ref) <= TOL[bf], rel_err(O, O_ref)
     _table("large scores recompute=%s" % recompute, grads, g_ref, TOL[bf])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_out_allocated_contiguous_like_the_reference(dtype):
+    """`out` is normally a permuted view of chunk-major storage; with contiguous_out it is the reference's own layout
+    (so `.view()` works on it), with the same values, and the backward reads it and a contiguous gradient alike."""
+    from universal_attention_triton_amd import universal_attention_autograd as ua
+    print("case contiguous out", dtype, flush=True)
+    b, h, r, L, d, c = 1, 2, 2, 256, 32, 64
+    n = L // c
+    inp = orc.make_inputs(b, h, r, L, d, c, dtype=dtype, seed=77)
+    g = torch.Generator().manual_seed(9)
+    g_out = torch.randn(b, h, r, L, d, n, generator=g).to(dtype)
+    g_denom = torch.randn(b, h, r, L, n, generator=g).to(dtype)
+    results = []
+    for contiguous in (False, True):
+        ua._ChunkedBase.contiguous_out = contiguous
+        try:
+            leaves = [inp[k].cuda().requires_grad_() for k in NAMES]
+            out, denom = ua.UniversalAttention.apply(*leaves)
+            assert out.shape == (b, h, r, L, d, n)
+            assert out.is_contiguous() == contiguous
+            if contiguous:
+                out.view(b * h * r, L, d * n)            # what fails on the permuted view
+            grads = torch.autograd.grad([out, denom], leaves, [g_out.cuda(), g_denom.cuda()])
+            torch.cuda.synchronize()
+            results.append((out.detach().clone(), denom.detach().clone(), grads))
+        finally:
+            ua._ChunkedBase.contiguous_out = False
+    (o0, d0, g0), (o1, d1, g1) = results
+    assert torch.equal(o0, o1) and torch.equal(d0, d1)
+    for name, x, y in zip(NAMES, g0, g1):
+        assert rel_err(y, x) <= 1e-6, (name, rel_err(y, x))
+    # the default layout is checked against the oracle in test_hip_backward.py; here the other four gradients once more
+    # (float32 dkc has its own bar there: the singular derivative of relu(G)^(2/3))
+    want = orc.chunked_backward(*[inp[k].float() for k in NAMES], g_out.float(), g_denom.float())
+    for name, x, w in zip(NAMES, g1, want):
+        if name != "kc":
+            assert rel_err(x.reshape(w.shape), w) <= TOL[dtype], (name, rel_err(x.reshape(w.shape), w))

@@ -99,8 +99,10 @@ def _prep(kc, vc, xq, static_src, static_dest):
     return kc, vc, xq, src, dest, gflag
 
 
-def chunked_forward(kc, vc, xq, static_src, static_dest, keep_state=False, recompute=False):
+def chunked_forward(kc, vc, xq, static_src, static_dest, keep_state=False, recompute=False, contiguous_out=False):
     """-> out [b,h,r,l,d,n] (chunk-major storage, returned as a permuted view), denom [b,h,r,l,n], state
+    contiguous_out: allocate `out` contiguous in the reference's index order instead (what `.view()` on it needs; the
+    kernels then write 2-byte elements n * 2 bytes apart and every pass over `out` is several times slower).
     keep_state: what chunked_backward gets from the forward.  False: nothing (it rebuilds everything, including a
     second run of the forward kernel).  "normalisers": the per-chunk normalisers in float32 (1/(d+1) of the size of
     `out`; the backward then only repacks the inputs and rebuilds the decay carries).  True: the whole forward state (the
@@ -113,8 +115,10 @@ def chunked_forward(kc, vc, xq, static_src, static_dest, keep_state=False, recom
     L = n * c
     desc = _desc(kc, xq, True, (_lib.UA_FLAG_RECOMPUTE if recompute else 0) | gflag)
     ws = _workspace(desc, _lib.UA_OP_FWD, xq.device)
-    store = torch.empty(b, h, r, n, L, d, dtype=xq.dtype, device=xq.device)
-    out = store.permute(0, 1, 2, 4, 5, 3)
+    if contiguous_out:
+        out = torch.empty(b, h, r, L, d, n, dtype=xq.dtype, device=xq.device)
+    else:
+        out = torch.empty(b, h, r, n, L, d, dtype=xq.dtype, device=xq.device).permute(0, 1, 2, 4, 5, 3)
     denom = torch.empty(b, h, r, L, n, dtype=xq.dtype, device=xq.device)
     _, oc = _chunked(out)
     lse2 = None

@@ -45,12 +45,17 @@ class _ChunkedBase(Function):
     # the backward a second run of the forward kernel; True: the whole forward state (ua_workspace_bytes(UA_OP_FWD)
     # bytes: packed inputs, decay carries, normalisers); False: nothing.
     keep_state = "normalisers"
+    # `out` is stored chunk-major ([b,h,r,n,L,d]) and returned as a permuted view with the reference's shape and values:
+    # every kernel then moves 16 bytes per lane.  True allocates it contiguous like the reference does, for callers
+    # that `.view()` it; the passes over it are then several times slower.
+    contiguous_out = False
 
     @staticmethod
     def forward(kc, vc, xq, static_src, static_dest):
         keep = _ChunkedBase.keep_state if any(t.requires_grad for t in (kc, vc, xq, static_src, static_dest)) else False
         out, denom, state = ops.chunked_forward(kc, vc, xq, static_src, static_dest, keep_state=keep,
-                                                recompute=_ChunkedBase.recompute)
+                                                recompute=_ChunkedBase.recompute,
+                                                contiguous_out=_ChunkedBase.contiguous_out)
         _put_state(out, state)
         return out, denom
 
