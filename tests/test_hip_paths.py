@@ -280,3 +280,34 @@ def test_out_allocated_contiguous_like_the_reference(dtype):
     for name, x, w in zip(NAMES, g1, want):
         if name != "kc":
             assert rel_err(x.reshape(w.shape), w) <= TOL[dtype], (name, rel_err(x.reshape(w.shape), w))
+
+
+@pytest.mark.parametrize("shape", [(1, 2, 2, 512, 64, 64), (1, 1, 1, 768, 128, 192), (2, 1, 1, 256, 128, 128)])
+def test_upstream_gradient_read_in_place_equals_its_packed_copy(shape):
+    """bf16, chunk a multiple of 64, nothing flowing to (query, later chunk) pairs: a chunk-major upstream gradient with
+    rows of exactly the padded head dim is gathered by the key-side kernel from the caller's tensor; any other storage
+    goes through a packed copy.  Same tiles either way; delta = sum_d out * g_out is summed in another order for the
+    other storage (float32 rounding), which flips the last bf16 bit of a handful of gradient elements."""
+    from universal_attention_triton_amd import ops
+    print("case g_out in place", shape, flush=True)
+    b, h, r, L, d, c = shape
+    n = L // c
+    dtype = torch.bfloat16
+    inp = orc.make_inputs(b, h, r, L, d, c, dtype=dtype, seed=55)
+    gen = torch.Generator().manual_seed(3)
+    live = (torch.arange(L).view(L, 1, 1) >= torch.arange(n).view(1, 1, n) * c)
+    g_ref_order = (torch.randn(b, h, r, L, d, n, generator=gen) * live).to(dtype).cuda()          # contiguous [.., L, d, n]
+    g_denom = (torch.randn(b, h, r, L, n, generator=gen) * live.view(L, n)).to(dtype).float().cuda()
+    ins = [inp[k].cuda() for k in NAMES]
+    out, denom, state = ops.chunked_forward(*ins, keep_state=True)
+    g_chunk_major = g_ref_order.permute(0, 1, 2, 5, 3, 4).contiguous().permute(0, 1, 2, 4, 5, 3)  # same values, [.., n, L, d] storage
+    assert torch.equal(g_chunk_major, g_ref_order) and not g_chunk_major.is_contiguous()
+    got_in_place = ops.chunked_backward(*ins, out, g_chunk_major, g_denom, state=state, skip_masked=True)
+    got_packed = ops.chunked_backward(*ins, out, g_ref_order, g_denom, state=state, skip_masked=True)
+    torch.cuda.synchronize()
+    for name, x, y in zip(NAMES, got_in_place, got_packed):
+        assert rel_err(x, y) <= 1e-4, (name, rel_err(x, y))
+        assert int((x != y).sum()) <= x.numel() // 1000, (name, int((x != y).sum()))
+    want = orc.chunked_backward(*[inp[k].float() for k in NAMES], g_ref_order.float().cpu(), g_denom.cpu())
+    for name, x, w in zip(NAMES, got_in_place, want):
+        assert rel_err(x.reshape(w.shape), w) <= TOL[dtype], (name, rel_err(x.reshape(w.shape), w))

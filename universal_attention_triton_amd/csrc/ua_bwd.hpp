@@ -51,6 +51,9 @@ struct BwdArgs {
   int direct, d_out;
   T *dk_out, *dv_out, *dsrc_out, *ddest_out;
   const T *src_in, *dest_in;
+  // chunked operator with tile exchange: dOp is not the packed copy but the caller's upstream gradient itself, stored
+  // chunk-major as rows of exactly D elements, [Zq*nch][L][D] with L a multiple of 32 (k_bwd_keys2 gathers its tiles)
+  int dO_rows;
 };
 
 // grid (key groups, Zk).  chunked == 0: key group = 128 consecutive keys, 4 waves.

@@ -393,7 +393,7 @@ hipError_t delta_t(const ua::RowsView& O, const ua::RowsView& dO, const ua::Rows
 // otherwise the key-stationary and query-stationary kernels over tiled working tensors
 int run_bwd_common(const ua_desc& d, const Layout& l, char* wf, char* wb, bool chunked, const void* src, const void* dest, void* dkc,
                    void* dvc, void* dxq, void* dsrc, void* ddest, hipStream_t s, const float* delta_given = nullptr,
-                   const float* lse2_given = nullptr) {
+                   const float* lse2_given = nullptr, const void* dO_rows = nullptr) {
   const bool is_chunked = chunked;
   chunked = is_chunked && !fast_chunk(d);      // from here on: the atomics path
   if (chunked) {
@@ -411,6 +411,7 @@ int run_bwd_common(const ua_desc& d, const Layout& l, char* wf, char* wb, bool c
   a.dVrow = (float*)(wb + l.dVrow); a.dsrc_raw = (float*)(wb + l.dsrc_raw);
   a.masked_nz = (const int*)(wb + l.masked_nz);
   a.dS_st = l.grad_tiles ? wb + l.dS_st : nullptr; a.dG_st = l.grad_tiles ? wb + l.dG_st : nullptr; a.Bt = l.tiles ? wf + l.Bt : nullptr;
+  if (dO_rows) { a.dOp = dO_rows; a.dO_rows = 1; }      // the caller's upstream gradient, read in place by k_bwd_keys2
   a.R = d.r; a.L = d.L; a.Lp = l.Lp; a.c = is_chunked ? d.chunk : 128; a.nch = l.nch; a.chunked = is_chunked ? 1 : 0;
   a.skip_masked = (d.flags & UA_FLAG_SKIP_MASKED) ? 1 : 0;
   a.split_r = (!chunked && d.r > 1) ? 1 : 0;
@@ -642,6 +643,7 @@ int ua_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
                                        (const int*)(wf + l.minkey), nullptr, nullptr, (float*)(wf + l.lse2), 0, 0, 0, 0, d.r, d.L, l.Lp,
                                        d.d, d.chunk, l.nch, l.Zq, s));
     }
+    bool in_place = false;
     {
       UA_PROF("pack_dO+delta", s);
       UA_HIP(zero_fill(wb + l.masked_nz, 256, s));
@@ -651,10 +653,18 @@ int ua_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
       if (delta) { /* ua_merge_bwd left it: neither out nor g_out is read for it */ }
       else if (d.dtype == UA_BF16) UA_HIP(delta_t<ua::bf16>(outv, gv, gdv, none, (float*)(wb + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s, detect, d.chunk));
       else UA_HIP(delta_t<float>(outv, gv, gdv, none, (float*)(wb + l.delta), nullptr, d.d, d.L, l.Lp, l.Zq * l.nch, s, detect, d.chunk));
-      UA_HIP(pack(d.dtype, l.D, gv, wb + l.dOp, l.grad_tiles ? nullptr : wb + l.dOT, d.d, d.L, l.Lp, l.Zq * l.nch, TR_PERM32, s, nullptr, nz,
-                  d.chunk));
+      // With the tile exchange only the key-side kernel reads the upstream gradient, and when nothing flows to the
+      // (query, later chunk) pairs (UA_FLAG_SKIP_MASKED) it can gather its tiles from the caller's tensor itself if that
+      // is stored chunk-major in rows of exactly D elements: no packed copy (half of g_out read, as much written).
+      in_place = l.grad_tiles && (d.flags & UA_FLAG_SKIP_MASKED) && d.d == l.D && d.L % 32 == 0 && g_out->stride_d == 1 &&
+                 g_out->stride_t == d.d && g_out->stride_i == (int64_t)d.L * d.d && g_out->stride_z == (int64_t)l.nch * d.L * d.d &&
+                 (uintptr_t)g_out->ptr % 16 == 0;
+      if (!in_place)
+        UA_HIP(pack(d.dtype, l.D, gv, wb + l.dOp, l.grad_tiles ? nullptr : wb + l.dOT, d.d, d.L, l.Lp, l.Zq * l.nch, TR_PERM32, s, nullptr, nz,
+                    d.chunk));
     }
-    return run_bwd_common(d, l, wf, wb, true, static_src, static_dest, dkc, dvc, dxq, dsrc, ddest, s, delta, lse2_in);
+    return run_bwd_common(d, l, wf, wb, true, static_src, static_dest, dkc, dvc, dxq, dsrc, ddest, s, delta, lse2_in,
+                          in_place ? g_out->ptr : nullptr);
   }
   if (delta) return fail(UA_EINVAL, "a precomputed delta needs UA_FLAG_SKIP_MASKED and a chunk that is a multiple of 64");
   if (!fwd_state) {

@@ -883,6 +883,20 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   Stager<TT, 8> stT;
   stN.init(w, lane, D * (long)sizeof(T), 32);
   stT.init(w, lane, Lp * (long)sizeof(T), D);
+  // Upstream-gradient tiles.  Normally the packed copy (tiles like those of K and Q).  Chunked operator with a.dO_rows:
+  // the caller's own tensor, rows of D elements: lane l of copy instruction i fetches the 16 bytes that belong at LDS
+  // unit 64 i + l = (k-group, position) from row `position`, so that the LDS image is the same (32 rows of 16 bytes
+  // per instruction instead of 1 KB in one piece).
+  const bool dO_in_place = CH && TR && a.dO_rows;
+  const long dO_len = dO_in_place ? L : Lp;             // rows per (query head, chunk)
+  Stager<TN, 8> stG = stN;
+  if (dO_in_place) {
+#pragma unroll
+    for (int k = 0; k < Stager<TN, 8>::PER; ++k) {
+      const int n = (w + k * 8) * 64 + lane;
+      stG.off[k] = (n & 31) * (D * (int)sizeof(T)) + (n >> 5) * 16;
+    }
+  }
 
   Frag<T> kp[NK], vf[NK];
   {
@@ -923,10 +937,10 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
     const long zq_ = zq0 + (MR ? (s) % R : 0);                                              \
     const long qo_ = (zq_ * Lp + 32 * tb_) * D;   /* tile base, natural and transposed */      \
     const long zg_ = zq_ * nch + ch0;             /* z index of dO, delta, lse2 */             \
-    const long go_ = (zg_ * Lp + 32 * tb_) * D;                                             \
+    const long go_ = (zg_ * dO_len + 32 * tb_) * D;                                         \
     stN.issue((base), Kz + (long)(32 * tb_) * D, w);                                        \
     stN.issue((base) + TN::BYTES, a.Qp + qo_, w);                                           \
-    stN.issue((base) + 2 * TN::BYTES, a.dOp + go_, w);                                      \
+    stG.issue((base) + 2 * TN::BYTES, a.dOp + go_, w);                                      \
     if (!TR) {                                                                              \
       stT.issue((base) + 3 * TN::BYTES, KTz + (long)(32 * tb_) * D, w);                     \
       stT.issue((base) + 3 * TN::BYTES + TT::BYTES, a.QT + qo_, w);                         \
@@ -943,7 +957,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
     }                                                                                       \
     if (BI) issue_row_nt((base) + TILES + 1024 + w * 1024, bt_src + (tri_bias_row(tb_) << 10)); \
     if (CH && two) {                                                                        \
-      stN.issue((base) + DO2, a.dOp + go_ + (long)Lp * D, w);                               \
+      stG.issue((base) + DO2, a.dOp + go_ + dO_len * D, w);                                 \
       if (!TR) stT.issue((base) + DO2T, a.dOT + go_ + (long)Lp * D, w);                     \
       if (w == 1) {                                                                         \
         const float* src_ = ((lane & 8) ? a.delta : a.lse2) + (zg_ + 1) * Lp + 32 * tb_ + 4 * (lane & 7); \

@@ -17,6 +17,7 @@ static BwdArgs<T> typed(const BwdArgsV& v) {
   a.R = v.R; a.L = v.L; a.Lp = v.Lp; a.c = v.c; a.nch = v.nch; a.chunked = v.chunked; a.skip_masked = v.skip_masked; a.split_r = v.split_r; a.key_parts = v.key_parts > 0 ? v.key_parts : 1;
   a.direct = v.direct; a.d_out = v.d_out; a.dk_out = (T*)v.dk_out; a.dv_out = (T*)v.dv_out; a.dsrc_out = (T*)v.dsrc_out;
   a.ddest_out = (T*)v.ddest_out; a.src_in = (const T*)v.src_in; a.dest_in = (const T*)v.dest_in;
+  a.dO_rows = v.dO_rows;
   return a;
 }
 

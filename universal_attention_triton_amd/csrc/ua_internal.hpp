@@ -18,6 +18,7 @@ struct BwdArgsV {
   int direct, d_out;
   void *dk_out, *dv_out, *dsrc_out, *ddest_out;
   const void *src_in, *dest_in;
+  int dO_rows;
 };
 
 // Every launcher returns hipGetLastError() after enqueuing.  dtype: 0 fp32, 1 bf16.  D in {64,128}.
