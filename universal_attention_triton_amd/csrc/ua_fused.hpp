@@ -82,6 +82,7 @@ __device__ __forceinline__ void issue_row_nt(void* lds_base, const void* src_lan
 //   Dsuf[z][t16][s] = sum_{t >= 16*(t16+1)} dBias[s,t]
 // ---------------------------------------------------------------------------------------------
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 struct TrueC { static constexpr bool value = true; };
 struct FalseC { static constexpr bool value = false; };
 
@@ -290,7 +291,8 @@ __global__ void __launch_bounds__(256) k_chunk_masked_out(const T* __restrict__ 
     const int vpr = d / V;                                      // vectors per row
     for (int idx = tid; idx < (r1 - r0) * vpr; idx += 256) {
       const int t = r0 + idx / vpr, cv = idx % vpr;
-      *reinterpret_cast<uint4*>(base + (long)t * co.st + cv * V) = *reinterpret_cast<const uint4*>(mean + cv * V);
+      // written once and read by nobody in the reference's call sequence (the merge skips slices of zero weight)
+      __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(mean + cv * V), reinterpret_cast<u32x4*>(base + (long)t * co.st + cv * V));
     }
   } else {
     for (int idx = tid; idx < (r1 - r0) * d; idx += 256) {
