@@ -137,6 +137,50 @@ def parity_one_head(cfg, inp, O, grads, head=(0, 0)):
 MEASURED_TRAFFIC = {(2, "k_bwd_keys"): 7.18e9}
 
 
+def bench_sdpa(args, cfg):
+    """Calibration, not the product: PyTorch's own scaled_dot_product_attention (plain causal attention, no decay bias)
+    at the config's shape, forward and forward + backward, with each backend that runs here."""
+    import torch.nn.functional as F
+    b, h, L, d = cfg["b"], cfg["h"] * cfg["r"], cfg["L"], cfg["d"]
+    dt = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float32
+    q = torch.randn(b, h, L, d, device="cuda", dtype=dt, requires_grad=True)
+    k = torch.randn_like(q, requires_grad=True)
+    v = torch.randn_like(q, requires_grad=True)
+    do = torch.randn_like(q)
+
+    def timed(bwd, n=20):
+        def run():
+            o = F.scaled_dot_product_attention(q, k, v, is_causal=True)
+            if bwd:
+                torch.autograd.grad(o, [q, k, v], do)
+        for _ in range(3):
+            run()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            run()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / n
+
+    res = {"default backend": {"fwd_ms": round(timed(False), 4), "fwd_bwd_ms": round(timed(True), 4)}}
+    try:
+        from torch.nn.attention import SDPBackend, sdpa_kernel
+        for name, be in (("flash", SDPBackend.FLASH_ATTENTION), ("memory-efficient", SDPBackend.EFFICIENT_ATTENTION)):
+            try:
+                with sdpa_kernel(be):
+                    res[name] = {"fwd_ms": round(timed(False), 4), "fwd_bwd_ms": round(timed(True), 4)}
+            except Exception as e:      # a backend that does not take this shape
+                res[name] = {"error": str(e)[:80]}
+    except ImportError:
+        pass
+    best = min(x["fwd_bwd_ms"] for x in res.values() if "fwd_bwd_ms" in x)
+    print(json.dumps({"metric": "torch scaled_dot_product_attention, causal, no decay bias: fwd+bwd", "value": best, "unit": "ms",
+                      "n_gpus": 1, "steps": 20, "warmup": 3, "ms_per_step": best, "higher_is_better": False, "scaling": "weak",
+                      "vs_baseline": None, "dtype": cfg["dtype"], "data": "synthetic",
+                      "config": {"workload": "plain causal attention at the shape of BASELINE config %d: b=%d heads=%d L=%d d=%d"
+                                 % (args.config, b, h, L, d), "backends": res}}))
+
+
 def bench_affinity(args, cfg, inp):
     """The stand-alone decay bias (AffinityScores: k, src, dest -> aff [b,h,L,L]) forward and backward at the config's
     key shape; both directions are bound by the L x L tensor they write or read."""
@@ -184,7 +228,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-parity", action="store_true", help="skip the one-head oracle check of the outputs and gradients")
     ap.add_argument("--chunk", type=int, default=None, help="--api chunked: keys per chunk (default: the config's, 128)")
-    ap.add_argument("--api", choices=["fused", "chunked", "affinity"], default="fused",
+    ap.add_argument("--api", choices=["fused", "chunked", "affinity", "sdpa"], default="fused",
                     help="fused (default): universal_attention(); chunked: the reference's call sequence "
                          "UniversalAttention.apply + SMVecMatMul.apply, which materialises out[b,h,r,L,d,n]")
     ap.add_argument("--no-pruned", action="store_true",
@@ -218,6 +262,8 @@ def main():
 
     if args.api == "affinity":
         return bench_affinity(args, cfg, inp)
+    if args.api == "sdpa":
+        return bench_sdpa(args, cfg)
     if args.api == "chunked":
         import universal_attention_autograd as ref_api
 
