@@ -9,6 +9,7 @@ upstream gradient dO shaped like the output).  Prints ONE JSON line:
             dK(decay side) = (2+4r) d L^2 b h flops per launch) against the bf16 dense MFMA peak, its duration
             measured with hipEvents on the launch stream during the timed steps
   config.pruned_mode  the same step with the optional pruning of provably negligible pairs (never part of `value`)
+  config.recompute_mode  the same step with UA_FLAG_RECOMPUTE: no per-pair tensor passes through HBM (never `value`)
   cpu_baseline  the oracle (a port of the reference's torch operator) timed on the host cores on a bounded sample:
             whole kv heads of the same workload, one after the other, until about 10 s have passed
 """
@@ -272,13 +273,13 @@ def main():
             O = ref_api.SMVecMatMul.apply(out_c, denom_c)
             return torch.autograd.grad(O, leaves, dO) if cfg["bwd"] else O
     elif cfg["bwd"]:
-        def step(prune=False):
-            O = universal_attention(*leaves, prune=prune)
+        def step(prune=False, recompute=False):
+            O = universal_attention(*leaves, prune=prune, recompute=recompute)
             return torch.autograd.grad(O, leaves, dO)
     else:
-        def step(prune=False):
+        def step(prune=False, recompute=False):
             with torch.no_grad():
-                return universal_attention(*leaves, prune=prune)
+                return universal_attention(*leaves, prune=prune, recompute=recompute)
 
     if args.calibrate_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").fill_(1.0)
@@ -388,6 +389,21 @@ def main():
         ms_p = (time.perf_counter() - t0) * 1e3 / args.steps
         out["config"]["pruned_mode"] = {"ms_per_step": round(ms_p, 4), "speedup": round(ms / ms_p, 2),
                                         "note": "optional exact pruning of negligible pairs; not counted in value"}
+    # the same step with UA_FLAG_RECOMPUTE (bf16): every kernel evaluates the affinity chain and the score / decay
+    # gradients itself, so that neither the bias nor the gradients of a (key, query) pair ever travel through HBM (only
+    # one carry per key and 16 queries does); more vector work, a quarter of the workspace
+    if not args.no_pruned and cfg["dtype"] == "bf16" and cfg["d"] <= 128:
+        n_rc = max(3, args.steps // 4)
+        for _ in range(2):
+            step(recompute=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n_rc):
+            step(recompute=True)
+        torch.cuda.synchronize()
+        ms_r = (time.perf_counter() - t0) * 1e3 / n_rc
+        out["config"]["recompute_mode"] = {"ms_per_step": round(ms_r, 4), "tflops": round((f_fwd + f_bwd) / (ms_r * 1e-3) / 1e12, 2),
+                                           "note": "optional: no per-pair tensor passes through HBM; not `value`"}
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(cfg, args.config)
     print(json.dumps(out))
