@@ -1578,33 +1578,83 @@ k_bwd_queries3(BwdArgs<T> a, T* __restrict__ dq, int d) {
   UA_PIPE_RANGE(kt_min, n_kt, n_kt, UA_ISSUE, UA_COMPUTE);
 #undef UA_ISSUE
 #undef UA_COMPUTE
+  // Epilogue.  A result tile holds (query 4g + v, feature 16n + col) in lane (g, col); stored from there, a wave moves
+  // 32-byte pieces with one instruction per (v, n) and fetches the row side of dk the same way.  The tiles go through the
+  // wave's share of the (now idle) stages instead, 64 features at a time, and leave as pieces of rows: lane (g, col) then
+  // holds features 4 col .. 4 col + 3 of queries 4i + g, i = 0..3, so that 16 lanes move 128 contiguous bytes of dq / dk
+  // and 256 of the row side of dk.
+  static_assert(NST == 2, "the epilogue stages its tiles in both stage buffers");
+  __syncthreads();                      // every wave is done with the stages
+  constexpr int RS = 64 + 4;            // floats per staged row: the four row groups of a store hit different banks
+  static_assert(4 * 16 * RS * 4 <= SB, "staging area");
+  float* xs = reinterpret_cast<float*>((w < 4 ? stage0 : stage1) + (w & 3) * (16 * RS * 4));
+  const bool vec_ok = (d & 3) == 0 && ((reinterpret_cast<uintptr_t>(dq) | reinterpret_cast<uintptr_t>(a.dk_out)) & 7) == 0;
+  auto stage_half = [&] __device__ (const f32x4 (&X)[ND], int hf, f32x4 (&out)[4]) {
 #pragma unroll
-  for (int v = 0; v < 4; ++v) {
-    const int t = 16 * tq + 4 * g + v;
-    if (t < L) {
+    for (int nn = 0; nn < 4; ++nn)
 #pragma unroll
-      for (int n = 0; n < ND; ++n) {
-        const int dd = 16 * n + col;
-        if (dd < d) dq[((long)zq * L + t) * d + dd] = cvt<T>(dQ[n][v]);
+      for (int v = 0; v < 4; ++v) xs[(4 * g + v) * RS + 16 * nn + col] = X[4 * hf + nn][v];
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) out[i] = *reinterpret_cast<const f32x4*>(xs + (4 * i + g) * RS + 4 * col);
+    __builtin_amdgcn_wave_barrier();
+  };
+  auto store4 = [&] __device__ (T* dst, long row, int f0, const f32x4& x) {      // 4 consecutive features of a row of d
+    if (vec_ok) {
+      if (f0 < d) {
+        union { T h[4]; u32x2 u; } pk;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) pk.h[e] = cvt<T>(x[e]);
+        __builtin_nontemporal_store(pk.u, reinterpret_cast<u32x2*>(dst + row * d + f0));
       }
-    }
-    if (a.direct) {       // r = 1: dk = row side (k_bwd_keys2) + column side, ddest = (k_u . dkcol_u) / (2 dest_u)
-      float dot = 0.f;
-      if (t < L) {
-#pragma unroll
-        for (int n = 0; n < ND; ++n) {
-          const int dd = 16 * n + col;
-          if (dd < d) {
-            dot = __builtin_fmaf(dKc[n][v], (float)a.Kp[nat_off<D>(zq, Lp, t, dd)], dot);
-            a.dk_out[((long)zq * L + t) * d + dd] = cvt<T>(a.dKrow[((long)zq * Lp + t) * D + dd] + dKc[n][v]);
-          }
-        }
-      }
-      dot = allsum16(dot);
-      if (col == 0 && t < L) a.ddest_out[(long)zq * L + t] = cvt<T>(dot / (2.0f * (float)a.dest_in[(long)zq * L + t]));
     } else {
 #pragma unroll
-      for (int n = 0; n < ND; ++n) a.dKdacc[((long)zq * Lp + t) * D + 16 * n + col] = dKc[n][v];
+      for (int e = 0; e < 4; ++e)
+        if (f0 + e < d) dst[row * d + f0 + e] = cvt<T>(x[e]);
+    }
+  };
+  float dot[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int hf = 0; hf < D / 64; ++hf) {
+    const int f0 = 64 * hf + 4 * col;
+    // the row side of dk and the keys themselves, fetched before the tiles are staged
+    f32x4 krow[4];
+    u32x2 kraw[4];
+    if (a.direct) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int t = 16 * tq + 4 * i + g;        // < Lp: both tensors are padded
+        krow[i] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(a.dKrow + ((long)zq * Lp + t) * D + f0));
+        kraw[i] = *reinterpret_cast<const u32x2*>(a.Kp + nat_off<D>(zq, Lp, t, f0));
+      }
+    }
+    f32x4 x[4];
+    stage_half(dQ, hf, x);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int t = 16 * tq + 4 * i + g;
+      if (t < L) store4(dq, (long)zq * L + t, f0, x[i]);
+    }
+    stage_half(dKc, hf, x);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int t = 16 * tq + 4 * i + g;
+      if (a.direct) {       // r = 1: dk = row side (k_bwd_keys2) + column side, ddest = (k_u . dkcol_u) / (2 dest_u)
+        const T* kk = reinterpret_cast<const T*>(&kraw[i]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) dot[i] = __builtin_fmaf(x[i][e], (float)kk[e], dot[i]);      // padded features: k = 0
+        if (t < L) store4(a.dk_out, (long)zq * L + t, f0, x[i] + krow[i]);
+      } else {
+        *reinterpret_cast<f32x4*>(a.dKdacc + ((long)zq * Lp + t) * D + f0) = x[i];
+      }
+    }
+  }
+  if (a.direct) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int t = 16 * tq + 4 * i + g;
+      const float sum = allsum16(dot[i]);
+      if (col == 0 && t < L) a.ddest_out[(long)zq * L + t] = cvt<T>(sum / (2.0f * (float)a.dest_in[(long)zq * L + t]));
     }
   }
 }
