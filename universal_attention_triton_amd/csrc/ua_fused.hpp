@@ -622,11 +622,15 @@ k_fwd_fused3(const bf16* __restrict__ Qp, const bf16* __restrict__ Kp, const bf1
   __shared__ __attribute__((aligned(256))) char sPbuf[8 * 4 * ST::BYTES];     // per wave: P of (query tile, 32-key half)
   typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
-  int bx, zy;
-  xcd_map(bx, zy);
+  // A workgroup handles two blocks of 32 NB queries one after the other, jt and (number of blocks - 1 - jt): every pair
+  // visits the same number of key tiles, so the launch is a whole number of equal rounds with half the workgroup changes
+  // (see k_bwd_keys2).  The body is expanded once per block.
+  int bx0, zy;
+  xcd_map(bx0, zy);
+  const int n_blk = (Lp / 32 + NB - 1) / NB;
+  auto sweep = [&](const int jt) __attribute__((always_inline)) {
   const int zq = RB == 1 ? zy : (zy / (R / RB)) * R + (zy % (R / RB)) * RB + w % RB;
   const int zk = zq / R, nT16 = Lp / 16, nT32 = Lp / 32;
-  const int jt = gridDim.x - 1 - bx;                          // heaviest workgroups first
   const int qb_raw = NB * jt + w / RB;
   const bool live = qb_raw < nT32;                            // the last workgroup may hold waves past the end
   const int qb = live ? qb_raw : nT32 - 1;                    // 32-query block of this wave
@@ -796,6 +800,12 @@ k_fwd_fused3(const bf16* __restrict__ Qp, const bf16* __restrict__ Kp, const bf1
         if (t < L) lse[(long)zq * L + t] = l2v * kLn2;
       }
     }
+  };
+  sweep(n_blk - 1 - bx0);
+  if (n_blk - 1 - bx0 != bx0) {
+    __syncthreads();       // the stages are free
+    sweep(bx0);
+  }
 }
 
 // The A operand [16 features 16n.. x 32 positions] of a "transposed" product out of the NATURAL tile [32 positions][D]

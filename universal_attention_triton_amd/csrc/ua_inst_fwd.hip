@@ -90,7 +90,7 @@ static hipError_t fused_bi(int variant, const void* Qp, const void* Kp, const vo
   if constexpr (D == 256) variant = 1;       // 16 queries per wave: the accumulators of a 32-query block do not fit
   if constexpr (D != 256) if (variant == 0) {
 #define UA_F3(RB_)                                                                                                          \
-  hipLaunchKernelGGL((k_fwd_fused3<D, RB_>), dim3((Lp / 32 + 8 / RB_ - 1) / (8 / RB_), Zq / RB_), dim3(512), 0, s, (const T*)Qp, \
+  hipLaunchKernelGGL((k_fwd_fused3<D, RB_>), dim3(((Lp / 32 + 8 / RB_ - 1) / (8 / RB_) + 1) / 2, Zq / RB_), dim3(512), 0, s, (const T*)Qp, \
                      (const T*)Kp, (const T*)VT, (T*)O, lse, lse2, reach, minkey, R, L, Lp, d, (const _Float16*)Bt)
     if (R % 4 == 0) UA_F3(4);
     else if (R % 2 == 0) UA_F3(2);
