@@ -225,6 +225,16 @@ __device__ __forceinline__ void xcd_map(int& bx, int& by) {
     bx = slot % gx;
   }
 }
+// CUs of the current device (launchers choose between one and two work items per workgroup by it)
+inline int device_cus() {
+  static const int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 0;
+    return n > 0 ? n : 256;
+  }();
+  return cus;
+}
+
 // The tensors of 1 KB tiles the 16-bit kernels exchange only hold the causal triangle, row after row:
 //   bias tiles:      row = 32-query block tb, key tiles j = 0 .. 2 tb + 1          -> the row starts at tile tb (tb + 1)
 //   gradient tiles:  row = 16-query tile tq,  32-key halves h = 0 .. tq / 2        -> the row starts at tile tri_grad_row(tq)

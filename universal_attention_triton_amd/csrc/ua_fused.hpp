@@ -802,7 +802,7 @@ k_fwd_fused3(const bf16* __restrict__ Qp, const bf16* __restrict__ Kp, const bf1
     }
   };
   sweep(n_blk - 1 - bx0);
-  if (n_blk - 1 - bx0 != bx0) {
+  if (gridDim.x != n_blk && n_blk - 1 - bx0 != bx0) {     // (launches of few workgroups keep one block each)
     __syncthreads();       // the stages are free
     sweep(bx0);
   }
@@ -1214,7 +1214,7 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   }
   };
   sweep(bx0);
-  if (n_kg - 1 - bx0 != bx0) {
+  if (gridDim.x != n_kg && n_kg - 1 - bx0 != bx0) {       // (launches of few workgroups keep one key group each)
     __syncthreads();       // the stages are free
     sweep(n_kg - 1 - bx0);
   }

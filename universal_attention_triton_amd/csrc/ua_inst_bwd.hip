@@ -52,7 +52,9 @@ template __global__ void k_bwd_keys2<bf16, 128, 2, true, true, true>(BwdArgs<bf1
 
 template <class T, int D, int NST, bool MR, bool CH, bool TO>
 static hipError_t bwd2_mr(const BwdArgs<T>& a, int Lp, int Zk, hipStream_t s) {
-  hipLaunchKernelGGL((k_bwd_keys2<T, D, NST, MR, CH, TO>), dim3((Lp / 128 + 1) / 2, Zk), dim3(512), 0, s, a);     // two key groups per workgroup
+  // two key groups per workgroup once every CU gets at least two of the single ones
+  const int n_kg = Lp / 128, gx = (long)n_kg * Zk >= 2 * device_cus() ? (n_kg + 1) / 2 : n_kg;
+  hipLaunchKernelGGL((k_bwd_keys2<T, D, NST, MR, CH, TO>), dim3(gx, Zk), dim3(512), 0, s, a);
   return hipGetLastError();
 }
 template <class T, int D, int NST>

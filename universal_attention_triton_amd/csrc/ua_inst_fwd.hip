@@ -89,9 +89,14 @@ static hipError_t fused_bi(int variant, const void* Qp, const void* Kp, const vo
   using T = bf16;
   if constexpr (D == 256) variant = 1;       // 16 queries per wave: the accumulators of a 32-query block do not fit
   if constexpr (D != 256) if (variant == 0) {
+    // two query blocks per workgroup once every CU gets at least two of the single ones
 #define UA_F3(RB_)                                                                                                          \
-  hipLaunchKernelGGL((k_fwd_fused3<D, RB_>), dim3(((Lp / 32 + 8 / RB_ - 1) / (8 / RB_) + 1) / 2, Zq / RB_), dim3(512), 0, s, (const T*)Qp, \
-                     (const T*)Kp, (const T*)VT, (T*)O, lse, lse2, reach, minkey, R, L, Lp, d, (const _Float16*)Bt)
+  do {                                                                                                                      \
+    const int n_blk_ = (Lp / 32 + 8 / RB_ - 1) / (8 / RB_);                                                                 \
+    const int gx_ = (long)n_blk_ * (Zq / RB_) >= 2 * device_cus() ? (n_blk_ + 1) / 2 : n_blk_;                             \
+    hipLaunchKernelGGL((k_fwd_fused3<D, RB_>), dim3(gx_, Zq / RB_), dim3(512), 0, s, (const T*)Qp,                          \
+                       (const T*)Kp, (const T*)VT, (T*)O, lse, lse2, reach, minkey, R, L, Lp, d, (const _Float16*)Bt);      \
+  } while (0)
     if (R % 4 == 0) UA_F3(4);
     else if (R % 2 == 0) UA_F3(2);
     else UA_F3(1);
