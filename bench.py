@@ -132,10 +132,10 @@ def parity_one_head(cfg, inp, O, grads, head=(0, 0)):
 
 # HBM bytes per launch of the roofline kernel, from the TCC counters FETCH_SIZE and WRITE_SIZE of two `rocprofv3 --pmc`
 # runs of this script, each scaled by what the same counter reads for the plain 1 GiB copy of --calibrate-copy
-# (profiles/bench_cfg2_fused_fwd_bwd.md, taken 2026-11-25: 2.66 GB read + 4.51 GB written by k_bwd_keys2; the reads
+# (profiles/bench_cfg2_fused_fwd_bwd.md, taken 2026-11-25: 2.60 GB read + 4.52 GB written by k_bwd_keys2; the reads
 # are the fp16 bias tiles plus operand tiles, the writes the dS / dG tiles k_bwd_queries3 consumes).  The counters cannot
 # be collected by a plain run of this script, so the figure is a dated measurement; configurations without one report null.
-MEASURED_TRAFFIC = {(2, "k_bwd_keys"): 7.18e9}
+MEASURED_TRAFFIC = {(2, "k_bwd_keys"): 7.11e9}
 
 
 def bench_sdpa(args, cfg):
