@@ -598,7 +598,8 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW
 
 // ---------------------------------------------------------------------------------------------
 // Fused forward of the 16-bit operator with bias tiles, one 32-query block per wave.
-// grid (ceil(Lp/32 / NB), Zk * R / RB), 8 waves, NB = 8 / RB blocks per workgroup; wave w owns block NB jt + w / RB of
+// grid (n or ceil(n / 2), Zk * R / RB) with n = ceil(Lp/32 / NB) workgroup blocks jt (the second form: blocks jt and
+// n - 1 - jt one after the other, see the body), 8 waves, NB = 8 / RB 32-query blocks per workgroup block; wave w owns block NB jt + w / RB of
 // query group w % RB of the workgroup's RB groups (grouped queries share the key and value tiles of a step).
 // Against k_fwd_fused2<BI> (16 queries per wave): every key / value operand read from LDS feeds two matrix
 // instructions (the two 16-query tiles of the block), the staged tiles serve 256 queries instead of 128, and a bias
@@ -831,7 +832,8 @@ __device__ __forceinline__ Frag<T> ld8_tr(const T* tile, int n, int lane) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Key-stationary backward (fused mode).  grid (Lp/128, Zk); 8 waves; wave w owns keys 128g+16w..+15 and
+// Key-stationary backward (fused mode).  grid (n or ceil(n / 2), Zk) with n = Lp/128 key groups g (the second form: groups
+// g and n - 1 - g one after the other, see the body); 8 waves; wave w owns keys 128g+16w..+15 and
 // sweeps the 32-query blocks from the last one down to its own; one (query block, query group) per step.
 // MR = more than one query group per kv head (the decay state of a query block then lives across steps).
 // ---------------------------------------------------------------------------------------------
