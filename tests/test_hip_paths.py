@@ -311,3 +311,26 @@ def test_upstream_gradient_read_in_place_equals_its_packed_copy(shape):
     want = orc.chunked_backward(*[inp[k].float() for k in NAMES], g_ref_order.float().cpu(), g_denom.cpu())
     for name, x, w in zip(NAMES, got_in_place, want):
         assert rel_err(x.reshape(w.shape), w) <= TOL[dtype], (name, rel_err(x.reshape(w.shape), w))
+
+
+@pytest.mark.parametrize("shape", [(1, 176, 1, 640, 64), (1, 88, 2, 896, 128)])
+def test_launches_of_paired_work_items_with_an_odd_number_of_items(shape):
+    """Launches with at least two workgroups per CU pair their work items (the key-stationary backward sweeps key groups
+    g and last - g in one workgroup, the forward over bias tiles query blocks j and last - j): here the number of items is
+    odd, so the middle one stays alone (5 or 7 key groups, 3 or 4 query blocks), and several heads spread over the
+    launch are held to the float64 dense oracle."""
+    from universal_attention_triton_amd import ops
+    b, h, r, L, d = shape
+    bf = torch.bfloat16
+    inp = orc.make_inputs(b, h, r, L, d, L, dtype=bf, seed=4242, gate_mean=0.0)
+    dev = {k: v.cuda() for k, v in inp.items()}
+    a = [dev[k] for k in NAMES]
+    O, lse, state = ops.fused_forward(*a, keep_state=True)
+    grads = ops.fused_backward(*a, O, lse, dev["dO"], state=state)
+    torch.cuda.synchronize()
+    for hh in (0, 1, h // 2, h - 1):
+        one = {k: v[:, hh:hh + 1] for k, v in inp.items()}
+        O_ref, lse_ref, g_ref = dense_reference(one)
+        assert rel_err(O[:, hh:hh + 1], O_ref) <= TOL[bf], hh
+        assert float((lse[:, hh:hh + 1].cpu().double() - lse_ref).abs().max()) <= 10 * TOL[bf], hh
+        _table("head %d of %s" % (hh, (shape,)), [x[:, hh:hh + 1] for x in grads], g_ref, TOL[bf])
