@@ -416,8 +416,11 @@ int run_bwd_common(const ua_desc& d, const Layout& l, char* wf, char* wb, bool c
   a.skip_masked = (d.flags & UA_FLAG_SKIP_MASKED) ? 1 : 0;
   a.split_r = (!chunked && d.r > 1) ? 1 : 0;
   a.key_parts = l.key_parts;
-  // merged bf16 operator with one query group: the two kernels write the caller's gradients themselves
-  const bool direct = l.tiles && d.r == 1 && !gates_f32(d);
+  // bf16 tile exchange with one query group: the two kernels write the caller's gradients themselves.  The chunked
+  // operator qualifies when the caller asserts that nothing flows to (query, later chunk) pairs, so that the query side is
+  // known here to run from the tiles.
+  const bool from_tiles = l.tiles || (is_chunked && l.grad_tiles && (d.flags & UA_FLAG_SKIP_MASKED));
+  const bool direct = from_tiles && d.r == 1 && !gates_f32(d);
   a.direct = direct ? 1 : 0; a.d_out = d.d; a.dk_out = dkc; a.dv_out = dvc; a.dsrc_out = dsrc; a.ddest_out = ddest;
   a.src_in = src; a.dest_in = dest;
   {
@@ -428,7 +431,7 @@ int run_bwd_common(const ua_desc& d, const Layout& l, char* wf, char* wb, bool c
     UA_PROF("k_bwd_queries", s);
     // chunked operator with tiles: both are enqueued, the flag k_delta left on the device decides which one works
     if (l.grad_tiles) UA_HIP(ua::launch_bwd_queries_from_tiles(l.D, a, dxq, d.d, l.Zq, s, tuned_variant(d, UA_TUNE_BWD_QUERIES)));
-    if (!l.tiles) UA_HIP(ua::launch_bwd_queries(d.dtype, l.D, a, dxq, d.d, l.Zk, s));
+    if (!from_tiles) UA_HIP(ua::launch_bwd_queries(d.dtype, l.D, a, dxq, d.d, l.Zk, s));
   }
   if (direct) return UA_OK;
   UA_PROF("k_bwd_finish", s);

@@ -1194,13 +1194,13 @@ __global__ void __launch_bounds__(512) k_bwd_keys2(BwdArgs<T> a) {
   {
     float b, af, tot;
     group_scan(dsrc_acc, gm, b, af, tot);
-    if (BI && !MR && a.direct) {      // straight into the caller's tensor: dsrc = sum dA A / (3 src)
+    if (TO && !MR && a.direct) {      // straight into the caller's tensor: dsrc = sum dA A / (3 src)
       if (g == 0 && spos < L) a.dsrc_out[(long)zo * L + spos] = cvt<T>(1.5f * tot / (3.0f * (float)a.src_in[(long)zo * L + spos]));
     } else if (g == 0) {
       a.dsrc_raw[(long)zo * Lp + spos] = 1.5f * tot;    // sum dA A = 3/2 sum dG G
     }
   }
-  const bool direct = BI && !MR && a.direct;
+  const bool direct = TO && !MR && a.direct;
 #pragma unroll
   for (int n = 0; n < ND; ++n) {
     const long o = ((long)zo * Lp + spos) * D + 16 * n + 4 * g;
