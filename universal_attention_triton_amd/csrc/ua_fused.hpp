@@ -1542,12 +1542,15 @@ k_bwd_queries3(BwdArgs<T> a, T* __restrict__ dq, int d) {
   constexpr int TILES = HV * TT::BYTES, WAVE = 2 * HV * ST::BYTES, SB = TILES + 8 * WAVE + 1024;
   UA_STAGES(SB);
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
-  int bx, zq;
-  xcd_map(bx, zq);
+  int bx0, zq;
+  xcd_map(bx0, zq);
   const int Lp = a.Lp, L = a.L, nT16 = Lp / 16, R = a.R, zk = zq / R, r = zq % R;
   // chunked operator with live (query, later chunk) pairs: their tiles are not exchanged, k_bwd_queries2 runs instead
   if (a.chunked && !a.skip_masked && *a.masked_nz != 0) return;
-  const int jt = gridDim.x - 1 - bx, tq = 8 * jt + w, tbq = tq >> 1;
+  const int n_blk = Lp / 128;
+  // two query blocks of complementary length per workgroup, the body expanded once per block (see k_bwd_keys2)
+  auto sweep = [&](const int jt) __attribute__((always_inline)) {
+  const int tq = 8 * jt + w, tbq = tq >> 1;
   Stager<TT, 8> stT;
   stT.init(w, lane, Lp * (long)sizeof(T), D);
   f32x4 dQ[ND], dKc[ND];
@@ -1681,6 +1684,29 @@ k_bwd_queries3(BwdArgs<T> a, T* __restrict__ dq, int d) {
       const int t = 16 * tq + 4 * i + g;
       const float sum = allsum16(dot[i]);
       if (col == 0 && t < L) a.ddest_out[(long)zq * L + t] = cvt<T>(sum / (2.0f * (float)a.dest_in[(long)zq * L + t]));
+    }
+  }
+  };
+  // Several blocks per workgroup, the body expanded once per block (steps of 32 keys only: with steps of 64 the
+  // expanded kernel is scheduled worse even for a single block).  Blocks of complementary length, heaviest first: all
+  // workgroups are equally long, the launch is a whole number of rounds, and the epilogues - whose traffic slows the
+  // stream of every other workgroup far beyond its bytes - fall together instead of spreading over the
+  // launch.  Four blocks j, n/2 - 1 - j, n/2 + j, n - 1 - j when the grid says so, else two, else one.
+  if constexpr (HV == 2) {
+    sweep(n_blk - 1 - bx0);
+  } else if (gridDim.x * 4 == n_blk) {
+    sweep(n_blk - 1 - bx0);
+    __syncthreads();       // the stages and the staging area are free
+    sweep(n_blk / 2 + bx0);
+    __syncthreads();
+    sweep(n_blk / 2 - 1 - bx0);
+    __syncthreads();
+    sweep(bx0);
+  } else {
+    sweep(n_blk - 1 - bx0);
+    if (gridDim.x != n_blk && n_blk - 1 - bx0 != bx0) {
+      __syncthreads();
+      sweep(bx0);
     }
   }
 }

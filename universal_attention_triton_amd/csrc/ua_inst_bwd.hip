@@ -53,7 +53,7 @@ template __global__ void k_bwd_keys2<bf16, 128, 2, true, true, true>(BwdArgs<bf1
 template <class T, int D, int NST, bool MR, bool CH, bool TO>
 static hipError_t bwd2_mr(const BwdArgs<T>& a, int Lp, int Zk, hipStream_t s) {
   // two key groups per workgroup once every CU gets at least two of the single ones
-  const int n_kg = Lp / 128, gx = (long)n_kg * Zk >= 2 * device_cus() ? (n_kg + 1) / 2 : n_kg;
+    const int n_kg = Lp / 128, gx = (long)n_kg * Zk >= 2 * device_cus() ? (n_kg + 1) / 2 : n_kg;
   hipLaunchKernelGGL((k_bwd_keys2<T, D, NST, MR, CH, TO>), dim3(gx, Zk), dim3(512), 0, s, a);
   return hipGetLastError();
 }
@@ -118,7 +118,15 @@ template __global__ void k_bwd_queries3<bf16, 256, 2, 1>(BwdArgs<bf16>, bf16*, i
 template __global__ void k_bwd_queries3<bf16, 128, 2, 2>(BwdArgs<bf16>, bf16*, int);
 hipError_t launch_bwd_queries_from_tiles(int D, const BwdArgsV& v, void* dq, int d, int Zq, hipStream_t s, int variant) {
   const BwdArgs<bf16> a = typed<bf16>(v);
-  const dim3 grid(v.Lp / 128, Zq);
+  // steps of 32 keys (two workgroups per CU): four query blocks per workgroup once every CU gets at least eight of the
+  // single ones, two once it gets four; steps of 64 keys: one block per workgroup
+  const int n_blk = v.Lp / 128;
+  const long n_wg = (long)n_blk * Zq;
+  const bool half_steps = !(variant == 1 && D != 256);
+  const int gx = !half_steps ? n_blk
+                 : (n_blk % 4 == 0 && n_wg >= 8L * device_cus()) ? n_blk / 4
+                 : n_wg >= 4L * device_cus() ? (n_blk + 1) / 2 : n_blk;
+  const dim3 grid(gx, Zq);
 #define UA_Q3(D_, HV_) hipLaunchKernelGGL((k_bwd_queries3<bf16, D_, 2, HV_>), grid, dim3(512), 0, s, a, (bf16*)dq, d)
   if (D == 256) UA_Q3(256, 1);              // steps of 32 keys only: a stage of 64 keys would not fit twice
   else if (variant == 1) { if (D == 64) UA_Q3(64, 2); else UA_Q3(128, 2); }
