@@ -253,7 +253,7 @@ template <class T> struct ChunkOut {
 // is uniform there: out = mean of the chunk's values (through a dtype-rounded 1/c), denom = float32(-1e12).
 // grid (ceil(max rows / kMaskedSlab), nch, Zq), 256 threads: slab x of chunk i writes rows [x kMaskedSlab, (x + 1) kMaskedSlab)
 // ∩ [0, i*c) of out[.., i].  vec: rows of out[.., i] are contiguous in dd, 16-byte aligned and d is a multiple of the vector.
-constexpr int kMaskedSlab = 1024;
+constexpr int kMaskedSlab = 4096;
 template <class T, int D>
 __global__ void __launch_bounds__(256) k_chunk_masked_out(const T* __restrict__ Vp, ChunkOut<T> co, int R, int L, int Lp, int d,
                                                           int vec) {
@@ -289,6 +289,17 @@ __global__ void __launch_bounds__(256) k_chunk_masked_out(const T* __restrict__ 
   T* base = co.out + (long)zq * co.sz + (long)i * co.si;
   if (vec) {
     const int vpr = d / V;                                      // vectors per row
+    if (256 % vpr == 0) {
+      // a thread keeps its piece of the row in registers and walks down the rows: nothing but stores in the loop (plain
+      // ones: 6 % faster here than non-temporal ones; slabs of 4096 rows instead of 1024: the mean is computed a quarter
+      // as often; together 0.55 -> 0.43 ms for the 2.15 GB of the headline shape with chunk 128)
+      const int cv = tid % vpr, rstep = 256 / vpr;
+      const u32x4 val = *reinterpret_cast<const u32x4*>(mean + cv * V);
+      T* p = base + (long)(r0 + tid / vpr) * co.st + cv * V;
+      const long pstep = (long)rstep * co.st;
+#pragma unroll 8
+      for (int t = r0 + tid / vpr; t < r1; t += rstep, p += pstep) *reinterpret_cast<u32x4*>(p) = val;
+    } else
     for (int idx = tid; idx < (r1 - r0) * vpr; idx += 256) {
       const int t = r0 + idx / vpr, cv = idx % vpr;
       // written once and read by nobody in the reference's call sequence (the merge skips slices of zero weight)
