@@ -363,13 +363,16 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW
   // wave w: block w / (2 RB) of the workgroup, query group (w / 2) % RB of the workgroup's RB, half w % 2 of the block
   const int zq = RB == 1 ? zy : (zy / (R / RB)) * R + (zy % (R / RB)) * RB + (w >> 1) % RB;
   const int zk = zq / R, nT16 = Lp / 16;
-  const int jt = gridDim.x - 1 - bx;
+  // chunked operator, 16-bit outputs: per-wave [16 queries][D + 8] tile through which a chunk's result is transposed
+  __shared__ __attribute__((aligned(16))) T sObuf[(CHUNKED && sizeof(T) == 2) ? NW * 16 * (D + 8) : 8];
+  const int n_blk = (nT16 + NW - 1) / NW;                    // workgroup blocks of 16 NW queries
+  // chunked operator: a workgroup may handle two blocks of complementary length, jt and n_blk - 1 - jt, the body
+  // expanded once per block (see k_bwd_keys2)
+  auto sweep = [&](const int jt) __attribute__((always_inline)) {
   const int blk = w / (2 * RB), wb = w % (2 * RB), tq_raw = 2 * (NB * jt + blk) + (w & 1);
   const bool live = tq_raw < nT16;                           // the last workgroup may hold waves past the end
   const int tq = live ? tq_raw : nT16 - 1;                   // 16-query tile of this wave
   char* sPw = sPbuf + w * 2 * ST::BYTES;     // P of the two 32-key halves of a step
-  // chunked operator, 16-bit outputs: per-wave [16 queries][D + 8] tile through which a chunk's result is transposed
-  __shared__ __attribute__((aligned(16))) T sObuf[(CHUNKED && sizeof(T) == 2) ? NW * 16 * (D + 8) : 8];
   T* sOw = sObuf + ((CHUNKED && sizeof(T) == 2) ? w * 16 * (D + 8) : 0);
   const GroupMasks gm = group_masks(lane);
   Stager<TN, NW> stN;
@@ -604,6 +607,16 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW
       lse2[(long)zq * Lp + t] = (t < L) ? l2v : 0.f;
       if (t < L) lse[(long)zq * L + t] = l2v * kLn2;
     }
+  }
+  };
+  if constexpr (CHUNKED) {
+    sweep(n_blk - 1 - bx);                                   // heaviest first
+    if ((int)gridDim.x != n_blk && n_blk - 1 - bx != bx) {
+      __syncthreads();       // the stages are free
+      sweep(bx);
+    }
+  } else {
+    sweep((int)gridDim.x - 1 - bx);
   }
 }
 

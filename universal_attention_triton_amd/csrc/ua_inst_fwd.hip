@@ -156,7 +156,9 @@ static hipError_t chunked2_t(const void* Qp, const void* Kp, const void* Vp, con
   constexpr long VV = 16 / (long)sizeof(T);
   const int ovec = out && o_sd == 1 && d % VV == 0 && (uintptr_t)out % 16 == 0 && o_sz % VV == 0 && o_st % VV == 0 && o_si % VV == 0;
   ChunkOut<T> co{(T*)out, (T*)denom, o_sz, o_st, o_sd, o_si, c, nch, ovec};
-  hipLaunchKernelGGL((k_fwd_fused2<T, D, NST, NW, true>), dim3((Lp / 16 + NW - 1) / NW, Zq), dim3(64 * NW), 0, s, (const T*)Qp,
+  // two query blocks per workgroup once every CU gets at least four of the single ones
+  const int n_blk = (Lp / 16 + NW - 1) / NW, gx = (long)n_blk * Zq >= 4L * device_cus() ? (n_blk + 1) / 2 : n_blk;
+  hipLaunchKernelGGL((k_fwd_fused2<T, D, NST, NW, true>), dim3(gx, Zq), dim3(64 * NW), 0, s, (const T*)Qp,
                      (const T*)Kp, (const T*)VT, lsrc, ldest, C, (T*)nullptr, (float*)nullptr, lse2, reach, minkey, R, L, Lp, d, co, (const _Float16*)nullptr);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
