@@ -194,7 +194,8 @@ int ua_affinity_bwd(const ua_desc* desc, const ua_rows* k, const void* src, cons
 enum {
   UA_TUNE_FWD_RECOMPUTE = 2, /* == UA_OP_FUSED_FWD.  Forward without bias tiles (fp32, UA_FLAG_RECOMPUTE): bf16 0 = 8 waves
                                 two LDS stages, 1 = 8 waves one stage, 2 = 12 waves, 3 = 16 waves, 4 = 4 waves; fp32: one */
-  UA_TUNE_CARRY = 16,        /* bias pre-pass of the bf16 operator: 0 = 8 waves x 16 keys per workgroup, 1 = 4 waves */
+  UA_TUNE_CARRY = 16,        /* bias pre-pass of the bf16 operator: 0 = 8 waves x 16 keys per workgroup, 1 = 4 waves,
+                                2 = 4 waves, two key groups of complementary length per workgroup */
   UA_TUNE_FWD_TILES = 17,    /* bf16 forward over bias tiles: 0 = one 32-query block per wave (256-query workgroups, two
                                 LDS stages), 1 = 16 queries per wave (128-query workgroups, one stage, two per CU),
                                 2 = 16 queries per wave, 64-query workgroups (r = 1 only) */

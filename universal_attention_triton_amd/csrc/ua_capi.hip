@@ -86,7 +86,7 @@ int n_variants(const ua_desc& d, int slot) {
   const bool bf = d.dtype == UA_BF16;
   switch (slot) {
     case UA_TUNE_FWD_RECOMPUTE: return ua::fwd_fused_variants(d.dtype, padded_dim(d.d));
-    case UA_TUNE_CARRY: return bf ? 2 : 1;
+    case UA_TUNE_CARRY: return bf ? 3 : 1;
     case UA_TUNE_FWD_TILES: return bf ? (d.d > 128 ? 1 : (d.r % 2 == 0 ? 2 : 3)) : 1;     // above 128: 16 queries per wave only
     case UA_TUNE_BWD_PARTS: return bf ? n_divisors(d.r) : 1;
     case UA_TUNE_BWD_QUERIES: return bf && d.d <= 128 ? 2 : 1;
@@ -104,8 +104,10 @@ int heuristic_variant(const ua_desc& d, int slot) {
   const long Zk = (long)d.b * d.h, Zq = Zk * d.r;
   const int Lp = (int)align_up((size_t)d.L, 128);
   switch (slot) {
-    case UA_TUNE_CARRY:      // under two 8-wave workgroups per CU the sweep latency of a workgroup bounds the launch
-      return Zk * (Lp / 128) < 512 ? 1 : 0;
+    case UA_TUNE_CARRY: {    // 4-wave workgroups won at every tuned shape; two key groups each when the single ones make
+      const long n4 = Zk * (Lp / 64);      // one to four rounds of the 1024 resident workgroups
+      return (n4 >= 1024 && n4 < 4096) ? 2 : 1;
+    }
     case UA_TUNE_FWD_TILES:  // 256-query workgroups need about four per CU to balance; small launches run 64-query pieces
       if (Zq * (Lp / 256) >= 1024) return 0;
       return (d.r % 2 == 0 || Zq * (Lp / 128) >= 1536) ? 1 : 2;

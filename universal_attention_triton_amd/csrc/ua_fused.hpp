@@ -110,8 +110,16 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2)
   constexpr int NK = D / 32, SB = TN::BYTES + 1024;   // tile + [ldest of the block: 32 floats]
   UA_STAGES(SB);
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 15, g = lane >> 4;
-  int bx, z;
-  xcd_map(bx, z);
+  // A launch of half as many workgroups has each sweep two key groups, bx and (number of key groups - 1 - bx), one after
+  // the other with the body expanded once per key group (see k_bwd_keys2).  It pays in small launches (b = 2, h = 16,
+  // L = 2048, d = 64: 0.074 -> 0.056 ms) and costs in large ones (b = 1, h = 32, L = 8192: 0.70 -> 0.83 ms), so it is a
+  // variant of the tuning slot.
+  int bx0, z;
+  xcd_map(bx0, z);
+  const int n_kg = Lp / (16 * NW);
+  __shared__ int n_dead;
+  __shared__ float red[2][NW];
+  auto sweep = [&](const int bx) __attribute__((always_inline)) {
   const int nT = Lp / 32, nT16 = Lp / 16, sb16 = NW * bx + w, first = (NW / 2) * bx;
   const int spos = 16 * sb16 + col;
   const GroupMasks gm = group_masks(lane);
@@ -133,8 +141,6 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2)
   const T* Kz = Kp + (long)z * Lp * D;
   bool dead = false;
   int last = sb16 >> 1;
-  __shared__ int n_dead;
-  __shared__ float red[2][NW];
   float thr = -3.0e38f;
   if (tid == 0) n_dead = 0;
   if (knorm2) {
@@ -227,6 +233,12 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2)
 #undef UA_COMPUTE_FAST
 #undef UA_COMPUTE_SLOW
   if (reach && lane == 0) reach[z * nT16 + sb16] = last;
+  };
+  sweep(bx0);
+  if ((int)gridDim.x != n_kg && n_kg - 1 - bx0 != bx0) {
+    __syncthreads();       // the stages, n_dead and red are free
+    sweep(n_kg - 1 - bx0);
+  }
 }
 
 // minkey[z][tb] = first key tile (of 16) that reaches query block tb; it never decreases with tb.

@@ -21,8 +21,9 @@ static hipError_t carry_t(const void* Kp, const float* lsrc, const float* ldest,
   _Float16* none = nullptr;
   // bias tiles, variant 1: 4-wave workgroups (launches of under two 8-wave workgroups per CU are bound by the latency
   // of a workgroup's serial sweep and run faster as twice as many 4-wave workgroups)
-  if (tiled && Bt && sizeof(T) == 2 && variant == 1)
-    hipLaunchKernelGGL((k_carry2<T, D, NST, true, true, 4>), dim3(Lp / 64, Zk), dim3(256), 0, s, (const T*)Kp, lsrc, ldest, C, Lp, knorm2, qnorm2, R, reach, (_Float16*)Bt);
+  // variant 2: the same with two key groups per workgroup (half the workgroups; pays in small launches)
+  if (tiled && Bt && sizeof(T) == 2 && (variant == 1 || variant == 2))
+    hipLaunchKernelGGL((k_carry2<T, D, NST, true, true, 4>), dim3(variant == 2 ? (Lp / 64 + 1) / 2 : Lp / 64, Zk), dim3(256), 0, s, (const T*)Kp, lsrc, ldest, C, Lp, knorm2, qnorm2, R, reach, (_Float16*)Bt);
   else if (tiled && Bt && sizeof(T) == 2) hipLaunchKernelGGL((k_carry2<T, D, NST, true, true>), dim3(Lp / 128, Zk), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, C, Lp, knorm2, qnorm2, R, reach, (_Float16*)Bt);
   else if constexpr (D == 256) return hipErrorInvalidValue;
   else if (tiled) hipLaunchKernelGGL((k_carry2<T, D, NST, true, false>), dim3(Lp / 128, Zk), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, C, Lp, knorm2, qnorm2, R, reach, none);
