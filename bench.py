@@ -355,10 +355,11 @@ def main():
         out["roofline"] = roof
         out["config"]["workload"] += "; chunked API (reference call sequence, chunk %d)" % cfg["c"]
         out["config"].pop("pct_of_mfma_peak", None)
-        # the same sequence with the whole forward state kept for the backward (keep_state = True: + one forward state of
-        # memory between the two, no second decay pre-pass and no repacking in the backward)
-        from universal_attention_triton_amd import universal_attention_autograd as own_api
-        own_api._ChunkedBase.keep_state = True
+        # the same sequence with only the float32 normalisers kept for the backward instead of the whole forward state
+        # (1/(d+1) of the size of `out`; the backward then repacks the inputs and repeats the decay pre-pass)
+        from universal_attention_triton_amd import ops, universal_attention_autograd as own_api
+        default_keep = own_api._ChunkedBase.keep_state
+        own_api._ChunkedBase.keep_state = "normalisers"
         try:
             n_full = max(3, args.steps // 4)
             for _ in range(2):
@@ -368,10 +369,14 @@ def main():
             for _ in range(n_full):
                 step()
             torch.cuda.synchronize()
-            out["config"]["keep_state_true"] = {"ms_per_step": round((time.perf_counter() - t0) * 1e3 / n_full, 4),
-                                                "note": "optional: forward state retained for the backward; not `value`"}
+            out["config"]["keep_state_normalisers"] = {"ms_per_step": round((time.perf_counter() - t0) * 1e3 / n_full, 4),
+                                                       "note": "optional: only the normalisers retained for the backward; not `value`"}
         finally:
-            own_api._ChunkedBase.keep_state = "normalisers"
+            own_api._ChunkedBase.keep_state = default_keep
+        out["config"]["bytes_retained_fwd_to_bwd"] = {
+            "forward_state": int(ops.retained_bytes(*[x.detach() for x in leaves], chunked=True)),
+            "out_and_denom": int(cfg["b"] * cfg["h"] * cfg["r"] * cfg["L"] * (cfg["d"] + 1) * (cfg["L"] // cfg["c"])
+                                 * (2 if cfg["dtype"] == "bf16" else 4))}
         if not args.no_cpu:
             out["cpu_baseline"] = cpu_baseline(cfg, args.config)
         print(json.dumps(out))

@@ -282,6 +282,41 @@ def test_out_allocated_contiguous_like_the_reference(dtype):
             assert rel_err(x.reshape(w.shape), w) <= TOL[dtype], (name, rel_err(x.reshape(w.shape), w))
 
 
+@pytest.mark.parametrize("dtype,c", [(torch.float32, 64), (torch.bfloat16, 128), (torch.bfloat16, 32)])
+def test_what_the_chunked_function_keeps_for_its_backward_does_not_change_the_gradients(dtype, c):
+    """The chunked Functions keep the whole forward state by default; with only the normalisers, or nothing, the
+    backward rebuilds what it misses from the five inputs and must arrive at the same gradients, bit for bit where
+    the kernels add in a fixed order (chunk a multiple of 64; the others add up dq with atomics)."""
+    from universal_attention_triton_amd import universal_attention_autograd as ua
+    print("case chunked keep modes", dtype, c, flush=True)
+    b, h, r, L, d = 1, 2, 2, 384, 64
+    n = L // c
+    inp = orc.make_inputs(b, h, r, L, d, c, dtype=dtype, seed=31)
+    g = torch.Generator().manual_seed(5)
+    g_out = torch.randn(b, h, r, L, d, n, generator=g).to(dtype).cuda()
+    g_denom = torch.randn(b, h, r, L, n, generator=g).to(dtype).cuda()
+    assert ua._ChunkedBase.keep_state is True
+    results = []
+    for keep in (True, "normalisers", False):
+        ua._ChunkedBase.keep_state = keep
+        try:
+            leaves = [inp[k].cuda().requires_grad_() for k in NAMES]
+            out, denom = ua.UniversalAttention.apply(*leaves)
+            grads = torch.autograd.grad([out, denom], leaves, [g_out, g_denom])
+            torch.cuda.synchronize()
+            results.append((out.detach().clone(), grads))
+        finally:
+            ua._ChunkedBase.keep_state = True
+    for o, grads in results[1:]:
+        assert torch.equal(o, results[0][0])
+        for name, x, y in zip(NAMES, grads, results[0][1]):
+            assert torch.equal(x, y) if c % 64 == 0 else rel_err(x, y) <= 2.0 ** -7, (name, rel_err(x, y))
+    want = orc.chunked_backward(*[inp[k].float() for k in NAMES], g_out.float().cpu(), g_denom.float().cpu())
+    for name, x, w in zip(NAMES, results[0][1], want):
+        if name != "kc" or dtype == torch.bfloat16:      # float32 dkc has its own bar in test_hip_backward.py
+            assert rel_err(x.reshape(w.shape), w) <= TOL[dtype], (name, rel_err(x.reshape(w.shape), w))
+
+
 @pytest.mark.parametrize("shape", [(1, 2, 2, 512, 64, 64), (1, 1, 1, 768, 128, 192), (2, 1, 1, 256, 128, 128)])
 def test_upstream_gradient_read_in_place_equals_its_packed_copy(shape):
     """bf16, chunk a multiple of 64, nothing flowing to (query, later chunk) pairs: a chunk-major upstream gradient with

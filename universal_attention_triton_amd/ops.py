@@ -251,13 +251,14 @@ def fused_backward(kc, vc, xq, static_src, static_dest, O, lse, dO, state=None, 
     return dk, dv, dq, dsrc.to(src_dtype), ddest.to(dest_dtype)
 
 
-def retained_bytes(kc, vc, xq, static_src, static_dest, recompute=False):
-    """Bytes of forward state the fused operator keeps alive between forward and backward (0 with recompute)."""
+def retained_bytes(kc, vc, xq, static_src, static_dest, recompute=False, chunked=False):
+    """Bytes of forward state the fused operator (chunked=True: the chunked operator with keep_state=True) keeps alive
+    between forward and backward (fused operator with recompute: 0)."""
     kc, vc, xq, src, dest, gflag = _prep(kc, vc, xq, static_src, static_dest)
-    if recompute:
+    if recompute and not chunked:
         return 0
-    desc = _desc(kc, xq, False, gflag)
-    return _lib.load().ua_workspace_bytes(ctypes.byref(desc), _lib.UA_OP_FUSED_FWD)
+    desc = _desc(kc, xq, chunked, gflag | (_lib.UA_FLAG_RECOMPUTE if recompute else 0))
+    return _lib.load().ua_workspace_bytes(ctypes.byref(desc), _lib.UA_OP_FWD if chunked else _lib.UA_OP_FUSED_FWD)
 
 
 def _merge_views(mat):

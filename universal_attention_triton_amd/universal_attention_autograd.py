@@ -41,10 +41,13 @@ class _ChunkedBase(Function):
     # recomputes the score and decay gradients instead of reading them from 2*L*L bytes per head)
     recompute = False
     # What the backward gets from the forward besides the five inputs the reference keeps (universal_attention.py:27-31)
-    # and `out`: "normalisers" (default): the per-chunk normalisers in float32, 1/(d+1) of the size of `out`, which spare
-    # the backward a second run of the forward kernel; True: the whole forward state (ua_workspace_bytes(UA_OP_FWD)
-    # bytes: packed inputs, decay carries, normalisers); False: nothing.
-    keep_state = "normalisers"
+    # and `out`: True (default, like the fused operator): the whole forward state (ua_workspace_bytes(UA_OP_FWD) bytes:
+    # packed inputs, decay carries of L * L / 4 bytes per kv head, float32 normalisers; 0.94 GB next to the 4.3 GB of
+    # `out` at b=1 h=32 L=8192 d=128 chunk 128), so the backward neither repacks the inputs nor repeats the decay
+    # pre-pass; "normalisers": only the
+    # per-chunk normalisers in float32, 1/(d+1) of the size of `out`, which spare the backward a second run of the
+    # forward kernel; False: nothing.
+    keep_state = True
     # `out` is stored chunk-major ([b,h,r,n,L,d]) and returned as a permuted view with the reference's shape and values:
     # every kernel then moves 16 bytes per lane.  True allocates it contiguous like the reference does, for callers
     # that `.view()` it; the passes over it are then several times slower.
