@@ -9,8 +9,10 @@ from tests.util import TOL, rel_err
 pytestmark = pytest.mark.gpu
 
 # b, h, L, d (ragged L, padded d).  bf16 with L a multiple of 8 runs the tile-exchanging backward, everything else the one
-# with the float L x L running sum.
-SHAPES = [(1, 2, 64, 16), (2, 2, 192, 64), (1, 1, 320, 80), (1, 2, 517, 128), (1, 2, 1032, 128)]
+# with the float L x L running sum.  The last two launch more workgroups than the part has CUs, so that every workgroup
+# takes two key groups of complementary length (5 and 3 groups: the middle one stays alone).
+SHAPES = [(1, 2, 64, 16), (2, 2, 192, 64), (1, 1, 320, 80), (1, 2, 517, 128), (1, 2, 1032, 128), (1, 66, 520, 64),
+          (2, 44, 384, 128)]
 
 
 def _inputs(b, h, L, d, dtype, seed):
