@@ -185,6 +185,37 @@ def test_memory_kept_between_forward_and_backward_at_the_headline_shape():
         assert torch.cuda.memory_allocated() - base <= (8 << 20)
 
 
+def test_memory_kept_between_forward_and_backward_by_the_chunked_functions():
+    """bf16, b=1 h=8 L=4096 d=128 chunk 128: between forward and backward the chunked Function holds its inputs, `out`,
+    `denom` (what the reference holds too) and, by default, the forward state (ops.retained_bytes(chunked=True): packed
+    inputs, decay carries, normalisers); with "normalisers" only those (1/(d+1) of `out`), with False nothing more."""
+    from universal_attention_triton_amd import ops
+    from universal_attention_triton_amd import universal_attention_autograd as ua
+    b, h, r, L, d, c = 1, 8, 1, 4096, 128, 128
+    n = L // c
+    inp = orc.make_inputs(b, h, r, L, d, c, dtype=torch.bfloat16, seed=1003)
+    leaves = [inp[k_].cuda().requires_grad_() for k_ in NAMES]
+    torch.cuda.synchronize()
+    base = torch.cuda.memory_allocated()
+    out_bytes = b * h * r * L * (d + 1) * n * 2
+    state = ops.retained_bytes(*[x.detach() for x in leaves], chunked=True)
+    assert state < out_bytes // 3
+    slack = 8 << 20
+    for keep, extra in ((True, state), ("normalisers", b * h * r * n * L * 4), (False, 0)):
+        ua._ChunkedBase.keep_state = keep
+        try:
+            out, denom = ua.UniversalAttention.apply(*leaves)
+            torch.cuda.synchronize()
+            held = torch.cuda.memory_allocated() - base
+            assert out_bytes + extra - slack <= held <= out_bytes + extra + slack, (keep, held, out_bytes, extra)
+            grads = torch.autograd.grad([out, denom], leaves, [torch.ones_like(out), torch.zeros_like(denom)])
+            del out, denom, grads
+            torch.cuda.synchronize()
+            assert torch.cuda.memory_allocated() - base <= slack
+        finally:
+            ua._ChunkedBase.keep_state = True
+
+
 @pytest.mark.parametrize("shape", [(1, 2, 1, 320, 160), (1, 1, 2, 200, 256), (2, 1, 4, 128, 136)])
 def test_head_dims_above_128_bf16_fused_operator(shape):
     """The reference's second-generation kernel takes head dims up to 256 (zero-padded to a power of two,
