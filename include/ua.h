@@ -202,8 +202,11 @@ enum {
   UA_TUNE_BWD_PARTS = 18,    /* key side of the bf16 backward with r > 1: variant i divides the query groups of a kv
                                 head into the i-th smallest divisor of r parts with a sweep each (0 = one shared sweep).
                                 Changes ua_workspace_bytes: set it before sizing the workspace. */
-  UA_TUNE_BWD_QUERIES = 19   /* query side of the bf16 backward over gradient tiles: 0 = steps of 32 keys, two workgroups
+  UA_TUNE_BWD_QUERIES = 19,  /* query side of the bf16 backward over gradient tiles: 0 = steps of 32 keys, two workgroups
                                 per CU; 1 = steps of 64 keys, one workgroup per CU */
+  UA_TUNE_BWD_KEYS = 20      /* key side of the bf16 backward over bias tiles, r = 1, head dim 65..128: 0 = 16 keys per
+                                wave on 16x16 tiles, two waves per SIMD; 1 = 32 keys per wave on 32x32 tiles, one wave per
+                                SIMD, the step laid out by hand */
 };
 /* ua_autotune(desc, op, ...) with op = UA_OP_FUSED_FWD or UA_OP_FUSED_BWD times every variant of every kernel slot on
  * that op's path for desc (hipEvents on `stream`, synchronises) and records the fastest of each.  `ws` must hold what

@@ -15,10 +15,19 @@ GRADS = ("dkc", "dvc", "dxq", "dsrc", "ddest")
 
 
 def _table(tag, got, want, tol):
+    """tol: one bar for the five gradients, or {gradient: bar} (missing names take the "*" entry)"""
     errs = {n: rel_err(g.reshape(w.shape), w) for n, g, w in zip(GRADS, got, want)}
-    print(tag, {k: "%.2e" % v for k, v in errs.items()}, flush=True)
-    bad = {k: v for k, v in errs.items() if not v <= tol}
+    bars = {n: (tol.get(n, tol.get("*")) if isinstance(tol, dict) else tol) for n in GRADS}
+    print(tag, {k: "%.2e (bar %.1e)" % (v, bars[k]) for k, v in errs.items()}, flush=True)
+    bad = {k: (v, bars[k]) for k, v in errs.items() if not v <= bars[k]}
     assert not bad, (tag, bad)
+
+
+def _fp32_key_gradient_bar(oracle_dkc, exact_dkc):
+    """float32 bar of the key gradient: d/dG relu(G)^(2/3) is singular at G -> 0+, and the reference's own float32
+    operator misses float64 by more than 1e-4 on random keys; the kernel gets twice the error of the oracle's float32
+    restatement on the same inputs, and never less than the plain 1e-4.  Every other gradient is held to 1e-4."""
+    return max(1e-4, 2 * rel_err(oracle_dkc, exact_dkc))
 
 
 @pytest.mark.parametrize("entry", ["autograd2", "triton_side"])
@@ -31,7 +40,7 @@ def test_backward_through_the_2d_layout_matches_reference_golden(name, entry):
     from universal_attention_triton_amd.universal_attention import UniversalAttention as TritonSide
     t, dtype, (b, h, r, l, d, c, seed) = load_golden(name)
     qc = int(np.load(os.path.join(os.path.dirname(__file__), "golden", name + ".npz"))["qc"][0])
-    tol = TOL[dtype] if dtype == torch.float32 else 2.5e-2     # bf16: the golden carries the reference's own bf16 noise
+    tol = TOL[dtype]
     fn = ua.UniversalAttention2 if entry == "autograd2" else TritonSide
     xq2 = t["xq"].to(dtype).view(b, h, r, l // qc, qc, d)
     sd2 = t["static_dest"].to(dtype).view(b, h, l // qc, qc)
@@ -55,13 +64,20 @@ def test_backward_through_the_2d_layout_matches_oracle_larger_case(dtype):
     g_out = torch.randn(b, h, r, L, d, L // c, generator=g).to(dtype)
     g_denom = torch.randn(b, h, r, L, L // c, generator=g).to(dtype)
     want = orc.chunked_backward(*[inp[k].float() for k in NAMES], g_out.float(), g_denom.float())
+    tol = TOL[dtype]
+    if dtype == torch.float32:
+        # arbitrary upstream on the chunked operator: the -1e12 fill only swamps the score in float32, so float64 cannot
+        # serve; the restatement's own float32 error in the key gradient is measured as its largest move under other
+        # summation orders of the head dimension (same mathematics, other rounding of the key-key products)
+        from tests.test_hip_backward import _summation_order_sensitivity
+        tol = {"*": 1e-4, "dkc": max(1e-4, 2 * _summation_order_sensitivity(inp, g_out, g_denom.float(), want[0]))}
     xq2 = inp["xq"].view(b, h, r, L // qc, qc, d)
     sd2 = inp["static_dest"].view(b, h, L // qc, qc)
     leaves = [x.cuda().requires_grad_() for x in (inp["kc"], inp["vc"], xq2, inp["static_src"], sd2)]
     out, denom = ua.UniversalAttention2.apply(*leaves)
     grads = torch.autograd.grad([out, denom], leaves, [g_out.cuda(), g_denom.cuda()])
     torch.cuda.synchronize()
-    _table("2-D layout oracle %s" % dtype, grads, want, 4e-4 if dtype == torch.float32 else TOL[dtype])
+    _table("2-D layout oracle %s" % dtype, grads, want, tol)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -72,6 +88,11 @@ def test_all_five_gradients_through_the_qkv_calling_convention(dtype):
     B, Hkv, r, L, d = 1, 2, 3, 200, 80
     inp = orc.make_inputs(B, Hkv, r, L, d, 8, dtype=dtype, seed=43)
     O_ref, _, g_ref = dense_reference(inp)
+    tol = TOL[dtype]
+    if dtype == torch.float32:
+        out32, denom32 = orc.chunked_forward(*[inp[k_] for k_ in NAMES])
+        d_out, d_denom = orc.merge_backward(out32, denom32, inp["dO"])
+        tol = {"*": 1e-4, "dkc": _fp32_key_gradient_bar(orc.chunked_backward(*[inp[k_] for k_ in NAMES], d_out, d_denom)[0], g_ref[0])}
     k = inp["kc"].reshape(B, Hkv, L, d).cuda().requires_grad_()
     v = inp["vc"].reshape(B, Hkv, L, d).cuda().requires_grad_()
     q = inp["xq"].transpose(1, 2).reshape(B, r * Hkv, L, d).cuda().requires_grad_()       # head j = rep * Hkv + kv
@@ -85,7 +106,7 @@ def test_all_five_gradients_through_the_qkv_calling_convention(dtype):
         torch.cuda.synchronize()
         assert rel_err(o.view(B, r, Hkv, L, d).transpose(1, 2), O_ref) <= TOL[dtype]
         got = [gk, gv, gq.view(B, r, Hkv, L, d).transpose(1, 2), gs, gd]
-        _table("attention() %s ac=%s" % (dtype, ac), got, g_ref, 4e-4 if dtype == torch.float32 else TOL[dtype])
+        _table("attention() %s ac=%s" % (dtype, ac), got, g_ref, tol)
         results.append(got)
     for a_, b_ in zip(*results):
         assert rel_err(a_, b_) <= (1e-5 if dtype == torch.float32 else 2e-3)
@@ -398,5 +419,5 @@ def test_launches_of_paired_work_items_with_an_odd_number_of_items(shape):
         one = {k: v[:, hh:hh + 1] for k, v in inp.items()}
         O_ref, lse_ref, g_ref = dense_reference(one)
         assert rel_err(O[:, hh:hh + 1], O_ref) <= TOL[bf], hh
-        assert float((lse[:, hh:hh + 1].cpu().double() - lse_ref).abs().max()) <= 10 * TOL[bf], hh
+        assert float((lse[:, hh:hh + 1].cpu().double() - lse_ref).abs().max()) <= TOL[bf], hh
         _table("head %d of %s" % (hh, (shape,)), [x[:, hh:hh + 1] for x in grads], g_ref, TOL[bf])

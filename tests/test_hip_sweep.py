@@ -46,6 +46,7 @@ def _reference_bars(inp, dtype, exact, tol):
 def test_fused_operator_random_shapes_and_flags():
     from universal_attention_triton_amd import ops
     rng = random.Random(20260)
+    relaxed = []          # cases judged by the reference algorithm's own error instead of the plain tolerance
     for it in range(40):
         b, h, r = rng.choice([1, 1, 2]), rng.choice([1, 2, 3]), rng.choice([1, 1, 2, 3, 4])
         L = rng.choice(LENGTHS)
@@ -67,7 +68,7 @@ def test_fused_operator_random_shapes_and_flags():
         torch.cuda.synchronize()
         O_ref, lse_ref, g_ref = dense_reference(inp)
         tol = TOL[dtype]
-        errs = {"O": rel_err(O, O_ref), "lse": float((lse.cpu().double() - lse_ref).abs().max()) / 10}
+        errs = {"O": rel_err(O, O_ref), "lse": float((lse.cpu().double() - lse_ref).abs().max())}
         for k, g, gr in zip(NAMES, grads, g_ref):
             if float(gr.abs().max()) == 0.0:        # L = 1: every gradient is exactly zero; here rounding noise of dP - delta
                 errs["d" + k] = float(g.float().abs().max().cpu()) * tol
@@ -77,11 +78,16 @@ def test_fused_operator_random_shapes_and_flags():
         if any(errs[k] > tol for k in errs if k.startswith("d")) and L > 1:
             # ill-conditioned inputs: hold the gradients to what the reference algorithm itself achieves in this dtype
             # (test_hip_paths holds dkc to 1e-4 on well-conditioned keys)
-            bars.update(_reference_bars(inp, dtype, g_ref, tol))
-            if dtype == torch.float32:
-                bars["dkc"] = max(4e-4, bars["dkc"])
+            missed = sorted(k for k in errs if k.startswith("d") and errs[k] > tol)
+            ref_bars = _reference_bars(inp, dtype, g_ref, tol)
+            for k in missed:          # only the tensors that missed take the reference's own error as their bar
+                bars[k] = ref_bars[k]
+            relaxed.append((it, case["shape"], case["dtype"], {k: "%.2e (bar %.2e)" % (errs[k], bars[k]) for k in missed}))
+            print("   relaxed:", relaxed[-1], flush=True)
         bad = {k: (v, bars[k]) for k, v in errs.items() if not v <= bars[k]}
         assert not bad, (case, bad)
+    print("cases judged by the reference algorithm's own error: %d of 40" % len(relaxed), relaxed, flush=True)
+    assert len(relaxed) <= 8, relaxed
 
 
 def test_chunked_operator_random_shapes_and_upstreams():

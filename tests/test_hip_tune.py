@@ -28,9 +28,12 @@ def test_every_variant_of_every_slot_on_the_default_path_meets_the_oracle(shape)
     a = [inp[k].cuda() for k in NAMES]
     dO = inp["dO"].cuda()
     O_ref, lse_ref, g_ref = dense_reference(inp)
-    for slot in ("carry", "fwd_tiles", "bwd_parts", "bwd_queries"):
+    for slot in ("carry", "fwd_tiles", "bwd_parts", "bwd_queries", "bwd_keys"):
         n = ops.tune_variants(a[0], a[2], slot)
-        assert n >= (1 if slot == "bwd_parts" and r == 1 else 2), (slot, n)
+        if slot == "bwd_keys":
+            assert n == (2 if r == 1 and d > 64 else 1), (slot, n)
+        else:
+            assert n >= (1 if slot == "bwd_parts" and r == 1 else 2), (slot, n)
         for v in range(n):
             ops.tune_set(a[0], a[2], v, slot)
             try:
@@ -61,7 +64,7 @@ def test_recomputing_forward_variants_agree_and_autotune_records_a_choice_per_sl
     for v in range(1, n):
         assert rel_err(results[v], results[0]) <= 2e-3, v            # same arithmetic, different summation order
     chosen = ops.autotune(*a)
-    assert set(chosen) == {"carry", "fwd_tiles", "bwd_parts", "bwd_queries"}, chosen
+    assert set(chosen) == {"carry", "fwd_tiles", "bwd_parts", "bwd_queries"}, chosen      # r = 2: one key-side variant
     for slot, v in chosen.items():
         assert 0 <= v < ops.tune_variants(a[0], a[2], slot) and ops.tune_choice(a[0], a[2], slot) == v
     O, _, _ = ops.fused_forward(*a)
@@ -90,7 +93,7 @@ def test_shipped_table_is_within_3_percent_of_autotune_on_this_device(cfg):
     inp = orc.make_inputs(b, h, r, L, d, 128, dtype=BF, seed=seed)
     a = [inp[k].cuda() for k in NAMES]
     dO = inp["dO"].cuda()
-    slots = [s for s in ("carry", "fwd_tiles", "bwd_parts", "bwd_queries") if ops.tune_variants(a[0], a[2], s) > 1]
+    slots = [s for s in ("carry", "fwd_tiles", "bwd_parts", "bwd_queries", "bwd_keys") if ops.tune_variants(a[0], a[2], s) > 1]
     shipped = {s: ops.tune_choice(a[0], a[2], s) for s in slots}
     tuned = ops.autotune(*a, dO=dO)
     tuned = {s: tuned[s] for s in slots}

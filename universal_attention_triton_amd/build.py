@@ -7,7 +7,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libua_hip.so")
-UNITS = ["ua_capi", "ua_inst_fwd", "ua_inst_bwd", "ua_inst_aff"]
+UNITS = ["ua_capi", "ua_inst_fwd", "ua_inst_bwd", "ua_inst_bwd4", "ua_inst_aff"]
 # packed-fp32 instructions are disabled for every device compile of this library
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-honor-nans", "-Wall", "-Wno-unused-function", "-Wno-unused-variable", "-Wno-unused-but-set-variable", "-Wno-unused-local-typedef", "-Wno-unused-value", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 

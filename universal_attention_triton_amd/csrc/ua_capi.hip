@@ -77,7 +77,7 @@ TuneKey tune_key(const ua_desc& d, int slot) {
 }
 bool known_slot(int slot) {
   return slot == UA_TUNE_FWD_RECOMPUTE || slot == UA_TUNE_CARRY || slot == UA_TUNE_FWD_TILES || slot == UA_TUNE_BWD_PARTS ||
-         slot == UA_TUNE_BWD_QUERIES;
+         slot == UA_TUNE_BWD_QUERIES || slot == UA_TUNE_BWD_KEYS;
 }
 int n_divisors(int r) { int n = 0; for (int p = 1; p <= r; ++p) n += r % p == 0; return n; }
 int nth_divisor(int r, int i) { for (int p = 1; p <= r; ++p) if (r % p == 0 && i-- == 0) return p; return 1; }
@@ -90,6 +90,7 @@ int n_variants(const ua_desc& d, int slot) {
     case UA_TUNE_FWD_TILES: return bf ? (d.d > 128 ? 1 : (d.r % 2 == 0 ? 2 : 3)) : 1;     // above 128: 16 queries per wave only
     case UA_TUNE_BWD_PARTS: return bf ? n_divisors(d.r) : 1;
     case UA_TUNE_BWD_QUERIES: return bf && d.d <= 128 ? 2 : 1;
+    case UA_TUNE_BWD_KEYS: return bf && padded_dim(d.d) == 128 && d.r == 1 ? 2 : 1;
   }
   return 1;
 }
@@ -418,6 +419,7 @@ int run_bwd_common(const ua_desc& d, const Layout& l, char* wf, char* wb, bool c
   a.skip_masked = (d.flags & UA_FLAG_SKIP_MASKED) ? 1 : 0;
   a.split_r = (!chunked && d.r > 1) ? 1 : 0;
   a.key_parts = l.key_parts;
+  a.keys_variant = l.tiles ? tuned_variant(d, UA_TUNE_BWD_KEYS) : 0;
   // bf16 tile exchange with one query group: the two kernels write the caller's gradients themselves.  The chunked
   // operator qualifies when the caller asserts that nothing flows to (query, later chunk) pairs, so that the query side is
   // known here to run from the tiles.
@@ -900,6 +902,14 @@ int ua_autotune(const ua_desc* desc, int op, void* ws, size_t ws_bytes, ua_strea
     a.dsrc_raw = (float*)(wb + ll.dsrc_raw); a.masked_nz = (const int*)(wb + ll.masked_nz);
     a.dS_st = wb + ll.dS_st; a.dG_st = wb + ll.dG_st; a.Bt = wf + ll.Bt;
     a.R = d.r; a.L = d.L; a.Lp = ll.Lp; a.c = 128; a.nch = 1; a.key_parts = ll.key_parts;
+    // one query group: the production path has both kernels write the caller's gradients from their epilogues and runs no
+    // finish pass, so the slots are timed that way, with throw-away outputs in the scratch (dv over the dV partial sums,
+    // dk over the column-side partial sums, the gate gradients over the dsrc partial sums; "gates" read from the log-gates)
+    if (d.r == 1 && !gates_f32(d)) {
+      a.direct = 1; a.d_out = d.d;
+      a.dv_out = wb + ll.dVrow; a.dk_out = wb + ll.dKdacc; a.dsrc_out = wb + ll.dsrc_raw; a.ddest_out = wb + ll.dsrc_raw;
+      a.src_in = wf + ll.lsrc; a.dest_in = wf + ll.ldest;
+    }
     return a;
   };
   if (d.r > 1 && !(d.flags & UA_FLAG_SHARE_GROUPS)) {
@@ -914,6 +924,16 @@ int ua_autotune(const ua_desc* desc, int op, void* ws, size_t ws_bytes, ua_strea
     if (ws_bytes < l.total) return fail(UA_EWORKSPACE, "the chosen number of parts needs %zu bytes of workspace", l.total);
     // leave tiles that match the chosen layout for the query side
     { const ua::BwdArgsV a = bwd_args(l); UA_HIP(ua::launch_bwd_keys(d.dtype, l.D, a, l.Zk, 0, s)); }
+  }
+  if (d.r == 1) {
+    // both variants leave the same tiles; the slot is timed on the production code path (results straight to the caller's
+    // tensors are replaced by the partial-sum buffers of the scratch)
+    if (int e = tune_slot(d, UA_TUNE_BWD_KEYS, s, [&](int v) {
+          ua::BwdArgsV a = bwd_args(l);
+          a.keys_variant = v;
+          UA_HIP(ua::launch_bwd_keys(d.dtype, l.D, a, l.Zk, 0, s));
+          return (int)UA_OK;
+        })) return e;
   }
   {
     const ua::BwdArgsV a = bwd_args(l);

@@ -19,6 +19,7 @@ struct BwdArgsV {
   void *dk_out, *dv_out, *dsrc_out, *ddest_out;
   const void *src_in, *dest_in;
   int dO_rows;
+  int keys_variant;     // UA_TUNE_BWD_KEYS
 };
 
 // Every launcher returns hipGetLastError() after enqueuing.  dtype: 0 fp32, 1 bf16.  D in {64,128}.
@@ -49,6 +50,8 @@ hipError_t launch_fwd_chunked2(int dtype, int D, const void* Qp, const void* Kp,
 // with a.chunked set: the chunked operator for a chunk that is a multiple of 64).
 // With a.key_parts > 1 (bf16 tiles, merged operator) the grid covers (kv head, part of its query groups) pairs.
 hipError_t launch_bwd_keys(int dtype, int D, const BwdArgsV& a, int Zk, int cols, hipStream_t s);
+// bf16 merged operator over bias tiles, one query group per kv head, D in {64,128}: 32 keys per wave (ua_keys4.hpp)
+hipError_t launch_bwd_keys4(int D, const BwdArgsV& a, int Zk, hipStream_t s);
 hipError_t launch_bwd_queries(int dtype, int D, const BwdArgsV& a, void* dq, int d, int Zk, hipStream_t s);
 // bf16 only, a.dS_st / a.dG_st filled by launch_bwd_keys (cols == 0): the query side as pure matrix work over those tiles
 // variant: UA_TUNE_BWD_QUERIES
