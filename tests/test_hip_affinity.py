@@ -50,9 +50,12 @@ def test_affinity_scores_forward_and_backward(shape, dtype):
     # from the float64 one (2e-4 at L = 517, 2e-3 at L = 1032)
     leaves32 = [x.float().requires_grad_() for x in (k, src, dest)]
     g32 = torch.autograd.grad(orc.affinity_scores(*leaves32), leaves32, daff.float() * visible)
-    tol_dk = max(TOL[dtype], 4e-4, 3 * rel_err(g32[0], gw[0]))
+    own = rel_err(g32[0], gw[0])
+    tol_dk = max(TOL[dtype], 3 * own)
+    print("  dk bar %.2e (stated %.0e, float32 evaluation of the oracle misses float64 by %.2e)" % (tol_dk, TOL[dtype], own), flush=True)
     for name, got, ref in zip(("dk", "dsrc", "ddest"), grads, gw):
         tol = TOL[dtype] if name != "dk" else tol_dk
+        print("  %-6s %.2e (bar %.2e)" % (name, rel_err(got, ref), tol), flush=True)
         assert rel_err(got, ref) <= tol, (name, rel_err(got, ref), tol)
 
 

@@ -8,7 +8,7 @@ import torch
 from universal_attention_triton_amd import _lib
 
 from oracle import ua_oracle as orc
-from tests.util import NAMES, TOL, dense_reference, load_golden, rel_err
+from tests.util import NAMES, TOL, dense_reference, key_gradient_bar, load_golden, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -32,9 +32,12 @@ def test_reference_call_sequence_through_the_drop_in_modules(name):
     grads = torch.autograd.grad(O, leaves, t["dO"].to(dtype).cuda())
     tol = TOL[dtype]
     assert rel_err(out, t["out"]) <= tol and rel_err(denom, t["denom"]) <= tol and rel_err(O, t["O"]) <= tol
+    inp = {k: t[k].to(dtype) for k in NAMES + ("dO",)}
+    bar_dkc = key_gradient_bar(inp, dtype, dense_reference(inp)[2][0])
     for g, k in zip(grads, ("c_dkc", "c_dvc", "c_dxq", "c_dsrc", "c_ddest")):
         assert g is not None and g.shape == leaves[("c_dkc", "c_dvc", "c_dxq", "c_dsrc", "c_ddest").index(k)].shape
-        bar = tol if k != "c_dkc" else max(tol, 4e-4)      # d/dk of relu(k.k)^(2/3): see test_hip_backward
+        bar = tol if k != "c_dkc" else bar_dkc
+        print("  %-8s %.2e (bar %.2e)" % (k, rel_err(g, t[k]), bar), flush=True)
         assert rel_err(g, t[k]) <= bar, (k, rel_err(g, t[k]))
 
 
@@ -90,8 +93,9 @@ def test_fused_operator_autograd_and_strided_inputs(dtype):
     O = universal_attention(*leaves)
     grads = torch.autograd.grad(O, leaves, dev["dO"].view(O.shape))
     assert rel_err(O, O_ref) <= TOL[dtype]
+    bar_dkc = key_gradient_bar(inp, dtype, g_ref[0])
     for k, g, gr in zip(NAMES, grads, g_ref):
-        assert rel_err(g, gr) <= (TOL[dtype] if k != "kc" else max(TOL[dtype], 4e-4)), (k, rel_err(g, gr))
+        assert rel_err(g, gr) <= (TOL[dtype] if k != "kc" else bar_dkc), (k, rel_err(g, gr))
     # 2-D query layout gives the same result in xq's shape
     xq2 = dev["xq"].view(b, h, r, L // 64, 64, d)
     O2, lse = universal_attention(dev["kc"], dev["vc"], xq2, dev["static_src"], dev["static_dest"].view(b, h, L // 64, 64), return_lse=True)
@@ -244,7 +248,7 @@ def test_edge_cases_of_the_inputs(case, dtype):
             # summation order of fp32 dot products, and dS is rounded to the operand dtype before its products
             assert float(g.float().norm()) <= 0.1 * tol * float(inp["dO"].float().norm()), (k, float(g.float().norm()))
             continue
-        bar = tol if k != "kc" else max(tol, 4e-4)
+        bar = tol if k != "kc" else key_gradient_bar(inp, dtype, gr)
         assert rel_err(g.reshape(gr.shape), gr) <= bar, (case, k, rel_err(g.reshape(gr.shape), gr))
 
 
@@ -296,8 +300,9 @@ def test_pruning_of_negligible_pairs_changes_nothing(case, dtype):
             assert rel_err(y2, x) <= tight, (name, rel_err(y2, x))
     O_ref, lse_ref, g_ref = dense_reference(inp)
     assert rel_err(res[True][0], O_ref) <= TOL[dtype]
+    bar_dkc = key_gradient_bar(inp, dtype, g_ref[0])
     for k, g, gr in zip(NAMES, res[True][2:], g_ref):
-        assert rel_err(g.reshape(gr.shape), gr) <= (TOL[dtype] if k != "kc" else max(TOL[dtype], 4e-4)), (k, rel_err(g.reshape(gr.shape), gr))
+        assert rel_err(g.reshape(gr.shape), gr) <= (TOL[dtype] if k != "kc" else bar_dkc), (k, rel_err(g.reshape(gr.shape), gr))
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -328,7 +333,7 @@ def test_decoder_front_end_takes_sequence_major_projections_without_copies(dtype
     assert rel_err(out.transpose(1, 2).reshape(O_ref.shape), O_ref) <= TOL[dtype]
     assert rel_err(gq.transpose(1, 2).reshape(g_ref[2].shape), g_ref[2]) <= TOL[dtype]
     assert rel_err(gv.transpose(1, 2).reshape(g_ref[1].shape), g_ref[1]) <= TOL[dtype]
-    assert rel_err(gk.transpose(1, 2).reshape(g_ref[0].shape), g_ref[0]) <= max(TOL[dtype], 4e-4)
+    assert rel_err(gk.transpose(1, 2).reshape(g_ref[0].shape), g_ref[0]) <= key_gradient_bar(inp, dtype, g_ref[0])
     gs = gs.view(b, s, 2, n_kv).permute(2, 0, 3, 1)
     assert rel_err(gs[0].reshape(g_ref[3].shape), g_ref[3]) <= TOL[dtype]
     assert rel_err(gs[1].reshape(g_ref[4].shape), g_ref[4]) <= TOL[dtype]

@@ -3,7 +3,7 @@ import pytest
 import torch
 
 from oracle import ua_oracle as orc
-from tests.util import NAMES, TOL, dense_reference, load_golden, rel_err
+from tests.util import NAMES, TOL, dense_reference, key_gradient_bar, load_golden, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -24,19 +24,6 @@ def _report(tag, got, want, tol, tol_dkc=None):
     assert not bad, bad
 
 
-def _reference_dkc_error(inp, dtype, exact):
-    """d/dk of relu(k_s.k_u)^(2/3) is (2/3)(k_s.k_u)^(-1/3): singular at 0+, so pairs with a tiny positive
-    product amplify the rounding of the product itself.  The reference algorithm run in the SAME dtype
-    therefore misses the float64 gradient by more than the tensor-wide tolerance on some inputs (2.7e-4
-    in fp32 on the 256x64 case).  Returns that error: the bar for dkc is the larger of the stated
-    tolerance and twice this self-error of the reference algorithm."""
-    args = [inp[k] for k in NAMES]
-    out, denom = orc.chunked_forward(*args)
-    d_out, d_denom = orc.merge_backward(out.float(), denom.float(), inp["dO"].float())
-    g = orc.chunked_backward(*args, d_out.to(dtype), d_denom)
-    return rel_err(g[0], exact)
-
-
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("shape", SHAPES)
 def test_fused_backward_matches_dense_autograd(shape, dtype):
@@ -50,7 +37,7 @@ def test_fused_backward_matches_dense_autograd(shape, dtype):
     grads = torch.autograd.grad(O, leaves, inp["dO"].cuda())
     torch.cuda.synchronize()
     assert rel_err(O, O_ref) <= TOL[dtype]
-    _report("fused", grads, g_ref, TOL[dtype], max(TOL[dtype], 2 * _reference_dkc_error(inp, dtype, g_ref[0])))
+    _report("fused", grads, g_ref, TOL[dtype], key_gradient_bar(inp, dtype, g_ref[0]))
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

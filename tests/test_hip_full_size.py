@@ -95,10 +95,23 @@ def test_config2_headline_bf16_forward_backward_h32_L8192_d128():
     _, _, grads2 = _run_fused(dev, scale=2.0)
     for g, g2 in zip(grads, grads2):
         assert torch.equal(g2.float(), 2.0 * g.float())
-    print("case cfg2 oracle head", flush=True)
-    z = (0, 17)
-    ref_O, ref_grads = _oracle_head(inp, z, True)
-    _check_head(O, grads, ref_O, ref_grads, z, TOL[BF16])
+    from universal_attention_triton_amd import ops
+    print("case cfg2 key-side kernel with 32 keys per wave", flush=True)
+    assert ops.tune_variants(dev["kc"], dev["xq"], "bwd_keys") == 2
+    ops.tune_set(dev["kc"], dev["xq"], 1, "bwd_keys")
+    try:
+        _, _, grads_v1 = _run_fused(dev)
+    finally:
+        ops.tune_set(dev["kc"], dev["xq"], -1, "bwd_keys")
+    for g, g1 in zip(grads, grads_v1):
+        assert torch.equal(g1[:, 30:32], g1[:, 0:2])
+        assert rel_err(g1, g) <= 6e-3, rel_err(g1, g)          # the same bf16 tiles, summed in another order
+    _check_dv_identity(dev, grads_v1, TOL[BF16])
+    for z in ((0, 17), (0, 4)):
+        print("case cfg2 oracle head", z, flush=True)
+        ref_O, ref_grads = _oracle_head(inp, z, True)
+        _check_head(O, grads, ref_O, ref_grads, z, TOL[BF16])
+        _check_head(O, grads_v1, ref_O, ref_grads, z, TOL[BF16])
 
 
 def test_config3_grouped_queries_h8_r4_L4096_d128():
@@ -115,10 +128,10 @@ def test_config3_grouped_queries_h8_r4_L4096_d128():
     _, _, grads2 = _run_fused(dev, scale=2.0)
     for g, g2 in zip(grads, grads2):
         assert torch.equal(g2.float(), 2.0 * g.float())
-    print("case cfg3 oracle head", flush=True)
-    z = (0, 5)
-    ref_O, ref_grads = _oracle_head(inp, z, True)
-    _check_head(O, grads, ref_O, ref_grads, z, TOL[BF16])
+    for z in ((0, 5), (0, 0)):
+        print("case cfg3 oracle head", z, flush=True)
+        ref_O, ref_grads = _oracle_head(inp, z, True)
+        _check_head(O, grads, ref_O, ref_grads, z, TOL[BF16])
 
 
 def test_config4_long_context_h8_L32768_d128_gates_near_one():
@@ -150,12 +163,12 @@ def test_config4_long_context_h8_L32768_d128_gates_near_one():
     torch.cuda.synchronize()
     assert torch.equal(Os, O[:, :, :, :T]) and torch.equal(lses, lse[:, :, :, :T])
     # the reference operator on one head of the prefix, and of the whole sequence (forward)
-    print("case cfg4 oracle prefix head", flush=True)
-    z = (0, 3)
     cpu_short = {k: v.cpu() for k, v in short.items()}
-    ref_O, ref_grads = _oracle_head(cpu_short, z, True)
     _, _, gshort = _run_fused(short)
-    _check_head(Os, gshort, ref_O, ref_grads, z, TOL[BF16])
+    for z in ((0, 7), (0, 3)):
+        print("case cfg4 oracle prefix head", z, flush=True)
+        ref_O, ref_grads = _oracle_head(cpu_short, z, True)
+        _check_head(Os, gshort, ref_O, ref_grads, z, TOL[BF16])
     # ... and of the whole sequence, forward and all five gradients (the merged result and its gradients do not
     # depend on the chunk size, so the oracle runs with chunks of 1024 keys to keep its per-chunk tensors small)
     print("case cfg4 oracle full-length head, forward + backward", flush=True)

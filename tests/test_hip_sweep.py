@@ -94,6 +94,7 @@ def test_chunked_operator_random_shapes_and_upstreams():
     from universal_attention_triton_amd import universal_attention_autograd as ua
     rng = random.Random(20261)
     done = 0
+    relaxed = []
     while done < 16:
         b, h, r = rng.choice([1, 1, 2]), rng.choice([1, 2, 3]), rng.choice([1, 1, 2, 3])
         c = rng.choice([16, 32, 64, 64, 96, 128, 128, 192, 256])
@@ -135,20 +136,22 @@ def test_chunked_operator_random_shapes_and_upstreams():
             errs["d" + k] = rel_err(x.reshape(y.shape), y)
         bars = {k: tol for k in errs}
         bars["denom"] = max(tol, 2 ** -8 if dtype == torch.bfloat16 else tol)      # denom is stored in the dtype
-        if dtype == torch.float32:
-            bars["dkc"] = 5e-4      # the float32 restatement itself moves this far under a permutation of the head dim
-            if errs["dkc"] > bars["dkc"]:
-                # a key-key product very close to 0+ (d/dG relu(G)^(2/3) is singular there): judge both float32 results
-                # by the float64 evaluation, the kernel being allowed three times the restatement's own error (the worst over
-                # the given, the reversed and fourteen random summation orders of the head dimension)
-                exact = orc.chunked_backward(*[inp[k].double() for k in NAMES], g_out.double(), g_denom.double())[0]
-                errs["dkc"] = rel_err(grads[0].reshape(exact.shape), exact)
-                bars["dkc"] = max(bars["dkc"], 2 * rel_err(want[0], exact))
-                gen = torch.Generator().manual_seed(1)
-                for trial in range(15):
-                    perm = torch.arange(d).flip(0) if trial == 0 else torch.randperm(d, generator=gen)
-                    a2 = [x[..., perm] for x in args32[:3]] + args32[3:]
-                    g2 = orc.chunked_backward(*a2, g_out.float()[..., perm, :], g_denom.float())[0]
-                    bars["dkc"] = max(bars["dkc"], 3 * rel_err(g2[..., torch.argsort(perm)], exact))
+        if dtype == torch.float32 and errs["dkc"] > bars["dkc"]:
+            # a key-key product very close to 0+ (d/dG relu(G)^(2/3) is singular there): judge both float32 results
+            # by the float64 evaluation, the kernel being allowed twice the restatement's own error and three times
+            # what the restatement moves under the reversed and fourteen random summation orders of the head dimension
+            exact = orc.chunked_backward(*[inp[k].double() for k in NAMES], g_out.double(), g_denom.double())[0]
+            errs["dkc"] = rel_err(grads[0].reshape(exact.shape), exact)
+            bars["dkc"] = max(tol, 2 * rel_err(want[0], exact))
+            gen = torch.Generator().manual_seed(1)
+            for trial in range(15):
+                perm = torch.arange(d).flip(0) if trial == 0 else torch.randperm(d, generator=gen)
+                a2 = [x[..., perm] for x in args32[:3]] + args32[3:]
+                g2 = orc.chunked_backward(*a2, g_out.float()[..., perm, :], g_denom.float())[0]
+                bars["dkc"] = max(bars["dkc"], 3 * rel_err(g2[..., torch.argsort(perm)], exact))
+            relaxed.append((done, "dkc %.2e under a computed bar of %.2e" % (errs["dkc"], bars["dkc"])))
+        print("  " + "  ".join("%s %.1e/%.0e" % (k, v, bars[k]) for k, v in errs.items()), flush=True)
         bad = {k: (v, bars[k]) for k, v in errs.items() if not v <= bars[k]}
         assert not bad, (case, bad)
+    print("cases with the key gradient judged by the restatement's own float32 error: %d of 16" % len(relaxed), relaxed, flush=True)
+    assert len(relaxed) <= 4, relaxed
