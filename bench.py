@@ -358,9 +358,7 @@ def main():
         # the same sequence with only the float32 normalisers kept for the backward instead of the whole forward state
         # (1/(d+1) of the size of `out`; the backward then repacks the inputs and repeats the decay pre-pass)
         from universal_attention_triton_amd import ops, universal_attention_autograd as own_api
-        default_keep = own_api._ChunkedBase.keep_state
-        own_api._ChunkedBase.keep_state = "normalisers"
-        try:
+        with own_api.chunked_options(keep_state="normalisers"):
             n_full = max(3, args.steps // 4)
             for _ in range(2):
                 step()
@@ -371,8 +369,6 @@ def main():
             torch.cuda.synchronize()
             out["config"]["keep_state_normalisers"] = {"ms_per_step": round((time.perf_counter() - t0) * 1e3 / n_full, 4),
                                                        "note": "optional: only the normalisers retained for the backward; not `value`"}
-        finally:
-            own_api._ChunkedBase.keep_state = default_keep
         out["config"]["bytes_retained_fwd_to_bwd"] = {
             "forward_state": int(ops.retained_bytes(*[x.detach() for x in leaves], chunked=True)),
             "out_and_denom": int(cfg["b"] * cfg["h"] * cfg["r"] * cfg["L"] * (cfg["d"] + 1) * (cfg["L"] // cfg["c"])

@@ -223,18 +223,15 @@ def test_memory_kept_between_forward_and_backward_by_the_chunked_functions():
     assert state < out_bytes // 3
     slack = 8 << 20
     for keep, extra in ((True, state), ("normalisers", b * h * r * n * L * 4), (False, 0)):
-        ua._ChunkedBase.keep_state = keep
-        try:
+        with ua.chunked_options(keep_state=keep):
             out, denom = ua.UniversalAttention.apply(*leaves)
-            torch.cuda.synchronize()
-            held = torch.cuda.memory_allocated() - base
-            assert out_bytes + extra - slack <= held <= out_bytes + extra + slack, (keep, held, out_bytes, extra)
-            grads = torch.autograd.grad([out, denom], leaves, [torch.ones_like(out), torch.zeros_like(denom)])
-            del out, denom, grads
-            torch.cuda.synchronize()
-            assert torch.cuda.memory_allocated() - base <= slack
-        finally:
-            ua._ChunkedBase.keep_state = True
+        torch.cuda.synchronize()
+        held = torch.cuda.memory_allocated() - base
+        assert out_bytes + extra - slack <= held <= out_bytes + extra + slack, (keep, held, out_bytes, extra)
+        grads = torch.autograd.grad([out, denom], leaves, [torch.ones_like(out), torch.zeros_like(denom)])
+        del out, denom, grads
+        torch.cuda.synchronize()
+        assert torch.cuda.memory_allocated() - base <= slack
 
 
 @pytest.mark.parametrize("shape", [(1, 2, 1, 320, 160), (1, 1, 2, 200, 256), (2, 1, 4, 128, 136)])
@@ -309,19 +306,16 @@ def test_out_allocated_contiguous_like_the_reference(dtype):
     g_denom = torch.randn(b, h, r, L, n, generator=g).to(dtype)
     results = []
     for contiguous in (False, True):
-        ua._ChunkedBase.contiguous_out = contiguous
-        try:
-            leaves = [inp[k].cuda().requires_grad_() for k in NAMES]
+        leaves = [inp[k].cuda().requires_grad_() for k in NAMES]
+        with ua.chunked_options(contiguous_out=contiguous):
             out, denom = ua.UniversalAttention.apply(*leaves)
-            assert out.shape == (b, h, r, L, d, n)
-            assert out.is_contiguous() == contiguous
-            if contiguous:
-                out.view(b * h * r, L, d * n)            # what fails on the permuted view
-            grads = torch.autograd.grad([out, denom], leaves, [g_out.cuda(), g_denom.cuda()])
-            torch.cuda.synchronize()
-            results.append((out.detach().clone(), denom.detach().clone(), grads))
-        finally:
-            ua._ChunkedBase.contiguous_out = False
+        assert out.shape == (b, h, r, L, d, n)
+        assert out.is_contiguous() == contiguous
+        if contiguous:
+            out.view(b * h * r, L, d * n)            # what fails on the permuted view
+        grads = torch.autograd.grad([out, denom], leaves, [g_out.cuda(), g_denom.cuda()])
+        torch.cuda.synchronize()
+        results.append((out.detach().clone(), denom.detach().clone(), grads))
     (o0, d0, g0), (o1, d1, g1) = results
     assert torch.equal(o0, o1) and torch.equal(d0, d1)
     for name, x, y in zip(NAMES, g0, g1):
@@ -347,18 +341,15 @@ def test_what_the_chunked_function_keeps_for_its_backward_does_not_change_the_gr
     g = torch.Generator().manual_seed(5)
     g_out = torch.randn(b, h, r, L, d, n, generator=g).to(dtype).cuda()
     g_denom = torch.randn(b, h, r, L, n, generator=g).to(dtype).cuda()
-    assert ua._ChunkedBase.keep_state is True
     results = []
     for keep in (True, "normalisers", False):
-        ua._ChunkedBase.keep_state = keep
-        try:
-            leaves = [inp[k].cuda().requires_grad_() for k in NAMES]
+        leaves = [inp[k].cuda().requires_grad_() for k in NAMES]
+        with ua.chunked_options(keep_state=keep):
             out, denom = ua.UniversalAttention.apply(*leaves)
-            grads = torch.autograd.grad([out, denom], leaves, [g_out, g_denom])
-            torch.cuda.synchronize()
-            results.append((out.detach().clone(), grads))
-        finally:
-            ua._ChunkedBase.keep_state = True
+        # the backward runs outside the block: it uses what its forward saw
+        grads = torch.autograd.grad([out, denom], leaves, [g_out, g_denom])
+        torch.cuda.synchronize()
+        results.append((out.detach().clone(), grads))
     for o, grads in results[1:]:
         assert torch.equal(o, results[0][0])
         for name, x, y in zip(NAMES, grads, results[0][1]):

@@ -1,5 +1,6 @@
 """Host-side operators over the C ABI: tensor plumbing only (device memory, strides, streams)."""
 import ctypes
+import weakref
 
 import torch
 
@@ -135,19 +136,20 @@ def _gate_grads(b, h, L, src, static_src, static_dest):
     return dsrc, torch.empty_like(dsrc)
 
 
-# What merge_backward leaves for a chunked_backward that receives exactly the gradients it produced: weak references
-# to the two gradient tensors (the entry dies with them) and the per-(row, chunk) term delta.
-_merge_handoff = {}
+# merge_backward attaches to the gradient tensor it returns for `mat` what a chunked_backward that receives exactly that
+# tensor can reuse: the per-(row, chunk) term delta = sum_d out g_out - g_denom, with the identities of the tensors it
+# belongs to.  The note lives on the tensor object and dies with it; a gradient that was accumulated with another one,
+# replaced by a hook or modified in place is another object or version and simply has no (valid) note.
+_NOTE = "_ua_merge_note"
 
 
 def _delta_from_merge(out, g_out, g_denom, L, n):
-    item = _merge_handoff.pop("last", None)
-    if item is None:
+    note = getattr(g_out, _NOTE, None)
+    if note is None:
         return None
-    w_mat, w_vec, out_id, v_mat, v_vec, delta = item
-    # the gradients: the very objects (an entry dies with them, so a new tensor at an old address cannot match), unmodified;
+    w_vec, out_id, v_mat, v_vec, delta = note
     # `out`: alive since the forward, so the tensor merged at that address with this shape and these strides was this one
-    if w_mat() is g_out and w_vec() is g_denom and out_id == (out.data_ptr(), tuple(out.shape), tuple(out.stride()), out._version) \
+    if w_vec() is g_denom and out_id == (out.data_ptr(), tuple(out.shape), tuple(out.stride()), out._version) \
             and g_out._version == v_mat and g_denom._version == v_vec and delta.shape[1] == n and delta.shape[2] >= L:
         return delta
     return None
@@ -159,6 +161,8 @@ def chunked_backward(kc, vc, xq, static_src, static_dest, out, g_out, g_denom, s
     backward takes delta = sum_d out g_out - g_denom from that call instead of reading both 4-GB-class tensors again,
     and knows that the gradients vanish where a query precedes a chunk."""
     src_dtype, dest_dtype = static_src.dtype, static_dest.dtype
+    if state is not None and state.numel() == 0:
+        state = None
     delta = None
     if kc.shape[3] % 64 == 0:
         delta = _delta_from_merge(out, g_out, g_denom, kc.shape[2] * kc.shape[3], kc.shape[2])
@@ -234,6 +238,8 @@ def fused_backward(kc, vc, xq, static_src, static_dest, O, lse, dO, state=None, 
     r = xq.shape[2]
     L = n * c
     desc = _desc(kc, xq, False, _fused_flags(prune, recompute, share_groups) | gflag)
+    if state is not None and state.numel() == 0:
+        state = None
     if state is not None and state.numel() < lib.ua_workspace_bytes(ctypes.byref(desc), _lib.UA_OP_FUSED_FWD):
         state = None
     ws = _ws if _ws is not None else _workspace(desc, _lib.UA_OP_FUSED_BWD_SCRATCH if state is not None else _lib.UA_OP_FUSED_BWD, xq.device)
@@ -307,9 +313,11 @@ def merge_backward(mat, vec, g):
                                 d_vec.data_ptr(), delta.data_ptr(), _stream()), "ua_merge_bwd")
     d_mat = d4.unflatten(0, tuple(mat.shape[:-3])) if mat.dim() != 4 else d4
     d_vec = d_vec.to(vec.dtype)
-    import weakref
-    _merge_handoff["last"] = (weakref.ref(d_mat), weakref.ref(d_vec), (mat.data_ptr(), tuple(mat.shape), tuple(mat.stride()), mat._version),
-                              d_mat._version, d_vec._version, delta)
+    try:
+        setattr(d_mat, _NOTE, (weakref.ref(d_vec), (mat.data_ptr(), tuple(mat.shape), tuple(mat.stride()), mat._version),
+                               d_mat._version, d_vec._version, delta))
+    except (AttributeError, TypeError):          # a tensor subclass without instance attributes: no note, no shortcut
+        pass
     return d_mat, d_vec
 
 

@@ -14,10 +14,11 @@ import torch
 from torch.autograd import Function
 
 from . import ops
-from .universal_attention_autograd import _ChunkedBase, _put_state, _take_state
+from . import universal_attention_autograd as _chunked
+from .universal_attention_autograd import _ChunkedBase
 
 
-class UniversalAttention(_ChunkedBase):
+class _CheckedChunked2D(_ChunkedBase):
     @staticmethod
     def forward(kc, vc, xq, static_src, static_dest):
         b, h, r, _n, _c, d = xq.shape
@@ -29,13 +30,22 @@ class UniversalAttention(_ChunkedBase):
         return _ChunkedBase.forward(kc, vc, xq, static_src, static_dest)
 
     @staticmethod
-    def backward(ctx, dout, ddenom):
+    def backward(ctx, dout, ddenom, _dstate=None):
         kc, vc, xq = ctx.saved_tensors[:3]
         b, h, r, _n, _c, d = xq.shape
         _, _, n_, c_, _ = kc.shape
         assert dout.shape == (b, h, r, n_ * c_, d, n_)
         assert ddenom.shape == (b, h, r, n_ * c_, n_)
         return _ChunkedBase.backward(ctx, dout, ddenom)
+
+
+class UniversalAttention(_chunked.UniversalAttention):
+    """.apply(kc, vc, xq, static_src, static_dest) -> (out, denom), 2-D query layout, with the reference entry point's
+    shape checks (Universal_Attention/universal_attention.py:8-13, :35-38)."""
+    function = _CheckedChunked2D
+
+
+_fused_bwd = _chunked.kernel_call(lambda *a: ops.fused_backward(*a[:8], state=a[8], prune=a[9], recompute=a[10]), "FusedBackward")
 
 
 class _FusedUniversalAttention(Function):
@@ -45,28 +55,27 @@ class _FusedUniversalAttention(Function):
         # reference's footprint (its five inputs, plus O and lse here)
         keep = keep_state and not recompute and any(t.requires_grad for t in (kc, vc, xq, static_src, static_dest))
         O, lse, state = ops.fused_forward(kc, vc, xq, static_src, static_dest, keep_state=keep, prune=prune, recompute=recompute)
-        O = O.view(*xq.shape)
-        _put_state(O, state)
-        return O, lse
+        if state is None:
+            state = torch.empty(0, dtype=torch.uint8, device=O.device)
+        return O.view(*xq.shape), lse, state
 
     @staticmethod
     def setup_context(ctx, inputs, output):
         kc, vc, xq, static_src, static_dest, prune, recompute, _ = inputs
-        O, lse = output
+        O, lse, state = output
         ctx.prune, ctx.recompute = prune, recompute
-        ctx.save_for_backward(kc, vc, xq, static_src, static_dest, O, lse)
-        ctx.state = _take_state(O)
-        ctx.mark_non_differentiable(lse)
+        # the forward state travels as a third, non-differentiable output that universal_attention() drops
+        ctx.save_for_backward(kc, vc, xq, static_src, static_dest, O, lse, state)
+        ctx.mark_non_differentiable(lse, state)
 
     @staticmethod
-    def backward(ctx, dO, _dlse):
-        kc, vc, xq, static_src, static_dest, O, lse = ctx.saved_tensors
+    def backward(ctx, dO, _dlse, _dstate=None):
+        kc, vc, xq, static_src, static_dest, O, lse, state = ctx.saved_tensors
         b, h, n, c, d = kc.shape
         r = xq.shape[2]
         dO = dO.reshape(b, h, r, n * c, d)
-        dk, dv, dq, dsrc, ddest = ops.fused_backward(kc, vc, xq, static_src, static_dest, O.reshape(b, h, r, n * c, d), lse, dO,
-                                                     state=ctx.state, prune=ctx.prune, recompute=ctx.recompute)
-        ctx.state = None
+        dk, dv, dq, dsrc, ddest = _fused_bwd.apply(kc, vc, xq, static_src, static_dest, O.reshape(b, h, r, n * c, d), lse, dO,
+                                                   state, ctx.prune, ctx.recompute)
         return dk, dv, dq.view(xq.shape), dsrc.view(static_src.shape), ddest.view(static_dest.shape), None, None, None
 
 
@@ -81,7 +90,7 @@ def universal_attention(kc, vc, xq, static_src, static_dest, return_lse=False, p
     (Universal_Attention/universal_attention.py:27-31); the backward then rebuilds the state first.
     recompute=True (bf16) implies that and also keeps the backward's workspace at O(L*L/16) bytes per head by
     recomputing the score and decay gradients in every kernel instead of exchanging tiles (UA_FLAG_RECOMPUTE)."""
-    O, lse = _FusedUniversalAttention.apply(kc, vc, xq, static_src, static_dest, prune, recompute, keep_state)
+    O, lse, _state = _FusedUniversalAttention.apply(kc, vc, xq, static_src, static_dest, prune, recompute, keep_state)
     return (O, lse) if return_lse else O
 
 
