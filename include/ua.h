@@ -71,7 +71,7 @@ enum {
  * fused operator without UA_FLAG_RECOMPUTE. */
 typedef struct ua_desc {
   int32_t b, h, r, L, d;
-  int32_t chunk; /* keys per chunk c (L % c == 0; c == 16 or c % 32 == 0, c <= 256); ignored by fused ops */
+  int32_t chunk; /* keys per chunk c (L % c == 0; a multiple of 64, or 16 or a multiple of 32 up to 256); ignored by fused ops */
   int32_t dtype; /* UA_F32 or UA_BF16, the dtype of every tensor except where noted */
   int32_t flags;
 } ua_desc;

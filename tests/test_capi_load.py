@@ -37,6 +37,17 @@ def test_descriptor_validation_and_workspace_sizes():
         assert lib.ua_workspace_bytes(ctypes.byref(bad), _lib.UA_OP_FWD) == 0
         assert frag in lib.ua_last_error()
     assert lib.ua_workspace_bytes(ctypes.byref(ok), 9) == 0
+    # chunks: any multiple of 64; 16 and the other multiples of 32 up to 256
+    for c, fine in ((512, True), (1024, True), (4096, True), (96, True), (16, True), (288, False), (48, False)):
+        d = _lib.UaDesc(1, 2, 1, 8192 if c != 288 else 288 * 4, 64, c, _lib.UA_BF16, 0)
+        d.L = c * 4 if c in (48, 96, 288) else 8192
+        assert (lib.ua_workspace_bytes(ctypes.byref(d), _lib.UA_OP_FWD) > 0) == fine, c
+    # more heads than grid rows: refused with the way out in the message (the Python operators split by themselves)
+    many = _lib.UaDesc(3, 16384, 2, 16, 16, 16, _lib.UA_F32, 0)
+    assert lib.ua_workspace_bytes(ctypes.byref(many), _lib.UA_OP_FUSED_FWD) == 0 and b"split the call along b or h" in lib.ua_last_error()
+    # head dims the reference's self-test reaches (512, Universal_Attention/triton/universal_attention_kernel.py:1189) are refused
+    wide = _lib.UaDesc(2, 4, 2, 2048, 512, 64, _lib.UA_BF16, 0)
+    assert lib.ua_workspace_bytes(ctypes.byref(wide), _lib.UA_OP_FWD) == 0 and b"256" in lib.ua_last_error()
 
 
 def test_workspace_follows_the_flags_and_the_group_layout():

@@ -3,7 +3,7 @@ import pytest
 import torch
 
 from oracle import ua_oracle as orc
-from tests.util import NAMES, TOL, dense_reference, key_gradient_bar, load_golden, rel_err
+from tests.util import NAMES, TOL, dense_reference, key_gradient_bar, load_golden, rel_err, summation_order_sensitivity as _summation_order_sensitivity
 
 pytestmark = pytest.mark.gpu
 
@@ -98,24 +98,6 @@ def test_merge_kernels_match_oracle():
         dm, dv = torch.autograd.grad(res, [m, v], g.cuda())
         assert rel_err(res, want) <= TOL[dtype]
         assert rel_err(dm, wd[0]) <= TOL[dtype] and rel_err(dv, wd[1]) <= TOL[dtype]
-
-
-def _summation_order_sensitivity(inp, g_out, g_denom, dkc):
-    """How far the float32 oracle's own dkc moves when the head dimension is summed in another order (features of k, v,
-    q and of the upstream gradient permuted, result permuted back; largest move over the reversed order and four
-    random ones): mathematically the same gradient, but the key-key products round differently and
-    (2/3)(k_s.k_u)^(-1/3) amplifies that for tiny positive products (one pair with k_s.k_u = 5.6e-6 carries half of
-    the whole tensor's error in the 512x64 case)."""
-    d = inp["kc"].shape[-1]
-    gen = torch.Generator().manual_seed(1)
-    worst = 0.0
-    for trial in range(5):
-        perm = torch.arange(d).flip(0) if trial == 0 else torch.randperm(d, generator=gen)
-        inv = torch.argsort(perm)
-        args = [inp[k].float()[..., perm] for k in ("kc", "vc", "xq")] + [inp[k].float() for k in ("static_src", "static_dest")]
-        g = orc.chunked_backward(*args, g_out.float()[..., perm, :], g_denom)
-        worst = max(worst, rel_err(g[0][..., inv], dkc))
-    return worst
 
 
 FAST_CHUNK_SHAPES = [  # chunk a multiple of 64: key-/query-stationary kernels; b, h, r, L, d, c

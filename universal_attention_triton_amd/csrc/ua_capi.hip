@@ -51,15 +51,27 @@ int check_desc(const ua_desc* d, bool chunked) {
   if (!d) return fail(UA_EINVAL, "null descriptor");
   if (d->dtype != UA_F32 && d->dtype != UA_BF16) return fail(UA_EINVAL, "dtype %d: only UA_F32 and UA_BF16 are supported", d->dtype);
   if (d->b < 1 || d->h < 1 || d->r < 1 || d->L < 1 || d->d < 1) return fail(UA_EINVAL, "b,h,r,L,d must be positive (got %d,%d,%d,%d,%d)", d->b, d->h, d->r, d->L, d->d);
-  if (d->d > 256) return fail(UA_EINVAL, "head dim %d > 256 is not supported", d->d);
+  // A (key, query) product contracts over the whole head dim inside one workgroup, whose LDS stages and accumulators
+  // are laid out for at most 256 features (the reference's second-generation kernel stops there too,
+  // universal_attention_kernel_opt.py:441-456; the self-test of its first one runs d = 512,
+  // Universal_Attention/triton/universal_attention_kernel.py:1189, which this library refuses)
+  if (d->d > 256) return fail(UA_EINVAL, "head dim %d > 256 is not supported (LDS stages and accumulators are laid out for at most 256 features)", d->d);
   if (d->d > 128 && (chunked || d->dtype != UA_BF16 || (d->flags & UA_FLAG_RECOMPUTE)))
-    return fail(UA_EINVAL, "head dim %d > 128: only the bf16 fused operator without UA_FLAG_RECOMPUTE", d->d);
-  if ((long)d->b * d->h * d->r > 65535) return fail(UA_EINVAL, "b*h*r = %ld exceeds the grid limit 65535", (long)d->b * d->h * d->r);
+    return fail(UA_EINVAL, "head dim %d > 128: only the bf16 fused operator without UA_FLAG_RECOMPUTE (float32 tiles of 256 features "
+                           "do not fit the LDS stages; the chunked operator has no 256-feature instantiation)", d->d);
+  // one grid row (y) per head; callers with more heads split the batch or the kv heads, which are independent
+  // (the Python operators do that by themselves)
+  if ((long)d->b * d->h * d->r > 65535)
+    return fail(UA_EINVAL, "b*h*r = %ld exceeds the grid limit 65535: split the call along b or h (heads are independent)", (long)d->b * d->h * d->r);
   if (chunked) {
     const int c = d->chunk;
     if (c < 1 || d->L % c != 0) return fail(UA_EINVAL, "chunk %d must divide L = %d", c, d->L);
-    if (!(c == 16 || c % 32 == 0) || c > 256) return fail(UA_EINVAL, "chunk %d unsupported: need 16 or a multiple of 32, at most 256", c);
-    if ((long)d->b * d->h * d->r * (d->L / c) > 65535) return fail(UA_EINVAL, "b*h*r*(L/chunk) exceeds the grid limit 65535");
+    // multiples of 64 of any size run on the query-/key-stationary kernels, which take the chunk as a run-time bound;
+    // 16 and the other multiples of 32 on the key-chunk-stationary ones, whose LDS holds a whole chunk
+    if (!(c % 64 == 0 || ((c == 16 || c % 32 == 0) && c <= 256)))
+      return fail(UA_EINVAL, "chunk %d unsupported: need a multiple of 64, or 16 or a multiple of 32 up to 256", c);
+    if ((long)d->b * d->h * d->r * (d->L / c) > 65535)
+      return fail(UA_EINVAL, "b*h*r*(L/chunk) exceeds the grid limit 65535: split the call along b or h (heads are independent)");
   }
   return UA_OK;
 }

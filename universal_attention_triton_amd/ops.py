@@ -1,5 +1,6 @@
 """Host-side operators over the C ABI: tensor plumbing only (device memory, strides, streams)."""
 import ctypes
+import functools
 import weakref
 
 import torch
@@ -100,6 +101,41 @@ def _prep(kc, vc, xq, static_src, static_dest):
     return kc, vc, xq, src, dest, gflag
 
 
+# One grid row per head: the entry points refuse more than 65535 of them (b * h * r, times the chunks per row for the
+# chunked operator).  Heads are independent, so the operators below split such a call along b, then h, run the pieces one
+# after the other and join the results; the pieces keep no forward state (the backward rebuilds it per piece).
+_GRID_ROWS = 65535
+
+
+def _split_over_heads(n_tensors, chunked):
+    def wrap(fn):
+        @functools.wraps(fn)
+        def run(*args, **kw):
+            kc, xq = args[0], args[2]
+            b, h = kc.shape[:2]
+            per_head = xq.shape[2] * (kc.shape[2] if chunked else 1)
+            if b * h * per_head <= _GRID_ROWS:
+                return fn(*args, **kw)
+            if per_head > _GRID_ROWS:
+                raise _lib.UaError("%d grid rows per kv head exceed the limit of %d" % (per_head, _GRID_ROWS))
+            step_h = min(h, _GRID_ROWS // per_head)
+            step_b = max(1, _GRID_ROWS // (h * per_head)) if step_h == h else 1
+            kw = {**kw, "state": None} if "state" in kw else dict(kw, **({"keep_state": False} if "keep_state" in kw else {}))
+            rows = []
+            for b0 in range(0, b, step_b):
+                row = []
+                for h0 in range(0, h, step_h):
+                    piece = [a[b0:b0 + step_b, h0:h0 + step_h] if i < n_tensors else a for i, a in enumerate(args)]
+                    row.append(fn(*piece, **kw))
+                rows.append([None if row[0][i] is None else (row[0][i] if len(row) == 1 else torch.cat([p[i] for p in row], 1))
+                             for i in range(len(row[0]))])
+            return tuple(None if rows[0][i] is None else (rows[0][i] if len(rows) == 1 else torch.cat([r_[i] for r_ in rows], 0))
+                         for i in range(len(rows[0])))
+        return run
+    return wrap
+
+
+@_split_over_heads(5, True)
 def chunked_forward(kc, vc, xq, static_src, static_dest, keep_state=False, recompute=False, contiguous_out=False):
     """-> out [b,h,r,l,d,n] (chunk-major storage, returned as a permuted view), denom [b,h,r,l,n], state
     contiguous_out: allocate `out` contiguous in the reference's index order instead (what `.view()` on it needs; the
@@ -155,6 +191,7 @@ def _delta_from_merge(out, g_out, g_denom, L, n):
     return None
 
 
+@_split_over_heads(8, True)
 def chunked_backward(kc, vc, xq, static_src, static_dest, out, g_out, g_denom, state=None, skip_masked=False, recompute=False):
     """state: what chunked_forward(keep_state=True) returned for the same inputs and flags, or None.
     When (g_out, g_denom) are the very tensors merge_backward produced from `out` (the reference's call sequence), the
@@ -203,6 +240,7 @@ def _fused_flags(prune, recompute, share_groups=False):
             | (_lib.UA_FLAG_SHARE_GROUPS if share_groups else 0))
 
 
+@_split_over_heads(5, False)
 def fused_forward(kc, vc, xq, static_src, static_dest, keep_state=False, prune=False, recompute=False, share_groups=False,
                   _ws=None):
     """-> O [b,h,r,l,d], lse [b,h,r,l] (float32), state
@@ -227,6 +265,7 @@ def fused_forward(kc, vc, xq, static_src, static_dest, keep_state=False, prune=F
     return O, lse, (ws if keep_state else None)
 
 
+@_split_over_heads(8, False)
 def fused_backward(kc, vc, xq, static_src, static_dest, O, lse, dO, state=None, prune=False, recompute=False, share_groups=False,
                    _ws=None):
     """state: what fused_forward(keep_state=True) returned for the same inputs and flags (skips the recompute and keeps

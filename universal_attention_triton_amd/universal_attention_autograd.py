@@ -73,7 +73,7 @@ def kernel_call(fn, name):
                                     "backward": staticmethod(backward)})
 
 
-_chunked_bwd = kernel_call(lambda *a: ops.chunked_backward(*a[:9], skip_masked=a[9], recompute=a[10]), "ChunkedBackward")
+_chunked_bwd = kernel_call(lambda *a: ops.chunked_backward(*a[:8], state=a[8], skip_masked=a[9], recompute=a[10]), "ChunkedBackward")
 _merge_bwd = kernel_call(lambda mat, vec, g: ops.merge_backward(mat, vec, g), "MergeBackward")
 
 
