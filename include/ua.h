@@ -204,9 +204,15 @@ enum {
                                 Changes ua_workspace_bytes: set it before sizing the workspace. */
   UA_TUNE_BWD_QUERIES = 19,  /* query side of the bf16 backward over gradient tiles: 0 = steps of 32 keys, two workgroups
                                 per CU; 1 = steps of 64 keys, one workgroup per CU */
-  UA_TUNE_BWD_KEYS = 20      /* key side of the bf16 backward over bias tiles, r = 1, head dim 65..128: 0 = 16 keys per
+  UA_TUNE_BWD_KEYS = 20,     /* key side of the bf16 backward over bias tiles, r = 1, head dim 65..128: 0 = 16 keys per
                                 wave on 16x16 tiles, two waves per SIMD; 1 = 32 keys per wave on 32x32 tiles, one wave per
                                 SIMD, the step laid out by hand */
+  UA_TUNE_CHUNKED_PAIR = 21, /* chunked operator, chunk a multiple of 64 (ua_fwd, ua_bwd): work items (query blocks of the
+                                forward, key groups of the backward's key side) per workgroup: 0 = two of complementary
+                                length once the launch gives every CU several single ones, 1 = one, 2 = two */
+  UA_TUNE_AFF_PAIR = 22      /* stand-alone bias (ua_affinity_fwd, ua_affinity_bwd): key groups per workgroup, as above.
+                                ua_autotune does not time these two slots: time the op itself under each variant
+                                (ua_tune_set), as the Python layer's autotune_chunked / autotune_affinity do */
 };
 /* ua_autotune(desc, op, ...) with op = UA_OP_FUSED_FWD or UA_OP_FUSED_BWD times every variant of every kernel slot on
  * that op's path for desc (hipEvents on `stream`, synchronises) and records the fastest of each.  `ws` must hold what

@@ -106,7 +106,8 @@ def test_tune_table_roundtrip_and_choice_order():
     lib = _lib.load()
     d = _lib.UaDesc(1, 2, 1, 1024, 128, 0, _lib.UA_BF16, 0)
     for slot, n_min in ((_lib.UA_TUNE_FWD_RECOMPUTE, 5), (_lib.UA_TUNE_CARRY, 2), (_lib.UA_TUNE_FWD_TILES, 3),
-                        (_lib.UA_TUNE_BWD_PARTS, 1), (_lib.UA_TUNE_BWD_QUERIES, 2), (_lib.UA_TUNE_BWD_KEYS, 2)):
+                        (_lib.UA_TUNE_BWD_PARTS, 1), (_lib.UA_TUNE_BWD_QUERIES, 2), (_lib.UA_TUNE_BWD_KEYS, 2),
+                        (_lib.UA_TUNE_CHUNKED_PAIR, 3), (_lib.UA_TUNE_AFF_PAIR, 3)):
         n = lib.ua_tune_variants(ctypes.byref(d), slot)
         assert n >= n_min, (slot, n)
         base = lib.ua_tune_choice(ctypes.byref(d), slot)

@@ -101,15 +101,114 @@ def test_shipped_table_is_within_3_percent_of_autotune_on_this_device(cfg):
         if tuned != shipped:
             # alternate between the two tables so that clock and temperature drift hit both alike
             t = {"shipped": [], "tuned": []}
-            for _ in range(3):
+            for _ in range(5):
                 for s in slots:
                     ops.tune_set(a[0], a[2], -1, s)
                 t["shipped"].append(_median_ms(a, dO))
                 for s in slots:
                     ops.tune_set(a[0], a[2], tuned[s], s)
                 t["tuned"].append(_median_ms(a, dO))
-            print("shipped", shipped, t["shipped"], "tuned", tuned, t["tuned"], flush=True)
-            assert min(t["shipped"]) <= 1.03 * min(t["tuned"]), (shipped, tuned, t)
+            med = {k: statistics.median(v) for k, v in t.items()}
+            # spread of a table's repeats without its fastest and slowest one (a first run after a switch is often an outlier)
+            spread = max((sorted(v)[-2] - sorted(v)[1]) / statistics.median(v) for v in t.values())
+            print("shipped", shipped, t["shipped"], "tuned", tuned, t["tuned"], "spread of the repeats %.1f %%" % (100 * spread), flush=True)
+            if spread > 0.03:
+                pytest.skip("repeats of one table differ by %.1f %% on this device: a 3 %% comparison is not resolved" % (100 * spread))
+            assert med["shipped"] <= 1.03 * med["tuned"], (shipped, tuned, t)
     finally:
         for s in slots:
             ops.tune_set(a[0], a[2], -1, s)
+
+
+def test_every_pairing_of_the_chunked_operator_and_of_the_bias_meets_the_oracle_and_their_tuners_record_a_choice():
+    """Slots `chunked_pair` and `aff_pair`: one or two work items per workgroup (or by launch size) give the same results
+    to rounding; autotune_chunked / autotune_affinity time the ops and leave a valid choice in the table."""
+    from universal_attention_triton_amd.affinity import AffinityScores
+    b, h, r, L, d, c = 1, 3, 2, 640, 64, 128                      # 5 key groups, 5 query blocks: odd, so pairs are ragged
+    for dtype in (BF, torch.float32):
+        inp = orc.make_inputs(b, h, r, L, d, c, dtype=dtype, seed=77)
+        a = [inp[k].cuda() for k in NAMES]
+        n = L // c
+        g = torch.Generator().manual_seed(2)
+        g_out = torch.randn(b, h, r, L, d, n, generator=g).to(dtype)
+        g_denom = torch.randn(b, h, r, L, n, generator=g).to(dtype).float()
+        args32 = [inp[k].float() for k in NAMES]
+        out_ref, _ = orc.chunked_forward(*args32)
+        want = orc.chunked_backward(*args32, g_out.float(), g_denom)
+        assert ops.tune_variants(a[0], a[2], "chunked_pair") == 3
+        res = []
+        for v in range(3):
+            ops.tune_set(a[0], a[2], v, "chunked_pair")
+            try:
+                out, denom, st = ops.chunked_forward(*a, keep_state=True)
+                grads = ops.chunked_backward(*a, out, g_out.cuda(), g_denom.cuda(), state=st)
+                torch.cuda.synchronize()
+            finally:
+                ops.tune_set(a[0], a[2], -1, "chunked_pair")
+            assert rel_err(out, out_ref) <= TOL[dtype], (v, rel_err(out, out_ref))
+            for name, x, y in zip(NAMES, grads, want):
+                if name != "kc" or dtype == BF:                    # the float32 key gradient has its own bars in test_hip_backward
+                    assert rel_err(x.reshape(y.shape), y) <= TOL[dtype], (v, name, rel_err(x.reshape(y.shape), y))
+            res.append((out,) + tuple(grads))
+        for v in (1, 2):
+            for x, y in zip(res[v], res[0]):
+                assert torch.equal(x, y), v                        # same work items, same order of additions inside each
+        chosen = ops.autotune_chunked(*a, repeats=2)
+        assert chosen.keys() == {"chunked_pair"} and 0 <= chosen["chunked_pair"] < 3
+        assert ops.tune_get(a[0], a[2], "chunked_pair") == chosen["chunked_pair"]
+        ops.tune_set(a[0], a[2], -1, "chunked_pair")
+        # the stand-alone bias
+        k = inp["kc"].reshape(b, h, L, d).cuda()
+        src, dest = inp["static_src"].reshape(b, h, L).cuda(), inp["static_dest"].cuda()
+        daff = torch.randn(b, h, L, L, generator=g).to(dtype).cuda()
+        desc = ops._affinity_args(k, src, dest)[3]
+        import ctypes
+        from universal_attention_triton_amd import _lib
+        lib = _lib.load()
+        assert lib.ua_tune_variants(ctypes.byref(desc), _lib.UA_TUNE_AFF_PAIR) == 3
+        res = []
+        for v in range(3):
+            _lib.check(lib.ua_tune_set(ctypes.byref(desc), _lib.UA_TUNE_AFF_PAIR, v), "ua_tune_set")
+            try:
+                aff = ops.affinity_forward(k, src, dest)
+                res.append((aff,) + tuple(ops.affinity_backward(k, src, dest, daff)))
+                torch.cuda.synchronize()
+            finally:
+                lib.ua_tune_set(ctypes.byref(desc), _lib.UA_TUNE_AFF_PAIR, -1)
+        for v in (1, 2):
+            for x, y in zip(res[v], res[0]):
+                assert torch.equal(x, y), v
+        leaves = [t.detach().requires_grad_() for t in (k, src, dest)]
+        assert torch.equal(AffinityScores.apply(*leaves), res[0][0])          # checked against the oracle in test_hip_affinity
+        chosen = ops.autotune_affinity(k, src, dest, repeats=2)
+        assert 0 <= chosen["aff_pair"] < 3 and lib.ua_tune_get(ctypes.byref(desc), _lib.UA_TUNE_AFF_PAIR) == chosen["aff_pair"]
+        lib.ua_tune_set(ctypes.byref(desc), _lib.UA_TUNE_AFF_PAIR, -1)
+
+
+def test_first_call_autotune_is_opt_in_through_the_environment(monkeypatch):
+    """UA_AUTOTUNE=1: the fused operator tunes itself the first time it meets a table key, once; without the variable it
+    never does."""
+    from universal_attention_triton_amd.universal_attention import universal_attention
+    inp = orc.make_inputs(1, 2, 1, 384, 128, 128, dtype=BF, seed=5)
+    a = [inp[k].cuda() for k in NAMES]
+    slots = [s for s in ("carry", "fwd_tiles", "bwd_queries", "bwd_keys") if ops.tune_variants(a[0], a[2], s) > 1]
+    O_ref, _, _ = dense_reference(inp)
+    monkeypatch.delenv("UA_AUTOTUNE", raising=False)
+    ops._first_call_tuned.clear()
+    universal_attention(*a)
+    assert all(ops.tune_get(a[0], a[2], s) == -1 for s in slots) and not ops._first_call_tuned
+    monkeypatch.setenv("UA_AUTOTUNE", "1")
+    calls = []
+    real = ops.autotune
+    monkeypatch.setattr(ops, "autotune", lambda *x, **kw: (calls.append(1), real(*x, **kw))[1])
+    try:
+        leaves = [t.clone().requires_grad_() for t in a]
+        O = universal_attention(*leaves)
+        O2 = universal_attention(*leaves)                 # same key: no second tuning run
+        assert len(calls) == 1 and all(ops.tune_get(a[0], a[2], s) >= 0 for s in slots)
+        assert rel_err(O, O_ref) <= TOL[BF] and torch.equal(O, O2)
+        torch.autograd.grad(O, leaves, inp["dO"].cuda())
+    finally:
+        for s in slots:
+            ops.tune_set(a[0], a[2], -1, s)
+        ops._first_call_tuned.clear()

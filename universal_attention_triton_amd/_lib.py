@@ -13,7 +13,9 @@ LIB_PATH = os.path.join(HERE, "libua_hip.so")
 UA_F32, UA_BF16 = 0, 1
 UA_OP_FWD, UA_OP_BWD, UA_OP_FUSED_FWD, UA_OP_FUSED_BWD, UA_OP_BWD_SCRATCH, UA_OP_FUSED_BWD_SCRATCH = 0, 1, 2, 3, 4, 5
 UA_TUNE_FWD_RECOMPUTE, UA_TUNE_CARRY, UA_TUNE_FWD_TILES, UA_TUNE_BWD_PARTS, UA_TUNE_BWD_QUERIES, UA_TUNE_BWD_KEYS = 2, 16, 17, 18, 19, 20
-TUNE_SLOTS = {"fwd_recompute": 2, "carry": 16, "fwd_tiles": 17, "bwd_parts": 18, "bwd_queries": 19, "bwd_keys": 20}
+UA_TUNE_CHUNKED_PAIR, UA_TUNE_AFF_PAIR = 21, 22
+TUNE_SLOTS = {"fwd_recompute": 2, "carry": 16, "fwd_tiles": 17, "bwd_parts": 18, "bwd_queries": 19, "bwd_keys": 20,
+              "chunked_pair": 21, "aff_pair": 22}
 UA_FLAG_SKIP_MASKED = 1
 UA_FLAG_RECOMPUTE = 4
 UA_FLAG_PRUNE = 2

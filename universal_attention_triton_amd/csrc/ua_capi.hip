@@ -89,7 +89,7 @@ TuneKey tune_key(const ua_desc& d, int slot) {
 }
 bool known_slot(int slot) {
   return slot == UA_TUNE_FWD_RECOMPUTE || slot == UA_TUNE_CARRY || slot == UA_TUNE_FWD_TILES || slot == UA_TUNE_BWD_PARTS ||
-         slot == UA_TUNE_BWD_QUERIES || slot == UA_TUNE_BWD_KEYS;
+         slot == UA_TUNE_BWD_QUERIES || slot == UA_TUNE_BWD_KEYS || slot == UA_TUNE_CHUNKED_PAIR || slot == UA_TUNE_AFF_PAIR;
 }
 int n_divisors(int r) { int n = 0; for (int p = 1; p <= r; ++p) n += r % p == 0; return n; }
 int nth_divisor(int r, int i) { for (int p = 1; p <= r; ++p) if (r % p == 0 && i-- == 0) return p; return 1; }
@@ -103,6 +103,8 @@ int n_variants(const ua_desc& d, int slot) {
     case UA_TUNE_BWD_PARTS: return bf ? n_divisors(d.r) : 1;
     case UA_TUNE_BWD_QUERIES: return bf && d.d <= 128 ? 2 : 1;
     case UA_TUNE_BWD_KEYS: return bf && padded_dim(d.d) == 128 && d.r == 1 ? 2 : 1;
+    case UA_TUNE_CHUNKED_PAIR: return 3;     // by launch size / one / two work items per workgroup (ua::paired_items)
+    case UA_TUNE_AFF_PAIR: return 3;
   }
   return 1;
 }
@@ -432,6 +434,7 @@ int run_bwd_common(const ua_desc& d, const Layout& l, char* wf, char* wb, bool c
   a.split_r = (!chunked && d.r > 1) ? 1 : 0;
   a.key_parts = l.key_parts;
   a.keys_variant = l.tiles ? tuned_variant(d, UA_TUNE_BWD_KEYS) : 0;
+  a.pair = is_chunked ? tuned_variant(d, UA_TUNE_CHUNKED_PAIR) : 0;
   // bf16 tile exchange with one query group: the two kernels write the caller's gradients themselves.  The chunked
   // operator qualifies when the caller asserts that nothing flows to (query, later chunk) pairs, so that the query side is
   // known here to run from the tiles.
@@ -618,7 +621,8 @@ int ua_fwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
     UA_HIP(ua::launch_fwd_chunked2(d.dtype, l.D, wf + l.Qp, wf + l.Kp, wf + l.Vp, wf + l.VT, (const float*)(wf + l.lsrc),
                                    (const float*)(wf + l.ldest), (const float*)(wf + l.C), (const int*)(wf + l.reach),
                                    (const int*)(wf + l.minkey), out->ptr, denom, lse2, out->stride_z, out->stride_t,
-                                   out->stride_d, out->stride_i, d.r, d.L, l.Lp, d.d, d.chunk, l.nch, l.Zq, s));
+                                   out->stride_d, out->stride_i, d.r, d.L, l.Lp, d.d, d.chunk, l.nch, l.Zq, s,
+                                   tuned_variant(d, UA_TUNE_CHUNKED_PAIR)));
     return UA_OK;
   }
   if (int e = pack_inputs(d, l, true, kc, vc, xq, static_src, static_dest, wf, s)) return e;
@@ -660,7 +664,7 @@ int ua_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
         UA_HIP(ua::launch_fwd_chunked2(d.dtype, l.D, wf + l.Qp, wf + l.Kp, wf + l.Vp, wf + l.VT, (const float*)(wf + l.lsrc),
                                        (const float*)(wf + l.ldest), (const float*)(wf + l.C), (const int*)(wf + l.reach),
                                        (const int*)(wf + l.minkey), nullptr, nullptr, (float*)(wf + l.lse2), 0, 0, 0, 0, d.r, d.L, l.Lp,
-                                       d.d, d.chunk, l.nch, l.Zq, s));
+                                       d.d, d.chunk, l.nch, l.Zq, s, tuned_variant(d, UA_TUNE_CHUNKED_PAIR)));
     }
     bool in_place = false;
     {
@@ -814,7 +818,7 @@ int ua_affinity_fwd(const ua_desc* desc, const ua_rows* k, const void* src, cons
   if (int e = aff_prepare(desc, k, src, dest, ws, ws_bytes, false, l, s)) return e;
   char* w = (char*)ws;
   UA_HIP(ua::launch_aff_fwd(desc->dtype, l.D, w + l.Kp, (const float*)(w + l.lsrc), (const float*)(w + l.ldest), aff, desc->L, l.Lp,
-                            l.Z, s));
+                            l.Z, s, tuned_variant(*desc, UA_TUNE_AFF_PAIR)));
   return UA_OK;
 }
 
@@ -829,7 +833,7 @@ int ua_affinity_bwd(const ua_desc* desc, const ua_rows* k, const void* src, cons
   UA_HIP(ua::launch_aff_bwd(desc->dtype, l.D, w + l.Kp, w + l.KT, (const float*)(w + l.lsrc), (const float*)(w + l.ldest), daff,
                             (float*)(w + l.DL), (float*)(w + l.row), (float*)(w + l.colp), (float*)(w + l.gs_row),
                             (float*)(w + l.gs_col), src, dest, dk, dsrc, ddest, desc->L, l.Lp, desc->d, l.Z, s,
-                            l.tiles ? w + l.Wst : nullptr));
+                            l.tiles ? w + l.Wst : nullptr, tuned_variant(*desc, UA_TUNE_AFF_PAIR)));
   return UA_OK;
 }
 

@@ -23,17 +23,17 @@ UA_INST(64) UA_INST(128)
 // Launches of more workgroups than CUs give every workgroup two key groups of complementary length (the kernels see it
 // from the grid): equal workgroups, half as many workgroup changes.  Launches that fit the CUs at once keep one group
 // per workgroup.  (Measured on L = 4096 with 8 to 16 heads: several unequal workgroups per CU are the slowest form.)
-static int paired_groups(int n_kg, int Z) { return (long)n_kg * Z > device_cus() ? (n_kg + 1) / 2 : n_kg; }
+static int paired_groups(int n_kg, int Z, int pair) { return paired_items(n_kg, (long)n_kg * Z > device_cus(), pair); }
 
 template <class T, int D>
-static hipError_t aff_fwd_t(const void* Kp, const float* lsrc, const float* ldest, void* aff, int L, int Lp, int Z, hipStream_t s) {
+static hipError_t aff_fwd_t(const void* Kp, const float* lsrc, const float* ldest, void* aff, int L, int Lp, int Z, hipStream_t s, int pair) {
   const int vec = ((uintptr_t)aff % 16 == 0 && L % (16 / (int)sizeof(T)) == 0) ? 1 : 0;      // rows start 16-byte aligned
-  hipLaunchKernelGGL((k_aff_fwd<T, D>), dim3(paired_groups(Lp / 128, Z), Z), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, (T*)aff, L, Lp, vec);
+  hipLaunchKernelGGL((k_aff_fwd<T, D>), dim3(paired_groups(Lp / 128, Z, pair), Z), dim3(512), 0, s, (const T*)Kp, lsrc, ldest, (T*)aff, L, Lp, vec);
   return hipGetLastError();
 }
 hipError_t launch_aff_fwd(int dtype, int D, const void* Kp, const float* lsrc, const float* ldest, void* aff, int L, int Lp, int Z,
-                          hipStream_t s) {
-#define UA_ARGS Kp, lsrc, ldest, aff, L, Lp, Z, s
+                          hipStream_t s, int pair) {
+#define UA_ARGS Kp, lsrc, ldest, aff, L, Lp, Z, s, pair
   if (dtype == 1) return D == 64 ? aff_fwd_t<bf16, 64>(UA_ARGS) : aff_fwd_t<bf16, 128>(UA_ARGS);
   return D == 64 ? aff_fwd_t<float, 64>(UA_ARGS) : aff_fwd_t<float, 128>(UA_ARGS);
 #undef UA_ARGS
@@ -42,14 +42,14 @@ hipError_t launch_aff_fwd(int dtype, int D, const void* Kp, const float* lsrc, c
 template <class T, int D>
 static hipError_t aff_bwd_t(const void* Kp, const void* KT, const float* lsrc, const float* ldest, const void* daff, float* DL,
                             float* row, float* colp, float* gs_row, float* gs_col, const void* src, const void* dest, void* dk,
-                            void* dsrc, void* ddest, int L, int Lp, int d, int Z, hipStream_t s, void* Wst) {
+                            void* dsrc, void* ddest, int L, int Lp, int d, int Z, hipStream_t s, void* Wst, int pair) {
   hipError_t e;
   if constexpr (sizeof(T) == 2) {
     if (Wst) {      // rows of daff 16-byte aligned: the gradient W travels as bf16 tiles instead of the float L x L tensor
-      hipLaunchKernelGGL((k_aff_bwd_keys<T, D>), dim3(paired_groups(Lp / 128, Z), Z), dim3(512), 0, s, (const T*)Kp, (const T*)KT, lsrc, ldest,
+      hipLaunchKernelGGL((k_aff_bwd_keys<T, D>), dim3(paired_groups(Lp / 128, Z, pair), Z), dim3(512), 0, s, (const T*)Kp, (const T*)KT, lsrc, ldest,
                          (const T*)daff, (T*)Wst, row, gs_row, L, Lp);
       if ((e = hipGetLastError()) != hipSuccess) return e;
-      hipLaunchKernelGGL((k_aff_bwd_cols<T, D>), dim3(paired_groups(Lp / 128, Z), Z), dim3(512), 0, s, (const T*)KT, (const T*)Wst, colp, L, Lp);
+      hipLaunchKernelGGL((k_aff_bwd_cols<T, D>), dim3(paired_groups(Lp / 128, Z, pair), Z), dim3(512), 0, s, (const T*)KT, (const T*)Wst, colp, L, Lp);
       if ((e = hipGetLastError()) != hipSuccess) return e;
       hipLaunchKernelGGL((k_aff_finish<T>), dim3((L + 3) / 4, Z), dim3(256), 0, s, (const float*)row, (const float*)colp,
                          (const float*)gs_row, (const float*)nullptr, (const T*)src, (const T*)dest, (T*)dk, (T*)dsrc, (T*)ddest, L,
@@ -72,8 +72,8 @@ static hipError_t aff_bwd_t(const void* Kp, const void* KT, const float* lsrc, c
 }
 hipError_t launch_aff_bwd(int dtype, int D, const void* Kp, const void* KT, const float* lsrc, const float* ldest, const void* daff,
                           float* DL, float* row, float* colp, float* gs_row, float* gs_col, const void* src, const void* dest,
-                          void* dk, void* dsrc, void* ddest, int L, int Lp, int d, int Z, hipStream_t s, void* Wst) {
-#define UA_ARGS Kp, KT, lsrc, ldest, daff, DL, row, colp, gs_row, gs_col, src, dest, dk, dsrc, ddest, L, Lp, d, Z, s, Wst
+                          void* dk, void* dsrc, void* ddest, int L, int Lp, int d, int Z, hipStream_t s, void* Wst, int pair) {
+#define UA_ARGS Kp, KT, lsrc, ldest, daff, DL, row, colp, gs_row, gs_col, src, dest, dk, dsrc, ddest, L, Lp, d, Z, s, Wst, pair
   if (dtype == 1) return D == 64 ? aff_bwd_t<bf16, 64>(UA_ARGS) : aff_bwd_t<bf16, 128>(UA_ARGS);
   return D == 64 ? aff_bwd_t<float, 64>(UA_ARGS) : aff_bwd_t<float, 128>(UA_ARGS);
 #undef UA_ARGS

@@ -36,9 +36,9 @@ template __global__ void k_bwd_keys2<bf16, 128, 2, false, true, true>(BwdArgs<bf
 template __global__ void k_bwd_keys2<bf16, 128, 2, true, true, true>(BwdArgs<bf16>);
 
 template <class T, int D, int NST, bool MR, bool CH, bool TO>
-static hipError_t bwd2_mr(const BwdArgs<T>& a, int Lp, int Zk, hipStream_t s) {
+static hipError_t bwd2_mr(const BwdArgs<T>& a, int Lp, int Zk, hipStream_t s, int pair = 0) {
   // two key groups per workgroup once every CU gets at least two of the single ones
-    const int n_kg = Lp / 128, gx = (long)n_kg * Zk >= 2 * device_cus() ? (n_kg + 1) / 2 : n_kg;
+  const int n_kg = Lp / 128, gx = paired_items(n_kg, (long)n_kg * Zk >= 2 * device_cus(), pair);
   hipLaunchKernelGGL((k_bwd_keys2<T, D, NST, MR, CH, TO>), dim3(gx, Zk), dim3(512), 0, s, a);
   return hipGetLastError();
 }
@@ -53,9 +53,9 @@ static hipError_t bwd2_t(const BwdArgsV& v, int Zk, hipStream_t s) {
       return v.R / a.key_parts > 1 ? bwd2_mr<T, D, NST, true, false, true>(a, v.Lp, Zk * a.key_parts, s)
                                    : bwd2_mr<T, D, NST, false, false, true>(a, v.Lp, Zk * a.key_parts, s);
     if (v.dS_st)
-      return v.R > 1 ? bwd2_mr<T, D, NST, true, true, true>(a, v.Lp, Zk, s) : bwd2_mr<T, D, NST, false, true, true>(a, v.Lp, Zk, s);
+      return v.R > 1 ? bwd2_mr<T, D, NST, true, true, true>(a, v.Lp, Zk, s, v.pair) : bwd2_mr<T, D, NST, false, true, true>(a, v.Lp, Zk, s, v.pair);
   }
-  if (v.chunked) return v.R > 1 ? bwd2_mr<T, D, NST, true, true, false>(a, v.Lp, Zk, s) : bwd2_mr<T, D, NST, false, true, false>(a, v.Lp, Zk, s);
+  if (v.chunked) return v.R > 1 ? bwd2_mr<T, D, NST, true, true, false>(a, v.Lp, Zk, s, v.pair) : bwd2_mr<T, D, NST, false, true, false>(a, v.Lp, Zk, s, v.pair);
   return v.R > 1 ? bwd2_mr<T, D, NST, true, false, false>(a, v.Lp, Zk, s) : bwd2_mr<T, D, NST, false, false, false>(a, v.Lp, Zk, s);
 }
 template <class T, int D>

@@ -152,13 +152,13 @@ hipError_t launch_fwd_fused(int dtype, int D, int variant, const void* Qp, const
 template <class T, int D>
 static hipError_t chunked2_t(const void* Qp, const void* Kp, const void* Vp, const void* VT, const float* lsrc, const float* ldest,
                              const float* C, const int* reach, const int* minkey, void* out, void* denom, float* lse2, long o_sz,
-                             long o_st, long o_sd, long o_si, int R, int L, int Lp, int d, int c, int nch, int Zq, hipStream_t s) {
+                             long o_st, long o_sd, long o_si, int R, int L, int Lp, int d, int c, int nch, int Zq, hipStream_t s, int pair) {
   constexpr int NST = sizeof(T) == 2 ? 2 : 1, NW = 8;
   constexpr long VV = 16 / (long)sizeof(T);
   const int ovec = out && o_sd == 1 && d % VV == 0 && (uintptr_t)out % 16 == 0 && o_sz % VV == 0 && o_st % VV == 0 && o_si % VV == 0;
   ChunkOut<T> co{(T*)out, (T*)denom, o_sz, o_st, o_sd, o_si, c, nch, ovec};
   // two query blocks per workgroup once every CU gets at least four of the single ones
-  const int n_blk = (Lp / 16 + NW - 1) / NW, gx = (long)n_blk * Zq >= 4L * device_cus() ? (n_blk + 1) / 2 : n_blk;
+  const int n_blk = (Lp / 16 + NW - 1) / NW, gx = paired_items(n_blk, (long)n_blk * Zq >= 4L * device_cus(), pair);
   hipLaunchKernelGGL((k_fwd_fused2<T, D, NST, NW, true>), dim3(gx, Zq), dim3(64 * NW), 0, s, (const T*)Qp,
                      (const T*)Kp, (const T*)VT, lsrc, ldest, C, (T*)nullptr, (float*)nullptr, lse2, reach, minkey, R, L, Lp, d, co, (const _Float16*)nullptr);
   hipError_t e = hipGetLastError();
@@ -178,8 +178,8 @@ static hipError_t chunked2_t(const void* Qp, const void* Kp, const void* Vp, con
 hipError_t launch_fwd_chunked2(int dtype, int D, const void* Qp, const void* Kp, const void* Vp, const void* VT, const float* lsrc,
                                const float* ldest, const float* C, const int* reach, const int* minkey, void* out, void* denom,
                                float* lse2, long o_sz, long o_st, long o_sd, long o_si, int R, int L, int Lp, int d, int c, int nch,
-                               int Zq, hipStream_t s) {
-#define UA_ARGS Qp, Kp, Vp, VT, lsrc, ldest, C, reach, minkey, out, denom, lse2, o_sz, o_st, o_sd, o_si, R, L, Lp, d, c, nch, Zq, s
+                               int Zq, hipStream_t s, int pair) {
+#define UA_ARGS Qp, Kp, Vp, VT, lsrc, ldest, C, reach, minkey, out, denom, lse2, o_sz, o_st, o_sd, o_si, R, L, Lp, d, c, nch, Zq, s, pair
   if (dtype == 1) return D == 64 ? chunked2_t<bf16, 64>(UA_ARGS) : chunked2_t<bf16, 128>(UA_ARGS);
   return D == 64 ? chunked2_t<float, 64>(UA_ARGS) : chunked2_t<float, 128>(UA_ARGS);
 #undef UA_ARGS

@@ -20,6 +20,7 @@ struct BwdArgsV {
   const void *src_in, *dest_in;
   int dO_rows;
   int keys_variant;     // UA_TUNE_BWD_KEYS
+  int pair;             // UA_TUNE_CHUNKED_PAIR (chunked operator): see paired_items
 };
 
 // Every launcher returns hipGetLastError() after enqueuing.  dtype: 0 fp32, 1 bf16.  D in {64,128}.
@@ -44,7 +45,12 @@ hipError_t launch_fwd_chunked(int dtype, int D, const void* Qp, const void* Kp, 
 hipError_t launch_fwd_chunked2(int dtype, int D, const void* Qp, const void* Kp, const void* Vp, const void* VT, const float* lsrc,
                                const float* ldest, const float* C, const int* reach, const int* minkey, void* out, void* denom,
                                float* lse2, long o_sz, long o_st, long o_sd, long o_si, int R, int L, int Lp, int d, int c, int nch,
-                               int Zq, hipStream_t s);
+                               int Zq, hipStream_t s, int pair = 0);
+// Work items per workgroup of the kernels that can take two of complementary length (`pair` arguments, BwdArgsV::pair):
+// 0 = two once the launch is large enough (the launcher's own rule), 1 = one, 2 = two.
+inline int paired_items(int n_items, bool large_launch, int pair) {
+  return (pair == 2 || (pair != 1 && large_launch)) ? (n_items + 1) / 2 : n_items;
+}
 // cols != 0: the kernel also produces dQ / dkcol through atomics (chunked mode, row-major working tensors);
 // cols == 0: it records the suffix carries and launch_bwd_queries finishes the query side (tiled working tensors;
 // with a.chunked set: the chunked operator for a chunk that is a multiple of 64).
@@ -59,11 +65,11 @@ hipError_t launch_bwd_queries_from_tiles(int D, const BwdArgsV& a, void* dq, int
 
 // Stand-alone decay bias (affinity scores): aff [Z][L][L] in the dtype; working tensors tiled like the fused operator's.
 hipError_t launch_aff_fwd(int dtype, int D, const void* Kp, const float* lsrc, const float* ldest, void* aff, int L, int Lp, int Z,
-                          hipStream_t s);
+                          hipStream_t s, int pair = 0);
 // DL [Z][L][L] float scratch; row, colp [Z][Lp][D] and gs_row, gs_col [Z][Lp] float scratch; src, dest: the caller's gates.
 // Wst (bf16, L a multiple of 8, daff 16-byte aligned): [Z][tri_tiles(Lp/32)][1 KB] scratch that replaces DL and gs_col
 hipError_t launch_aff_bwd(int dtype, int D, const void* Kp, const void* KT, const float* lsrc, const float* ldest, const void* daff,
                           float* DL, float* row, float* colp, float* gs_row, float* gs_col, const void* src, const void* dest,
-                          void* dk, void* dsrc, void* ddest, int L, int Lp, int d, int Z, hipStream_t s, void* Wst = nullptr);
+                          void* dk, void* dsrc, void* ddest, int L, int Lp, int d, int Z, hipStream_t s, void* Wst = nullptr, int pair = 0);
 
 }  // namespace ua

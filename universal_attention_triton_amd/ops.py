@@ -391,6 +391,85 @@ def autotune(kc, vc, xq, static_src, static_dest, dO=None, backward=True):
     return out
 
 
+
+def _time_variants(desc, slot, run, repeats=5):
+    """Times run() under every variant of `slot` for desc (median of `repeats` after one warm-up each, hipEvents on the
+    current stream), records the fastest in the library's table and returns it."""
+    lib = _lib.load()
+    n = lib.ua_tune_variants(ctypes.byref(desc), slot)
+    best, best_ms = 0, None
+    for v in range(n):
+        _lib.check(lib.ua_tune_set(ctypes.byref(desc), slot, v), "ua_tune_set")
+        run()
+        ms = []
+        for _ in range(repeats):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            run()
+            e1.record()
+            e1.synchronize()
+            ms.append(e0.elapsed_time(e1))
+        med = sorted(ms)[len(ms) // 2]
+        if best_ms is None or med < best_ms:
+            best, best_ms = v, med
+    _lib.check(lib.ua_tune_set(ctypes.byref(desc), slot, best), "ua_tune_set")
+    from . import tune
+    name = next(k for k, s_ in _lib.TUNE_SLOTS.items() if s_ == slot)
+    tune.record(desc, name, best)
+    return best
+
+
+def autotune_chunked(kc, vc, xq, static_src, static_dest, repeats=5):
+    """Chunked operator with a chunk that is a multiple of 64: times its forward + backward under each variant of the
+    slot `chunked_pair` (work items per workgroup) on these inputs and records the fastest.  -> {"chunked_pair": variant}"""
+    if kc.shape[3] % 64:
+        return {}
+    kc_, _, xq_, _, _, gflag = _prep(kc, vc, xq, static_src, static_dest)
+    desc = _desc(kc_, xq_, False, gflag)
+    g = {}
+
+    def run():
+        out, denom, state = chunked_forward(kc, vc, xq, static_src, static_dest, keep_state=True)
+        if "out" not in g:
+            g["out"], g["denom"] = torch.ones_like(out), torch.zeros(denom.shape, dtype=torch.float32, device=denom.device)
+        chunked_backward(kc, vc, xq, static_src, static_dest, out, g["out"], g["denom"], state=state)
+
+    with torch.no_grad():
+        return {"chunked_pair": _time_variants(desc, _lib.UA_TUNE_CHUNKED_PAIR, run, repeats)}
+
+
+def autotune_affinity(k, src, dest, repeats=5):
+    """Stand-alone bias: times its forward + backward under each variant of the slot `aff_pair` and records the fastest."""
+    k_, src_, dest_, desc, _ = _affinity_args(k, src, dest)
+    daff = torch.ones(*k.shape[:3], k.shape[2], dtype=k.dtype, device=k.device)
+
+    def run():
+        affinity_forward(k, src, dest)
+        affinity_backward(k, src, dest, daff)
+
+    with torch.no_grad():
+        return {"aff_pair": _time_variants(desc, _lib.UA_TUNE_AFF_PAIR, run, repeats)}
+
+
+_first_call_tuned = set()
+
+
+def autotune_on_first_call(kc, vc, xq, static_src, static_dest):
+    """UA_AUTOTUNE=1 in the environment: the fused operator tunes itself the first time it meets a table key (dtype,
+    padded head dim, r, size buckets of L and b*h), as the reference's @triton.autotune does per key
+    (universal_attention_kernel_opt.py:24-44).  Synchronises the device, so not for code under graph capture."""
+    import os
+    if os.environ.get("UA_AUTOTUNE") != "1" or torch.cuda.is_current_stream_capturing():
+        return None
+    b, h, n, c, d = kc.shape
+    L = n * c
+    key = (xq.dtype, 64 if d <= 64 else (128 if d <= 128 else 256), xq.shape[2], max(0, (L - 1).bit_length() - 7), (b * h - 1).bit_length())
+    if key in _first_call_tuned:
+        return None
+    _first_call_tuned.add(key)
+    with torch.no_grad():
+        return autotune(*[t.detach() for t in (kc, vc, xq, static_src, static_dest)])
+
 def _with_parts(desc, variant, fn):
     lib = _lib.load()
     if variant < 0:

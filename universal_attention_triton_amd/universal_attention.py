@@ -90,6 +90,7 @@ def universal_attention(kc, vc, xq, static_src, static_dest, return_lse=False, p
     (Universal_Attention/universal_attention.py:27-31); the backward then rebuilds the state first.
     recompute=True (bf16) implies that and also keeps the backward's workspace at O(L*L/16) bytes per head by
     recomputing the score and decay gradients in every kernel instead of exchanging tiles (UA_FLAG_RECOMPUTE)."""
+    ops.autotune_on_first_call(kc, vc, xq, static_src, static_dest)          # only with UA_AUTOTUNE=1
     O, lse, _state = _FusedUniversalAttention.apply(kc, vc, xq, static_src, static_dest, prune, recompute, keep_state)
     return (O, lse) if return_lse else O
 
