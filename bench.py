@@ -341,6 +341,16 @@ def main():
                 "forward_state": ops.retained_bytes(*[x.detach() for x in leaves]),
                 "O_and_lse": leaves[2].numel() * leaves[2].element_size() + leaves[2].numel() // cfg["d"] * 4,
                 "note": "the backward's scratch is allocated inside backward; keep_state=False retains O and lse only"}
+            # the same step holding nothing between forward and backward (the backward rebuilds the state first)
+            n_lean = max(3, args.steps // 4)
+            for _ in range(2):
+                torch.autograd.grad(universal_attention(*leaves, keep_state=False), leaves, dO)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(n_lean):
+                torch.autograd.grad(universal_attention(*leaves, keep_state=False), leaves, dO)
+            torch.cuda.synchronize()
+            out["config"]["bytes_retained_fwd_to_bwd"]["keep_state_false_ms_per_step"] = round((time.perf_counter() - t0) * 1e3 / n_lean, 4)
     if not args.no_parity and args.api in ("fused", "chunked"):
         res = step()
         torch.cuda.synchronize()
