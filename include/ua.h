@@ -112,7 +112,8 @@ size_t ua_workspace_bytes(const ua_desc* desc, int op);
  * static_src, static_dest: contiguous [b,h,L].  denom: contiguous [b,h,r,L,n] in desc->dtype.
  * lse2_out: NULL, or [b*h*r][L/chunk][Lp] float (Lp = L rounded up to 128) that receives the per-chunk normalisers in
  * float32 (log2 units; `denom` in bf16 is too coarse for the backward): the one part of the forward state that is
- * expensive to rebuild, 1/(d+1) of the size of `out`.  Hand it to ua_bwd as lse2_in. */
+ * expensive to rebuild, 1/(d+1) of the size of `out`.  Hand it to ua_bwd as lse2_in.  The workspace holds a copy
+ * either way, so it is a complete fwd_state for ua_bwd with or without lse2_in. */
 int ua_fwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
            const void* static_dest, const ua_chunked* out, void* denom, float* lse2_out, void* ws, size_t ws_bytes,
            ua_stream_t stream);
@@ -146,7 +147,8 @@ int ua_fused_fwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, cons
  * the library's load until the process ends.  Problems whose ua_workspace_bytes(desc, UA_OP_FUSED_FWD) exceeds it are
  * refused with UA_EWORKSPACE.  Calls no hipMalloc / hipFree.  All calls on one GPU share the array: two calls that
  * overlap on one GPU (different streams or threads) race, and the forward state a later ua_fused_bwd could reuse is not
- * kept (call ua_fused_bwd with fwd_state = NULL). */
+ * kept (call ua_fused_bwd with fwd_state = NULL).  The first call on a device looks up the array's address and sets
+ * kernel attributes: make it outside any stream capture; every later call only enqueues kernels. */
 #define UA_NOALLOC_SCRATCH_BYTES (64u << 20)
 size_t ua_noalloc_scratch_bytes(void);
 int ua_fused_fwd_noalloc(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,

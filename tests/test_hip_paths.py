@@ -412,3 +412,38 @@ def test_launches_of_paired_work_items_with_an_odd_number_of_items(shape):
         assert rel_err(O[:, hh:hh + 1], O_ref) <= TOL[bf], hh
         assert float((lse[:, hh:hh + 1].cpu().double() - lse_ref).abs().max()) <= TOL[bf], hh
         _table("head %d of %s" % (hh, (shape,)), [x[:, hh:hh + 1] for x in grads], g_ref, TOL[bf])
+
+
+def test_workspace_of_a_forward_that_also_wrote_the_normalisers_out_is_a_complete_state():
+    """ua_fwd with lse2_out leaves a copy of the normalisers in the workspace, so that workspace alone (fwd_state
+    without lse2_in) gives ua_bwd everything: same gradients, bit for bit, as after a forward without lse2_out."""
+    import ctypes
+    from universal_attention_triton_amd import _lib, ops
+    b, h, r, L, d, c = 1, 2, 2, 384, 64, 128
+    n = L // c
+    dtype = torch.bfloat16
+    inp = orc.make_inputs(b, h, r, L, d, c, dtype=dtype, seed=91)
+    ins = [inp[k].cuda() for k in NAMES]
+    gen = torch.Generator().manual_seed(4)
+    g_out = torch.randn(b, h, r, L, d, n, generator=gen).to(dtype).cuda()
+    g_denom = torch.randn(b, h, r, L, n, generator=gen).to(dtype).float().cuda()
+    out_ref, denom_ref, state_ref = ops.chunked_forward(*ins, keep_state=True)
+    want = ops.chunked_backward(*ins, out_ref, g_out, g_denom, state=state_ref)
+    # the same forward through the C entry point with lse2_out, then the backward on its workspace
+    lib = _lib.load()
+    kc, vc, xq, src, dest, gflag = ops._prep(*ins)
+    desc = ops._desc(kc, xq, True, gflag)
+    ws = ops._workspace(desc, _lib.UA_OP_FWD, xq.device)
+    ws.fill_(0x7f)                                                   # nothing may be left to chance
+    out = torch.empty(b, h, r, n, L, d, dtype=dtype, device="cuda").permute(0, 1, 2, 4, 5, 3)
+    denom = torch.empty(b, h, r, L, n, dtype=dtype, device="cuda")
+    lse2 = torch.empty(b * h * r * n * (-(-L // 128) * 128), dtype=torch.float32, device="cuda")
+    _, oc = ops._chunked(out)
+    _lib.check(lib.ua_fwd(ctypes.byref(desc), ctypes.byref(ops._rows_k(kc)), ctypes.byref(ops._rows_k(vc)), ctypes.byref(ops._rows_q(xq)),
+                          src.data_ptr(), dest.data_ptr(), ctypes.byref(oc), denom.data_ptr(), lse2.data_ptr(), ws.data_ptr(),
+                          ws.numel(), ops._stream()), "ua_fwd")
+    assert torch.equal(out, out_ref) and torch.equal(denom, denom_ref)
+    got = ops.chunked_backward(*ins, out, g_out, g_denom, state=ws)
+    torch.cuda.synchronize()
+    for name, x, y in zip(NAMES, got, want):
+        assert torch.equal(x, y), (name, rel_err(x, y))

@@ -12,25 +12,58 @@ from universal_attention_triton_amd import _lib, ops
 pytestmark = pytest.mark.gpu
 
 
-def _run_both(b, h, r, L, d, dtype, seed):
+def _run_both(b, h, r, L, d, dtype, seed, warm=True):
     inp = orc.make_inputs(b, h, r, L, d, 64, dtype=dtype, seed=seed)
     kc, vc, xq, src, dest = [inp[k].cuda() for k in ("kc", "vc", "xq", "static_src", "static_dest")]
     O_ref, lse_ref, _ = ops.fused_forward(kc, vc, xq, src, dest)
     O = torch.full((b, h, r, L, d), float("nan"), dtype=dtype, device="cuda")
     lse = torch.full((b, h, r, L), float("nan"), dtype=torch.float32, device="cuda")
+    src3, dest3 = src.reshape(b, h, L), dest.reshape(b, h, L)
+    if warm:       # the first call on a device looks up the address of the built-in scratch and sets kernel attributes
+        ops.fused_forward_noalloc(kc, vc, xq, src3, dest3, O, lse)
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated()
-    ops.fused_forward_noalloc(kc, vc, xq, src.reshape(b, h, L), dest.reshape(b, h, L), O, lse)
+    free_before = torch.cuda.mem_get_info()[0]          # the driver's view: would also show a hipMalloc inside the library
+    ops.fused_forward_noalloc(kc, vc, xq, src3, dest3, O, lse)
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before
     assert torch.equal(O, O_ref) and torch.equal(lse, lse_ref)
-    return O
+    return kc, vc, xq, src3, dest3, O, lse, O_ref, lse_ref
 
 
 def test_noalloc_forward_equals_workspace_forward_twice_second_smaller():
     _run_both(1, 4, 2, 1024, 128, torch.bfloat16, 11)
     _run_both(1, 2, 1, 320, 64, torch.bfloat16, 12)       # smaller: the scratch still holds the first call's state
     _run_both(2, 2, 1, 192, 48, torch.float32, 13)
+
+
+def test_noalloc_forward_under_graph_capture_after_an_eager_first_call():
+    """The first call per device must happen outside a capture (it looks up the scratch's address); later calls only
+    enqueue kernels, so they can be captured: three replays on fresh inputs, each against the eager workspace forward."""
+    b, h, r, L, d = 1, 2, 2, 320, 64
+    kc, vc, xq, src3, dest3, O, lse, _, _ = _run_both(b, h, r, L, d, torch.bfloat16, 21)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        ops.fused_forward_noalloc(kc, vc, xq, src3, dest3, O, lse)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ops.fused_forward_noalloc(kc, vc, xq, src3, dest3, O, lse)
+    for seed in (22, 23, 24):
+        fresh = orc.make_inputs(b, h, r, L, d, 64, dtype=torch.bfloat16, seed=seed)
+        for t, k in ((kc, "kc"), (vc, "vc"), (xq, "xq")):
+            t.copy_(fresh[k])
+        src3.copy_(fresh["static_src"].reshape(b, h, L))
+        dest3.copy_(fresh["static_dest"].reshape(b, h, L))
+        O.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        O_ref, lse_ref, _ = ops.fused_forward(kc, vc, xq, src3.view(b, h, L // 64, 64), dest3)
+        torch.cuda.synchronize()
+        assert torch.equal(O, O_ref) and torch.equal(lse, lse_ref), seed
 
 
 def test_noalloc_forward_refuses_what_does_not_fit():

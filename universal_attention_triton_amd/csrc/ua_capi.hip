@@ -610,6 +610,11 @@ int ua_fwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
   hipStream_t s = (hipStream_t)stream;
   const ua_desc& d = *desc;
   float* lse2 = lse2_out ? lse2_out : (float*)(wf + l.lse2);     // the per-chunk normalisers, float32, log2 units
+  // the workspace stays a complete forward state for ua_bwd also when the normalisers went to the caller's buffer
+  auto mirror_lse2 = [&]() -> int {
+    if (lse2_out) UA_HIP(hipMemcpyAsync(wf + l.lse2, lse2_out, (size_t)l.Zq * l.nch * l.Lp * 4, hipMemcpyDeviceToDevice, s));
+    return UA_OK;
+  };
   if (fast_chunk(d)) {
     if (int e = pack_inputs(d, l, false, kc, vc, xq, static_src, static_dest, wf, s)) return e;
     {
@@ -623,14 +628,14 @@ int ua_fwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_r
                                    (const int*)(wf + l.minkey), out->ptr, denom, lse2, out->stride_z, out->stride_t,
                                    out->stride_d, out->stride_i, d.r, d.L, l.Lp, d.d, d.chunk, l.nch, l.Zq, s,
                                    tuned_variant(d, UA_TUNE_CHUNKED_PAIR)));
-    return UA_OK;
+    return mirror_lse2();
   }
   if (int e = pack_inputs(d, l, true, kc, vc, xq, static_src, static_dest, wf, s)) return e;
   UA_PROF("k_fwd_chunked", s);
   UA_HIP(ua::launch_fwd_chunked(d.dtype, l.D, wf + l.Qp, wf + l.Kp, wf + l.VT, (const float*)(wf + l.lsrc),
                                 (const float*)(wf + l.ldest), out->ptr, denom, lse2, out->stride_z, out->stride_t, out->stride_d, out->stride_i, d.r, d.L,
                                 l.Lp, d.d, d.chunk, l.nch, l.Zk, s));
-  return UA_OK;
+  return mirror_lse2();
 }
 
 int ua_bwd(const ua_desc* desc, const ua_rows* kc, const ua_rows* vc, const ua_rows* xq, const void* static_src,
