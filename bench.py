@@ -233,11 +233,13 @@ def main():
                     help="fused (default): universal_attention(); chunked: the reference's call sequence "
                          "UniversalAttention.apply + SMVecMatMul.apply, which materialises out[b,h,r,L,d,n]")
     ap.add_argument("--no-pruned", action="store_true",
-                    help="skip the extra timing of the optional pruned mode (keeps a profiler's per-kernel statistics "
-                         "to the launches `value` is made of)")
+                    help="skip the extra timings of the optional modes (pruned, recomputing, less state kept for the "
+                         "backward): keeps a profiler's per-kernel statistics to the launches `value` is made of")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device-to-device copy, the known-size kernel that HBM counters of a "
                          "profiler run are scaled against")
+    ap.add_argument("--tune", action="append", default=[], metavar="SLOT=VARIANT",
+                    help="run with this kernel variant instead of the table's choice (e.g. bwd_keys=1); never the default line")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (every (batch, kv head) is independent; nothing here uses a "
@@ -260,6 +262,11 @@ def main():
     names = ("kc", "vc", "xq", "static_src", "static_dest")
     leaves = [inp[k].cuda().requires_grad_() for k in names]
     dO = inp["dO"].cuda()
+    if args.tune:
+        from universal_attention_triton_amd import ops as _ops
+        for item in args.tune:
+            slot, variant = item.split("=")
+            _ops.tune_set(leaves[0].detach(), leaves[2].detach(), int(variant), slot)
 
     if args.api == "affinity":
         return bench_affinity(args, cfg, inp)
@@ -327,7 +334,7 @@ def main():
                                % (args.config, "fwd+bwd" if cfg["bwd"] else "fwd only", cfg["b"], cfg["h"], cfg["r"], cfg["L"], cfg["d"],
                                   ", upstream dO like the output" if cfg["bwd"] else ""),
                    "pct_of_mfma_peak": round(100 * (f_fwd + f_bwd) / (ms * 1e-3) / 1e12 / peak, 2),
-                   "kernel_ms": kern},
+                   "kernel_ms": kern, **({"tune_override": args.tune} if args.tune else {})},
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
                      "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get((args.config, dom))},
     }
@@ -341,16 +348,17 @@ def main():
                 "forward_state": ops.retained_bytes(*[x.detach() for x in leaves]),
                 "O_and_lse": leaves[2].numel() * leaves[2].element_size() + leaves[2].numel() // cfg["d"] * 4,
                 "note": "the backward's scratch is allocated inside backward; keep_state=False retains O and lse only"}
-            # the same step holding nothing between forward and backward (the backward rebuilds the state first)
-            n_lean = max(3, args.steps // 4)
-            for _ in range(2):
-                torch.autograd.grad(universal_attention(*leaves, keep_state=False), leaves, dO)
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            for _ in range(n_lean):
-                torch.autograd.grad(universal_attention(*leaves, keep_state=False), leaves, dO)
-            torch.cuda.synchronize()
-            out["config"]["bytes_retained_fwd_to_bwd"]["keep_state_false_ms_per_step"] = round((time.perf_counter() - t0) * 1e3 / n_lean, 4)
+            if not args.no_pruned:
+                # the same step holding nothing between forward and backward (the backward rebuilds the state first)
+                n_lean = max(3, args.steps // 4)
+                for _ in range(2):
+                    torch.autograd.grad(universal_attention(*leaves, keep_state=False), leaves, dO)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(n_lean):
+                    torch.autograd.grad(universal_attention(*leaves, keep_state=False), leaves, dO)
+                torch.cuda.synchronize()
+                out["config"]["bytes_retained_fwd_to_bwd"]["keep_state_false_ms_per_step"] = round((time.perf_counter() - t0) * 1e3 / n_lean, 4)
     if not args.no_parity and args.api in ("fused", "chunked"):
         res = step()
         torch.cuda.synchronize()
@@ -368,17 +376,18 @@ def main():
         # the same sequence with only the float32 normalisers kept for the backward instead of the whole forward state
         # (1/(d+1) of the size of `out`; the backward then repacks the inputs and repeats the decay pre-pass)
         from universal_attention_triton_amd import ops, universal_attention_autograd as own_api
-        with own_api.chunked_options(keep_state="normalisers"):
-            n_full = max(3, args.steps // 4)
-            for _ in range(2):
-                step()
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            for _ in range(n_full):
-                step()
-            torch.cuda.synchronize()
-            out["config"]["keep_state_normalisers"] = {"ms_per_step": round((time.perf_counter() - t0) * 1e3 / n_full, 4),
-                                                       "note": "optional: only the normalisers retained for the backward; not `value`"}
+        if not args.no_pruned:
+            with own_api.chunked_options(keep_state="normalisers"):
+                n_full = max(3, args.steps // 4)
+                for _ in range(2):
+                    step()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(n_full):
+                    step()
+                torch.cuda.synchronize()
+                out["config"]["keep_state_normalisers"] = {"ms_per_step": round((time.perf_counter() - t0) * 1e3 / n_full, 4),
+                                                           "note": "optional: only the normalisers retained for the backward; not `value`"}
         out["config"]["bytes_retained_fwd_to_bwd"] = {
             "forward_state": int(ops.retained_bytes(*[x.detach() for x in leaves], chunked=True)),
             "out_and_denom": int(cfg["b"] * cfg["h"] * cfg["r"] * cfg["L"] * (cfg["d"] + 1) * (cfg["L"] // cfg["c"])
