@@ -67,10 +67,14 @@ class _FusedUniversalAttention(Function):
         # the forward state travels as a third, non-differentiable output that universal_attention() drops
         ctx.save_for_backward(kc, vc, xq, static_src, static_dest, O, lse, state)
         ctx.mark_non_differentiable(lse, state)
+        # no zero "gradients" are to be made up for lse and the state (a fill of the state's size per backward otherwise)
+        ctx.set_materialize_grads(False)
 
     @staticmethod
     def backward(ctx, dO, _dlse, _dstate=None):
         kc, vc, xq, static_src, static_dest, O, lse, state = ctx.saved_tensors
+        if dO is None:
+            return (None,) * 8
         b, h, n, c, d = kc.shape
         r = xq.shape[2]
         dO = dO.reshape(b, h, r, n * c, d)

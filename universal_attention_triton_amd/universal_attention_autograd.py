@@ -99,11 +99,19 @@ class _ChunkedBase(Function):
         # `out` is the tensor the caller holds anyway (SMVecMatMul saves it too): saving it costs no memory
         ctx.save_for_backward(kc, vc, xq, static_src, static_dest, out, state)
         ctx.mark_non_differentiable(state)
+        # no zero "gradient" is to be made up for the state output (it would be a fill of the state's size per backward)
+        ctx.set_materialize_grads(False)
         ctx.opt = dict(_options.get())          # same call, same context as forward(): the values it used
 
     @staticmethod
     def backward(ctx, g_out, g_denom, _g_state=None):
         kc, vc, xq, static_src, static_dest, out, state = ctx.saved_tensors
+        if g_out is None and g_denom is None:
+            return None, None, None, None, None
+        if g_out is None:
+            g_out = torch.zeros_like(out)
+        if g_denom is None:
+            g_denom = torch.zeros(out.shape[:4] + out.shape[5:], dtype=out.dtype, device=out.device)
         dk, dv, dq, dsrc, ddest = _chunked_bwd.apply(kc, vc, xq, static_src, static_dest, out, g_out, g_denom, state,
                                                      ctx.opt["skip_masked"], ctx.opt["recompute"])
         return dk, dv, dq.view(xq.shape), dsrc.view(static_src.shape), ddest.view(static_dest.shape)
