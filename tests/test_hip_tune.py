@@ -212,3 +212,31 @@ def test_first_call_autotune_is_opt_in_through_the_environment(monkeypatch):
         for s in slots:
             ops.tune_set(a[0], a[2], -1, s)
         ops._first_call_tuned.clear()
+
+
+@pytest.mark.parametrize("prune", [False, True])
+@pytest.mark.parametrize("shape", [(1, 2, 1, 1024 + 96, 100), (2, 1, 1, 2048, 128), (1, 3, 1, 130, 72)])
+def test_key_side_variant_with_32_keys_per_wave_on_ragged_shapes_and_with_pruning(shape, prune):
+    """Slot `bwd_keys`, variant 1 (one wave per SIMD, 32x32 tiles) against variant 0 and the oracle: L no multiple of 128,
+    padded head dims, gates that make the decay fast (so that UA_FLAG_PRUNE shortens the sweeps of both variants)."""
+    b, h, r, L, d = shape
+    inp = orc.make_inputs(b, h, r, L, d, 2, dtype=BF, seed=17, gate_mean=2.0)
+    k = inp["kc"].float() + 2.0 * inp["kc"].float()[:, :, :1, :1, :]              # correlated keys: fast decay
+    inp["kc"] = (k / k.norm(dim=-1, keepdim=True)).to(BF)
+    a = [inp[k_].cuda() for k_ in NAMES]
+    dO = inp["dO"].cuda()
+    O_ref, _, g_ref = dense_reference(inp)
+    assert ops.tune_variants(a[0], a[2], "bwd_keys") == 2
+    res = []
+    for v in (0, 1):
+        ops.tune_set(a[0], a[2], v, "bwd_keys")
+        try:
+            O, lse, ws = ops.fused_forward(*a, keep_state=True, prune=prune)
+            res.append(ops.fused_backward(*a, O, lse, dO, state=ws, prune=prune))
+            torch.cuda.synchronize()
+        finally:
+            ops.tune_set(a[0], a[2], -1, "bwd_keys")
+    for name, x0, x1, ref in zip(NAMES, res[0], res[1], g_ref):
+        assert torch.isfinite(x1.float()).all(), name
+        assert rel_err(x1, x0) <= 6e-3, (name, rel_err(x1, x0))
+        assert rel_err(x1.reshape(ref.shape), ref) <= TOL[BF], (name, rel_err(x1.reshape(ref.shape), ref))

@@ -98,6 +98,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
   for (int i = 0; i < 8; ++i) top = max(top, reach_z[i]);
   top = min(top, nTr - 1);
   const int myreach = min(max(reach_z[2 * w], reach_z[2 * w + 1]), top);
+  // the wave sweeps as far as the farther-reaching of its two 16-key tiles; the pre-pass wrote no bias tiles for the other
+  // one beyond that tile's own reach, so this lane's weights are zero in the blocks after `lane_reach`
+  const int lane_reach = reach_z[2 * w + (col >> 4)];
   const int total = top + 1 - first;
   // this wave takes part in steps s_lo .. s_hi (query blocks top - s): from the last block it reaches to its own
   const int s_lo = top - myreach, s_hi = top - sb32;
@@ -322,7 +325,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
           if constexpr (ph == 1) {
             const float bias = (float)((j & 1) ? hb1[4 * (j >> 1) + m] : hb0[4 * (j >> 1) + m]);
             float p = __builtin_amdgcn_exp2f(__builtin_fmaf(S[v], kLog2e, bias));
-            if (GEN) p = (masked && (tl0 + 8 * j + m) < 0) ? 0.f : p;
+            if (GEN) p = ((masked && (tl0 + 8 * j + m) < 0) || tb > lane_reach) ? 0.f : p;
             S[v] = p;
             dP[v] *= p;
           }
@@ -408,11 +411,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0)
     pre_write(stage_at(0));
     if (total > 1) issue(1, 1);
-    // steps in which every wave is past its first and before its last: s_lo < s < s_hi for all four, i.e.
-    // (last wave to join) < s < total - 4
+    // steps in which every wave is past its first and before its last and every 16-key tile is within its reach:
+    // (last tile to join) < s < total - 4
     int s_join = 0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) s_join = max(s_join, top - min(max(reach_z[2 * i], reach_z[2 * i + 1]), top));
+    for (int i = 0; i < 8; ++i) s_join = max(s_join, top - min(reach_z[i], top));
     const int fast0 = s_join + 1, fast1 = total - 4;
     int s = 0;
     for (; s < total && s < fast0; ++s) gen_step(s);
