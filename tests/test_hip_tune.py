@@ -215,10 +215,12 @@ def test_first_call_autotune_is_opt_in_through_the_environment(monkeypatch):
 
 
 @pytest.mark.parametrize("prune", [False, True])
-@pytest.mark.parametrize("shape", [(1, 2, 1, 1024 + 96, 100), (2, 1, 1, 2048, 128), (1, 3, 1, 130, 72)])
+@pytest.mark.parametrize("shape", [(1, 2, 1, 1024 + 96, 100), (2, 1, 1, 2048, 128), (1, 3, 1, 130, 72), (1, 36, 1, 1920 - 40, 128)])
 def test_key_side_variant_with_32_keys_per_wave_on_ragged_shapes_and_with_pruning(shape, prune):
     """Slot `bwd_keys`, variant 1 (one wave per SIMD, 32x32 tiles) against variant 0 and the oracle: L no multiple of 128,
-    padded head dims, gates that make the decay fast (so that UA_FLAG_PRUNE shortens the sweeps of both variants)."""
+    padded head dims, gates that make the decay fast (so that UA_FLAG_PRUNE shortens the sweeps of both variants); the
+    last shape is a launch of at least two workgroups per CU, whose workgroups sweep two key groups each (15 groups: the
+    middle one alone)."""
     b, h, r, L, d = shape
     inp = orc.make_inputs(b, h, r, L, d, 2, dtype=BF, seed=17, gate_mean=2.0)
     k = inp["kc"].float() + 2.0 * inp["kc"].float()[:, :, :1, :1, :]              # correlated keys: fast decay

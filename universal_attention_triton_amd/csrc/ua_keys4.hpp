@@ -85,13 +85,22 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
   __shared__ __attribute__((aligned(1024))) char lds[4 * SB];
   const unsigned lds0 = (unsigned)(size_t)lds;
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, col = lane & 31, hi = lane >> 5;
-  int kg, zo;
-  xcd_map(kg, zo);
+  int kg0, zo;
+  xcd_map(kg0, zo);
   const int zk = zo;
   const int Lp = a.Lp, L = a.L, nT16 = Lp / 16;
+  // a grid of half as many workgroups as key groups: this one sweeps group kg0 and then group (last - kg0), which
+  // together are as long as every other pair (equal workgroups, half as many workgroup changes)
+  const int n_kg = Lp / 128, n_items = (int)gridDim.x < n_kg ? 2 : 1;
+  for (int item = 0; item < n_items; ++item) {
+  const int kg = item == 0 ? kg0 : n_kg - 1 - kg0;
+  if (item == 1) {
+    if (kg == kg0) break;                        // odd number of groups: the middle one has no partner
+    __syncthreads();                             // the stages of the first sweep are free
+  }
   const int sb32 = 4 * kg + w, spos = 32 * sb32 + col;
   const int nTr = (L + 31) / 32, first = 4 * kg;
-  if (first >= nTr) return;                      // every key of this workgroup is padding
+  if (first >= nTr) continue;                    // every key of this group is padding
   const int* reach_z = a.reach + zk * nT16 + 8 * kg;
   int top = 0;
 #pragma unroll
@@ -453,6 +462,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
       }
     }
   }
+  }  // item
 }
 
 #undef UA_PINV
