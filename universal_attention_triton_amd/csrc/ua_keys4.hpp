@@ -276,13 +276,6 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     __builtin_amdgcn_sched_barrier(0);
     static_for<0, 48>([&](auto ic) __attribute__((always_inline)) {
       constexpr int i = decltype(ic)::value;
-      // ---- matrix instruction of the slot, and the operand PF slots ahead
-      if constexpr (i == 0) mma_v0(G, ring[i % PF], kp[i]);
-      else if constexpr (i < 8) mma_v(G, ring[i % PF], kp[i]);
-      else if constexpr (i < 24) { if constexpr ((i - 8) & 1) mma_v(dP, ring[i % PF], vf[(i - 8) >> 1]); else mma_v(S, ring[i % PF], kp[(i - 8) >> 1]); }
-      else if constexpr (i < 40) { if constexpr (i & 1) mma(dKt[((i - 24) >> 1) & 3], ring[i % PF], bs[(i - 24) >> 3]); else mma(dVt[((i - 24) >> 1) & 3], ring[i % PF], bp[(i - 24) >> 3]); }
-      else mma(dKt[(i - 40) & 3], ring[i % PF], bg[(i - 40) >> 2]);
-      if constexpr (i + PF < 48) ring[i % PF] = load_opnd(i + PF);
       // ---- vector work of the slot
       // The vector work of a slot runs in three passes over its elements: tie the inputs to the slot, compute, tie the
       // results to the slot - so that the chains of the slot's elements can be interleaved with one another (a
@@ -291,7 +284,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
       //   slots 10-34: decay chain; element v has its affinity in slot 10 + v + v / 2 (two slots out of three) and its
       //                dG / dl factor together with the next element's affinity
       //   slots 34-47: softmax chain; two elements in each of the first two slots, then one per slot
-      static_for<0, 48>([&](auto pc) __attribute__((always_inline)) {
+      // (the vector work has to be spread over all 48 slots: with the chains packed two elements per slot into slots
+      // 10-33, fewer wait states but matrix instructions alone in the last 14 slots, the step is 2 % slower)
+      auto vec = [&](auto pc) __attribute__((always_inline)) {
         constexpr int ph = decltype(pc)::value / 16, v = decltype(pc)::value % 16;
         constexpr bool u_v2 = i < 10 && (v * 10) / 16 == i;
         // element v: affinity in slot 10 + v + v / 2 (two slots out of three), its factor together with the next
@@ -346,7 +341,18 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
             }
           }
         }
-      });
+      };
+      // the inputs are tied to the slot BEFORE its matrix instruction: an instruction that reads a value right behind the
+      // (empty) assembly statement that ties it costs a wait state
+      static_for<0, 16>(vec);
+      // ---- matrix instruction of the slot, and the operand PF slots ahead
+      if constexpr (i == 0) mma_v0(G, ring[i % PF], kp[i]);
+      else if constexpr (i < 8) mma_v(G, ring[i % PF], kp[i]);
+      else if constexpr (i < 24) { if constexpr ((i - 8) & 1) mma_v(dP, ring[i % PF], vf[(i - 8) >> 1]); else mma_v(S, ring[i % PF], kp[(i - 8) >> 1]); }
+      else if constexpr (i < 40) { if constexpr (i & 1) mma(dKt[((i - 24) >> 1) & 3], ring[i % PF], bs[(i - 24) >> 3]); else mma(dVt[((i - 24) >> 1) & 3], ring[i % PF], bp[(i - 24) >> 3]); }
+      else mma(dKt[(i - 40) & 3], ring[i % PF], bg[(i - 40) >> 2]);
+      if constexpr (i + PF < 48) ring[i % PF] = load_opnd(i + PF);
+      static_for<16, 48>(vec);
       if constexpr (i == 9) {
         char* p = dG_base + (((!GEN || !first) ? grp_tile(2 * (tb + 1), sb32) : grp_tiles(Lp >> 5) - 2) << 10);
 #pragma unroll
