@@ -132,10 +132,12 @@ def parity_one_head(cfg, inp, O, grads, head=(0, 0)):
 
 # HBM bytes per launch of the roofline kernel, from the TCC counters FETCH_SIZE and WRITE_SIZE of two `rocprofv3 --pmc`
 # runs of this script, each scaled by what the same counter reads for the plain 1 GiB copy of --calibrate-copy
-# (profiles/bench_cfg2_fused_fwd_bwd.md, taken 2026-11-25: 2.60 GB read + 4.52 GB written by k_bwd_keys2; the reads
-# are the fp16 bias tiles plus operand tiles, the writes the dS / dG tiles k_bwd_queries3 consumes).  The counters cannot
-# be collected by a plain run of this script, so the figure is a dated measurement; configurations without one report null.
-MEASURED_TRAFFIC = {(2, "k_bwd_keys"): 7.11e9}
+# (profiles/counters_cfg2_keys_variants_cfg4_chunked.md, taken 2026-11-25; key: config, api, roofline kernel group).
+# Config 2: 2.60 GB read (the fp16 bias tiles plus operand tiles) + 4.52 GB written (the dS / dG tiles k_bwd_queries3
+# consumes) by k_bwd_keys2; config 4: 9.76 + 17.51 GB by k_bwd_keys4; the chunked call sequence at the config 2 shape:
+# 2.88 + 4.89 GB by k_bwd_keys2.  The counters cannot be collected by a plain run of this script, so the figures are dated
+# measurements; configurations without one report null.
+MEASURED_TRAFFIC = {(2, "fused", "k_bwd_keys"): 7.11e9, (4, "fused", "k_bwd_keys"): 27.27e9, (2, "chunked", "k_bwd_keys"): 7.76e9}
 
 
 def bench_sdpa(args, cfg):
@@ -336,7 +338,7 @@ def main():
                    "pct_of_mfma_peak": round(100 * (f_fwd + f_bwd) / (ms * 1e-3) / 1e12 / peak, 2),
                    "kernel_ms": kern, **({"tune_override": args.tune} if args.tune else {})},
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
-                     "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get((args.config, dom))},
+                     "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get((args.config, args.api, dom)) if not args.tune and not args.chunk else None},
     }
     if args.api == "fused":
         hk = hbm_kernels(cfg, kern)
