@@ -347,11 +347,16 @@ def merge_backward(mat, vec, g):
     dc = UaChunked(d4.data_ptr(), d4.stride(0), d4.stride(1), d4.stride(2), d4.stride(3))
     d_vec = torch.empty(*vec.shape, dtype=mat.dtype, device=mat.device)
     Lp = -(-L // 128) * 128
-    delta = torch.zeros(m4.shape[0], n, Lp, dtype=torch.float32, device=mat.device)
+    # the per-(row, chunk) term is only worth keeping where a chunked backward can take it: chunks that are a multiple of 64
+    delta = None
+    if L % n == 0 and (L // n) % 64 == 0:
+        delta = torch.zeros(m4.shape[0], n, Lp, dtype=torch.float32, device=mat.device)
     _lib.check(lib.ua_merge_bwd(_dtype_code(mat), rows, L, d, n, ctypes.byref(mc), vec_c.data_ptr(), g_c.data_ptr(), ctypes.byref(dc),
-                                d_vec.data_ptr(), delta.data_ptr(), _stream()), "ua_merge_bwd")
+                                d_vec.data_ptr(), delta.data_ptr() if delta is not None else None, _stream()), "ua_merge_bwd")
     d_mat = d4.unflatten(0, tuple(mat.shape[:-3])) if mat.dim() != 4 else d4
     d_vec = d_vec.to(vec.dtype)
+    if delta is None:
+        return d_mat, d_vec
     try:
         setattr(d_mat, _NOTE, (weakref.ref(d_vec), (mat.data_ptr(), tuple(mat.shape), tuple(mat.stride()), mat._version),
                                d_mat._version, d_vec._version, delta))
