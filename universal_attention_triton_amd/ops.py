@@ -125,7 +125,9 @@ def _split_over_heads(n_tensors, chunked):
             for b0 in range(0, b, step_b):
                 row = []
                 for h0 in range(0, h, step_h):
-                    piece = [a[b0:b0 + step_b, h0:h0 + step_h] if i < n_tensors else a for i, a in enumerate(args)]
+                    # tensors beyond the per-head ones (a forward state passed by position) belong to the whole call: dropped
+                    piece = [a[b0:b0 + step_b, h0:h0 + step_h] if i < n_tensors else (None if torch.is_tensor(a) else a)
+                             for i, a in enumerate(args)]
                     row.append(fn(*piece, **kw))
                 rows.append([None if row[0][i] is None else (row[0][i] if len(row) == 1 else torch.cat([p[i] for p in row], 1))
                              for i in range(len(row[0]))])
