@@ -154,6 +154,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
   // this lane's 16 bytes of the wave's two bias tiles (16 keys each) of query block 0
   const char* bt_src = reinterpret_cast<const char*>(a.Bt) + (((long)zk * tri_tiles(Lp >> 5) + 2 * sb32) << 10) + 16 * lane;
   const long st_head = grp_tiles(Lp >> 5) << 10;                   // bytes of gradient tiles per head
+  // tile indices inside a head in 32 bits (the scalar unit multiplies 64-bit values in several instructions, and a lone
+  // wave pays for every one of them); widened once for the byte offset
+  auto grp32 = [] __device__ (int tq, int h) __attribute__((always_inline)) -> long {
+    return (long)(unsigned)(16 * (tq >> 3) * ((tq >> 3) + 1) + 8 * h + (tq & 7)) << 10;
+  };
   // a lane's 8-byte pieces inside a (32 keys, 16 queries) gradient tile: queries 8 (j & 1) + 4 hi .. + 3 of the tile
   const int st_lane0 = StageT<bf16>::addr(perm32(col), 8 * hi), st_lane1 = StageT<bf16>::addr(perm32(col), 8 * (2 + hi));
   char* dS_base = reinterpret_cast<char*>(a.dS_st) + (long)zk * st_head;
@@ -198,7 +203,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
       dma16(ldz + 32 * tb + 4 * (lane & 7), base + TILES);      // every 128-byte piece of the row: ldest of the block
       st_pre = st_src[32 * tb];
     }
-    const char* bsrc = bt_src + (tri_bias_row(tb) << 10);
+    const char* bsrc = bt_src + ((long)(unsigned)(tb * (tb + 1)) << 10);
     dma16_nt(bsrc, base + TILES + 1024 + w * 2048);
     dma16_nt(bsrc + 1024, base + TILES + 1024 + w * 2048 + 1024);
   };
@@ -346,6 +351,14 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
       // (empty) assembly statement that ties it costs a wait state
       static_for<0, 16>(vec);
       // ---- matrix instruction of the slot, and the operand PF slots ahead
+      // one wait for the operands of two slots (every wait is an instruction the lone wave has to issue): behind the
+      // operands of slots i and i + 1 only those of slots i + 2 and i + 3 are in flight, one LDS read each for the input
+      // products and two for the transposed operands of the output products
+      if constexpr ((i & 1) == 0 && PF == 4) {
+        constexpr int behind = (i + 2 < 24 ? 1 : (i + 2 < 48 ? 2 : 0)) + (i + 3 < 24 ? 1 : (i + 3 < 48 ? 2 : 0));
+        __builtin_amdgcn_s_waitcnt(0xC07F | (behind << 8));          // lgkmcnt(behind), the other counters unconstrained
+        if constexpr (i >= 24) __builtin_amdgcn_sched_barrier(0);     // or the matrix builtin is moved in front of the wait
+      }
       if constexpr (i == 0) mma_v0(G, ring[i % PF], kp[i]);
       else if constexpr (i < 8) mma_v(G, ring[i % PF], kp[i]);
       else if constexpr (i < 24) { if constexpr ((i - 8) & 1) mma_v(dP, ring[i % PF], vf[(i - 8) >> 1]); else mma_v(S, ring[i % PF], kp[(i - 8) >> 1]); }
@@ -354,7 +367,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
       if constexpr (i + PF < 48) ring[i % PF] = load_opnd(i + PF);
       static_for<16, 48>(vec);
       if constexpr (i == 9) {
-        char* p = dG_base + (((!GEN || !first) ? grp_tile(2 * (tb + 1), sb32) : grp_tiles(Lp >> 5) - 2) << 10);
+        char* p = dG_base + ((!GEN || !first) ? grp32(2 * (tb + 1), sb32) : st_head - 2048);
 #pragma unroll
         for (int q = 0; q < 2; ++q) {
           __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&bg[q])[0], reinterpret_cast<u32x2*>(p + 1024 * q + st_lane0));
@@ -366,7 +379,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
     for (int q = 0; q < 2; ++q) { bp[q] = nbp[q]; bs[q] = nbs[q]; }
     {
-      char* p = dS_base + (grp_tile(2 * tb, sb32) << 10);
+      char* p = dS_base + grp32(2 * tb, sb32);
 #pragma unroll
       for (int q = 0; q < 2; ++q) {
         __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&bs[q])[0], reinterpret_cast<u32x2*>(p + 1024 * q + st_lane0));
@@ -397,7 +410,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     }
 #pragma unroll
     for (int q = 0; q < 2; ++q) bg[q] = as_operand<T>(dG, q);
-    char* p = dG_base + (grp_tile(2 * (top - s), sb32) << 10);
+    char* p = dG_base + grp32(2 * (top - s), sb32);
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
       __builtin_nontemporal_store(reinterpret_cast<const u32x2*>(&bg[q])[0], reinterpret_cast<u32x2*>(p + 1024 * q + st_lane0));
